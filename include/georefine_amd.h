@@ -1,0 +1,160 @@
+/*
+ * georefine_amd -- C ABI of the MI355X (gfx950) decode path for GeoRefine's
+ * lossless BF16 context codec.
+ *
+ * Two shared libraries implement this header:
+ *
+ *   libgeorefine_codec.so   host C++ (no GPU needed): the functions the reference
+ *                           binds with ctypes, same names and argument meaning.
+ *   libgeorefine_hip.so     device entry points.  The reference launches Triton
+ *                           kernels from Python for these steps, so each entry
+ *                           point cites the Python/Triton interface it replaces.
+ *
+ * Conventions: every function returns 0 on success and a small positive
+ * category code otherwise; nothing throws across the boundary.  Host functions
+ * own nothing but the encoder outputs, which are released with bcx_free /
+ * p_free.  Device functions take raw device pointers and a hipStream_t passed
+ * as void*, allocate nothing, never synchronise, and report data errors by
+ * OR-ing bits into a caller-provided device int32 (GRF_ERR_*), never by
+ * trapping.  All paths below are relative to the reference tree,
+ * GCR = context-runtime/georefine_context_runtime.
+ */
+#ifndef GEOREFINE_AMD_H
+#define GEOREFINE_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------ host codec */
+
+/* GCR/bitexact_context_ans.cpp:235  count, normalise and rANS-encode one symbol stream.
+ * kind 0: 10-bit main symbols, context (row class, column class); kind 1: 6-bit
+ * residuals, context = main symbol.  freq: caller buffer [nctx*vocab]. */
+int bcx_encode(const uint16_t *w, uint64_t n, uint32_t rows, uint32_t cols, const uint8_t *rc,
+               const uint8_t *cc, uint32_t nr, uint32_t nc, uint32_t kind, uint32_t *freq, uint8_t **stream,
+               size_t *stream_n);
+/* GCR/bitexact_context_ans.cpp:267  tables only */
+int bcx_frequencies(const uint16_t *w, uint64_t n, uint32_t rows, uint32_t cols, const uint8_t *rc,
+                    const uint8_t *cc, uint32_t nr, uint32_t nc, uint32_t kind, uint32_t *freq);
+/* GCR/bitexact_context_ans.cpp:291 and :309  (1 bad arguments, 2 invalid stream/tables, 3 internal) */
+int bcx_decode(const uint8_t *stream, size_t stream_n, uint64_t n, uint32_t rows, uint32_t cols,
+               const uint8_t *rc, const uint8_t *cc, uint32_t nr, uint32_t nc, uint32_t kind,
+               const uint16_t *resctx, const uint32_t *freq, uint16_t *out);
+int bcx_decode_compact(const uint8_t *stream, size_t stream_n, uint64_t n, uint32_t rows, uint32_t cols,
+                       const uint8_t *rc, const uint8_t *cc, uint32_t nr, uint32_t nc, uint32_t kind,
+                       const uint16_t *resctx, const uint32_t *freq, uint16_t *out);
+/* GCR/bitexact_context_ans.cpp:327 */
+void bcx_free(void *p);
+/* GCR/bitexact_context_ans.cpp:328 and :346  6-bit residuals, MSB first, zero padding */
+int bcx_pack6(const uint16_t *w, uint64_t n, uint8_t **out, size_t *bytes);
+int bcx_unpack6(const uint8_t *in, size_t bytes, uint64_t n, uint16_t *out);
+/* GCR/bitexact_context_gpu_index.cpp:21  frame-index builder: (state, byte offset) before
+ * every stride-th symbol; outputs written only on success; codes 1..6 */
+int bcx_checkpoint(const uint8_t *stream, size_t stream_bytes, uint64_t n, uint32_t rows, uint32_t cols,
+                   const uint8_t *rc, const uint8_t *cc, uint32_t nr, uint32_t nc, uint32_t kind,
+                   const uint16_t *resctx, const uint32_t *freq, uint32_t stride, uint32_t *states,
+                   uint32_t *offsets, uint16_t *out);
+/* GCR/bitexact_predictive_ans.cpp:10-12  generic context coder of the predictive frames */
+int p_encode(const uint16_t *v, const uint16_t *cx, uint64_t n, uint32_t nc, uint32_t vocab, uint32_t **freq,
+             uint8_t **stream, size_t *stream_n);
+int p_decode(const uint8_t *st, size_t bytes, uint64_t n, const uint16_t *cx, uint32_t nc, uint32_t vocab,
+             const uint32_t *freq, uint16_t *out);
+void p_free(void *p);
+/* GCR/bitexact_predictive_gpu_index.cpp:9 and :38 */
+int ppcx_checkpoint(const uint8_t *stream, size_t bytes, uint64_t n, const uint16_t *ctx, uint32_t nctx,
+                    uint32_t vocab, const uint32_t *freq, uint32_t stride, uint32_t *states, uint32_t *offsets,
+                    uint16_t *symbols);
+int ppcx_checkpoint_binary(const uint8_t *stream, size_t bytes, uint64_t n, const uint16_t *ctx, uint32_t nctx,
+                           uint32_t vocab, const uint32_t *freq, uint32_t stride, uint32_t *states,
+                           uint32_t *offsets, uint16_t *symbols);
+
+/* ------------------------------------------------------------------ device side */
+
+/* bits OR-ed into the caller's device error word */
+#define GRF_ERR_SYMBOL 1      /* slot maps to no symbol / zero frequency / dead context */
+#define GRF_ERR_OVERRUN 2     /* decoder wanted bytes past the end of a stream */
+#define GRF_ERR_UNDERFLOW 4   /* state still below 2^23 after two refill bytes */
+#define GRF_ERR_CHECKPOINT 8  /* segment did not end on the next checkpoint */
+
+/* return codes of the launch functions */
+#define GRF_OK 0
+#define GRF_BAD_ARGUMENT 1
+#define GRF_UNSUPPORTED 2
+#define GRF_LAUNCH_FAILED 3
+
+/* One entropy-coded symbol stream resident in device memory, with its
+ * checkpoint index and the lookup tables derived from its frequency rows.
+ *   cum     u32 [nctx][vocab+1]  inclusive prefix sums (cum[c][0] = 0)
+ *   bucket  u32 [nctx][256]      lo | hi<<16: first and last symbol whose slot
+ *                                range meets slots [b<<8, (b<<8)+255]
+ *   states / offsets  u32 [ceil(n/stride)]  decoder state and byte position
+ *                                before symbol k*stride */
+typedef struct grf_stream {
+  const uint8_t *bytes;
+  uint32_t n_bytes;
+  uint32_t vocab;
+  uint32_t nctx;
+  const uint32_t *cum;
+  const uint32_t *bucket;
+  const uint32_t *states;
+  const uint32_t *offsets;
+} grf_stream;
+
+/* A BCTX frame as the decode kernels see it (the buffers CudaContextTensor keeps,
+ * GCR/bitexact_context_gpu.py:96-125). mode 0: residual.bytes is the packed 6-bit
+ * stream and the other residual fields are unused; mode 128: residual is a full stream. */
+typedef struct grf_bctx_frame {
+  grf_stream main;
+  grf_stream residual;
+  const uint8_t *row_class;
+  const uint8_t *col_class;
+  uint32_t rows, cols;
+  uint32_t nc;
+  uint32_t mode;
+  uint32_t stride;
+} grf_bctx_frame;
+
+/* Replaces the Triton launch of decode_words (GCR/bitexact_context_gpu.py:149-150,
+ * kernel GCR/bitexact_context_gpu_kernels.py:114-169).  Decodes `count` checkpointed
+ * segments; segment j of the launch is block_ids[j] (device int64) or j itself when
+ * block_ids is NULL.  out holds count*stride words: out[j*stride + t]. */
+int grf_bctx_decode(const grf_bctx_frame *frame, const int64_t *block_ids, uint32_t count, uint16_t *out,
+                    int32_t *error, void *hip_stream);
+
+/* A PPCX frame (the buffers CudaPredictiveTensor keeps, GCR/bitexact_predictive_gpu.py:116-132).
+ * mode 0: residual.bytes is the packed 5-bit stream; mode 1: residual is a full stream. */
+typedef struct grf_ppcx_frame {
+  grf_stream main;
+  grf_stream residual;
+  const uint8_t *labels;
+  const uint8_t *flips;
+  const uint16_t *thresholds; /* 15 monotone ordinal keys */
+  uint32_t rows, cols;
+  uint32_t mode;
+  uint32_t stride;
+} grf_ppcx_frame;
+
+/* Replaces the Triton launch of the predictive decode_words
+ * (GCR/bitexact_predictive_gpu.py:172, kernel GCR/bitexact_predictive_gpu_kernels.py:24-58).
+ * reference: device BF16 words [rows*cols]; out: ceil(n/stride)*stride words. */
+int grf_ppcx_decode(const grf_ppcx_frame *frame, const uint16_t *reference, uint16_t *out, int32_t *error,
+                    void *hip_stream);
+
+/* Replaces the CUDA branch of predict() (GCR/bitexact_predictive_mix.py:91-102):
+ * out = high16( fl32(fl32(up*c0) + fl32(gate*c1)) + c2 ) with separate IEEE operations.
+ * coeff: BF16 [rows][3].  Sets GRF_ERR_SYMBOL in *error when any input, coefficient or
+ * result is not finite. */
+int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *coeff, uint16_t *out,
+                    uint32_t rows, uint32_t cols, int32_t *error, void *hip_stream);
+
+const char *grf_last_error(void);
+int grf_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
