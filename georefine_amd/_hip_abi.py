@@ -24,7 +24,17 @@ class GrfPpcxFrame(ctypes.Structure):
                 ("cols", ctypes.c_uint32), ("mode", ctypes.c_uint32), ("stride", ctypes.c_uint32)]
 
 
-DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_last_error", "grf_abi_version")
+class GrfBctxFused(ctypes.Structure):
+    _fields_ = [("main_bytes", ctypes.c_void_p), ("raw6", ctypes.c_void_p), ("seg_state", ctypes.c_void_p),
+                ("seg_offset", ctypes.c_void_p), ("tile_rows", ctypes.c_void_p), ("tile_class", ctypes.c_void_p),
+                ("lut", ctypes.c_void_p), ("tab", ctypes.c_void_p), ("col_class", ctypes.c_void_p)] + [
+        (name, ctypes.c_uint32) for name in (
+            "main_n_bytes", "rows", "cols", "nr", "nc", "lognc", "seg_len", "segs_per_row", "lanes_per_row",
+            "rows_per_tile", "n_slabs", "n_tiles", "shift", "lognb", "tabn", "piece_cap")]
+
+
+DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
+                  "grf_bctx_fused_decode", "grf_bctx_fused_lds_bytes", "grf_last_error", "grf_abi_version")
 
 
 def declare(L):
@@ -35,5 +45,11 @@ def declare(L):
     L.grf_ppcx_decode.restype = i
     L.grf_mix_predict.argtypes = [vp, vp, vp, vp, u32, u32, vp, vp]
     L.grf_mix_predict.restype = i
+    L.grf_bctx_gemv.argtypes = [ctypes.POINTER(GrfBctxFused), vp, u32, u32, vp, u32, vp, vp, vp]
+    L.grf_bctx_gemv.restype = i
+    L.grf_bctx_fused_decode.argtypes = [ctypes.POINTER(GrfBctxFused), vp, vp, vp]
+    L.grf_bctx_fused_decode.restype = i
+    L.grf_bctx_fused_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), u32]
+    L.grf_bctx_fused_lds_bytes.restype = u32
     L.grf_last_error.restype = ctypes.c_char_p
     L.grf_abi_version.restype = i

@@ -16,7 +16,7 @@ import math
 
 import numpy as np
 
-from . import _hip_abi, _native, _tables
+from . import _fused, _hip_abi, _native, _tables
 from . import bitexact_context_codec as base
 
 
@@ -44,8 +44,12 @@ def checkpoints(stream, freq, rows, columns, shape, nr, nc, stride, main=None):
     return states, offsets, out
 
 
-def index_frame(frame: bytes, stride: int = 1024):
-    """Parse, validate and index a frame; the decoded words must hash to the header digest."""
+def index_frame(frame: bytes, stride: int = 1024, *, fused_segment=None):
+    """Parse, validate and index a frame; the decoded words must hash to the header digest.
+
+    With ``fused_segment`` (a segment length dividing the row length) the result also
+    carries ``fused_states`` / ``fused_offsets``, the main-stream index at that length.
+    One validated walk serves both indexes when the lengths are multiples of each other."""
     if not isinstance(stride, int) or not 1 <= stride <= 65536:
         raise base.CodecError("invalid checkpoint stride")
     if len(frame) < base.HEADER.size + 32:
@@ -60,7 +64,16 @@ def index_frame(frame: bytes, stride: int = 1024):
         return out
     rows, columns, sf = info["rows"], info["columns"], info["main_freq"]
     sy, rs = info["main_stream"], info["residual_stream"]
-    states, offsets, main = checkpoints(sy, sf, rows, columns, (r, c), info["nr"], info["nc"], stride)
+    fine = fused_segment if (fused_segment and info["mode"] == 0) else None
+    if fine and stride % fine == 0:
+        fs, fo, main = checkpoints(sy, sf, rows, columns, (r, c), info["nr"], info["nc"], fine)
+        states, offsets = fs[::stride // fine].copy(), fo[::stride // fine].copy()
+    else:
+        states, offsets, main = checkpoints(sy, sf, rows, columns, (r, c), info["nr"], info["nc"], stride)
+        if fine:
+            fs, fo, _ = checkpoints(sy, sf, rows, columns, (r, c), info["nr"], info["nc"], fine)
+    if fine:
+        out.update(fused_states=fs, fused_offsets=fo, fused_segment=fine)
     out.update(rows=rows, columns=columns, main_freq=sf, main_stream=np.frombuffer(sy, dtype=np.uint8).copy(),
                main_states=states, main_offsets=offsets, residual_stream=np.frombuffer(rs, dtype=np.uint8).copy())
     if info["mode"] == 128:
@@ -90,12 +103,18 @@ def _device_stream(buffers, name, vocab, nctx):
 class HipContextTensor:
     """A BCTX-coded BF16 matrix resident on one MI355X."""
 
-    def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0"):
+    def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None):
         import torch
         if not torch.cuda.is_available():
             raise RuntimeError("a ROCm GPU is required")
         self._lib = _native.hip()  # fails loudly when the device library is absent
-        indexed = index_frame(frame, stride)
+        segment = None
+        if fused:
+            try:
+                segment = _fused.choose_segment(base.HEADER.unpack_from(frame)[6], fused_segment)
+            except (_fused.FusedUnsupported, Exception):
+                segment = None
+        indexed = index_frame(frame, stride, fused_segment=segment)
         self.shape = indexed["shape"]
         self.n = math.prod(self.shape)
         self.stride = stride
@@ -105,9 +124,26 @@ class HipContextTensor:
         self.frame_bytes = indexed["frame_bytes"]
         self.device = torch.device(device)
         self.buffers = {}
+        self.fused = None
+        self.fused_reason = "disabled" if not fused else "frame mode or geometry"
+        plan = None
+        if "fused_states" in indexed:
+            try:
+                plan = _fused.plan(self.shape, self.nr, self.nc, indexed["rows"], indexed["main_freq"],
+                                   indexed.pop("fused_states"), indexed.pop("fused_offsets"),
+                                   len(indexed["main_stream"]), indexed["fused_segment"])
+            except _fused.FusedUnsupported as exc:
+                self.fused_reason = str(exc)
+                indexed.pop("fused_states", None)
+                indexed.pop("fused_offsets", None)
+        self._main_bytes = len(indexed["main_stream"]) if "main_stream" in indexed else 0
+        if plan is not None:  # the fused kernels read 16-byte vectors: pad the stream's allocation
+            indexed["main_stream"] = np.concatenate((indexed["main_stream"], np.zeros(16, dtype=np.uint8)))
+            for key in ("seg_state", "seg_offset", "tile_rows", "tile_class", "lut", "tab"):
+                indexed["fused_" + key] = plan[key]
         for name, array in indexed.items():
             if isinstance(array, np.ndarray):
-                self.buffers[name] = torch.from_numpy(array).to(self.device)
+                self.buffers[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
         for name in ("main", "residual"):
             if name + "_freq" in indexed:
                 cum = _tables.cumulative(indexed[name + "_freq"])
@@ -125,7 +161,21 @@ class HipContextTensor:
             f.col_class = self.buffers["columns"].data_ptr()
             f.rows, f.cols = self.shape
             f.nc, f.mode, f.stride = self.nc, self.mode, stride
+            f.main.n_bytes = self._main_bytes
             self._frame = f
+        if plan is not None:
+            d = _hip_abi.GrfBctxFused()
+            b = self.buffers
+            d.main_bytes, d.raw6 = b["main_stream"].data_ptr(), b["residual_stream"].data_ptr()
+            d.seg_state, d.seg_offset = b["fused_seg_state"].data_ptr(), b["fused_seg_offset"].data_ptr()
+            d.tile_rows, d.tile_class = b["fused_tile_rows"].data_ptr(), b["fused_tile_class"].data_ptr()
+            d.lut, d.tab, d.col_class = b["fused_lut"].data_ptr(), b["fused_tab"].data_ptr(), b["columns"].data_ptr()
+            d.main_n_bytes = self._main_bytes
+            for key, value in plan["scalars"].items():
+                setattr(d, key, value)
+            self.fused = d
+            self.fused_plan = plan["scalars"]
+            self.fused_reason = ""
 
     # ------------------------------------------------------------------ decode
     def _decode_blocks(self, blocks=None, *, check=True):
@@ -150,11 +200,58 @@ class HipContextTensor:
             raise base.CodecError("HIP decoder checkpoint mismatch")
         return result.view(torch.bfloat16)
 
-    def decode(self, *, check=True):
+    def _launch(self, fn, *args):
+        import torch
+        with torch.cuda.device(self.device):
+            status = fn(*args, torch.cuda.current_stream(self.device).cuda_stream)
+        if status:
+            raise base.CodecError(f"device launch failed ({status}): "
+                                  + self._lib.grf_last_error().decode(errors="replace"))
+
+    def _check(self, check):
+        if check and self.error.item() != 0:
+            raise base.CodecError("HIP decoder checkpoint mismatch")
+
+    def decode(self, *, check=True, general=False):
+        """Dense BF16 matrix.  Fused frames use the store sink of the fused walker;
+        ``general=True`` forces the one-lane-per-segment kernel."""
         import torch
         if self.mode == 1:
             return self.buffers["raw"].view(torch.bfloat16).reshape(self.shape)
-        return self._decode_blocks(check=check)[:self.n].reshape(self.shape)
+        if self.fused is None or general:
+            return self._decode_blocks(check=check)[:self.n].reshape(self.shape)
+        out = torch.empty(self.n, device=self.device, dtype=torch.uint16)
+        self.error.zero_()
+        self._launch(self._lib.grf_bctx_fused_decode, ctypes.byref(self.fused), out.data_ptr(), self.error.data_ptr())
+        self._check(check)
+        return out.view(torch.bfloat16).reshape(self.shape)
+
+    def linear(self, x, bias=None, *, check=False):
+        """y = x @ W.T (+ bias) with W decoded inside the kernel; x is BF16 [..., K].
+
+        Up to 8 activation rows run the fused decode-GEMV; other cases decode and call
+        the dense matmul.  ``check=True`` reads the error word back (a host sync)."""
+        import torch
+        import torch.nn.functional as F
+        if x.dtype != torch.bfloat16 or x.shape[-1] != self.shape[1]:
+            raise ValueError("activation must be bfloat16 with the weight's input width")
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.shape[1])
+        m = x2.shape[0]
+        if self.fused is None or not 1 <= m <= 8:
+            return F.linear(x, self.decode(check=check), bias)
+        if x2.stride(-1) != 1:
+            x2 = x2.contiguous()
+        x2 = x2.to(self.device)
+        y = torch.empty((m, self.shape[0]), device=self.device, dtype=torch.bfloat16)
+        if bias is not None:
+            bias = bias.to(device=self.device, dtype=torch.bfloat16).contiguous()
+        self.error.zero_()
+        self._launch(self._lib.grf_bctx_gemv, ctypes.byref(self.fused), x2.data_ptr(), x2.stride(0), m,
+                     y.data_ptr(), y.stride(0), bias.data_ptr() if bias is not None else None,
+                     self.error.data_ptr())
+        self._check(check)
+        return y.reshape(*lead, self.shape[0])
 
     def gather_rows(self, ids, *, check=True):
         import torch

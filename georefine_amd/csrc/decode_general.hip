@@ -10,14 +10,17 @@
 #include "georefine_amd.h"
 #include "rans_device.h"
 
-namespace {
-
+namespace grf {
 thread_local std::string g_error;
-
-int fail(int code, const std::string &what) {
+int set_error(int code, const std::string &what) {
   g_error = what;
   return code;
 }
+}  // namespace grf
+
+namespace {
+
+int fail(int code, const std::string &what) { return grf::set_error(code, what); }
 
 constexpr int kThreads = 256;
 
@@ -165,7 +168,7 @@ int launch_status(const char *what) {
 
 extern "C" {
 
-const char *grf_last_error(void) { return g_error.c_str(); }
+const char *grf_last_error(void) { return grf::g_error.c_str(); }
 int grf_abi_version(void) { return 1; }
 
 int grf_bctx_decode(const grf_bctx_frame *frame, const int64_t *block_ids, uint32_t count, uint16_t *out,

@@ -151,6 +151,54 @@ int grf_ppcx_decode(const grf_ppcx_frame *frame, const uint16_t *reference, uint
 int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *coeff, uint16_t *out,
                     uint32_t rows, uint32_t cols, int32_t *error, void *hip_stream);
 
+/* A mode-0 BCTX frame prepared for the fused kernels.  Segments have a length that
+ * divides the row length, rows are grouped by row class into tiles, and the
+ * per-class lookup tables are laid out for LDS:
+ *   seg_state / seg_offset  u32 [rows*segs_per_row + 1]; the extra last entry is
+ *                           (2^23, main_n_bytes)
+ *   tile_rows   u32 [n_tiles*rows_per_tile]  row of each slot, 0xFFFFFFFF = empty
+ *   tile_class  u8  [n_tiles]                row class shared by the tile's rows
+ *   lut         u8  [nr][nc << lognb]        lognb = 16 - shift; sparse index of the
+ *                                            symbol owning the bucket's first slot
+ *   tab         u64 [nr][(tabn+1)*nc]        entry(sparse, cc) at sparse*nc + cc:
+ *                 low32 = start | (freq-1)<<16
+ *                 high32 = next_start (bits 0..16) | symbol<<21 | (freq < 2^shift)<<31
+ *   col_class   u8  [cols]
+ * main_bytes must be readable for 16 bytes past main_n_bytes. */
+typedef struct grf_bctx_fused {
+  const uint8_t *main_bytes;
+  const uint8_t *raw6;
+  const uint32_t *seg_state;
+  const uint32_t *seg_offset;
+  const uint32_t *tile_rows;
+  const uint8_t *tile_class;
+  const uint8_t *lut;
+  const uint64_t *tab;
+  const uint8_t *col_class;
+  uint32_t main_n_bytes;
+  uint32_t rows, cols;
+  uint32_t nr, nc, lognc;
+  uint32_t seg_len, segs_per_row;
+  uint32_t lanes_per_row, rows_per_tile, n_slabs, n_tiles;
+  uint32_t shift, lognb, tabn;
+  uint32_t piece_cap; /* LDS bytes reserved per row piece (multiple of 16) */
+} grf_bctx_fused;
+
+/* Fused decode-GEMV, the slot the reference leaves for "a backend with a fused GEMM"
+ * behind the CudaContextTensor contract (GCR/bitexact_context_serving.py:3-5; it replaces
+ * decode() + F.linear of BctxLinear.forward, :365-376).  y[m][n] = bf16(sum_k x[m][k] *
+ * W[n][k] + bias[n]) for 1 <= m_rows <= 8, fp32 accumulation in an order that does not
+ * depend on m_rows (the M-invariance contract of GS/miv_gemv.py:10-29).
+ * x: BF16 [m_rows][ldx], y: BF16 [m_rows][ldy], bias: BF16 [rows] or NULL. */
+int grf_bctx_gemv(const grf_bctx_fused *frame, const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint16_t *y,
+                  uint32_t ldy, const uint16_t *bias, int32_t *error, void *hip_stream);
+
+/* Same walker with a store sink: out[rows*cols] BF16 words (decode() for fused frames). */
+int grf_bctx_fused_decode(const grf_bctx_fused *frame, uint16_t *out, int32_t *error, void *hip_stream);
+
+/* LDS bytes a launch on this frame needs for the given m_rows (0 for the store sink). */
+uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, uint32_t m_rows);
+
 const char *grf_last_error(void);
 int grf_abi_version(void);
 

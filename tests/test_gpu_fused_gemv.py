@@ -1,0 +1,110 @@
+"""Fused decode-GEMV and the fused store sink against the oracle and float64 matmul."""
+import numpy as np
+import pytest
+
+from conftest import bf16_words, weight_like, words_to_float
+
+pytestmark = pytest.mark.gpu
+
+
+def _wide_range(rng, rows, cols):
+    """Magnitudes spread over ~40 binades: many rare symbols, exercises the forward scan."""
+    mag = np.exp2(rng.uniform(-30, 10, size=(rows, cols))).astype(np.float32)
+    return bf16_words(mag * rng.choice([-1.0, 1.0], size=(rows, cols)).astype(np.float32))
+
+
+def _tensor(words, nr=16, nc=4, **kw):
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd.bitexact_context_gpu import HipContextTensor
+    frame = codec.encode(words, row_classes=nr, col_classes=nc)
+    return frame, HipContextTensor(frame, stride=1024, device="cuda:0", **kw)
+
+
+SHAPES = [(64, 256), (100, 384), (37, 1024), (512, 1280), (16, 2176), (300, 48)]
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: f"{s[0]}x{s[1]}")
+@pytest.mark.parametrize("classes", [(16, 4), (1, 1), (64, 16), (4, 16)], ids=lambda c: f"nr{c[0]}nc{c[1]}")
+def test_fused_decode_bit_exact(oracle, shape, classes):
+    import torch
+    rng = np.random.default_rng(shape[0] * 7 + shape[1])
+    words = weight_like(rng, *shape)
+    frame, t = _tensor(words, *classes)
+    print(f"shape={shape} classes={classes} mode={t.mode} fused={t.fused is not None} {t.fused_reason}", flush=True)
+    if t.mode != 0:
+        pytest.skip("encoder did not choose mode 0")
+    assert t.fused is not None, t.fused_reason
+    expect = oracle.bctx_decode(frame)
+    got = t.decode().view(torch.uint16).cpu().numpy()
+    assert np.array_equal(got, expect)
+    assert np.array_equal(t.decode(general=True).view(torch.uint16).cpu().numpy(), expect)
+
+
+@pytest.mark.parametrize("segment", [16, 32, 64, 128, 256])
+def test_fused_decode_every_segment_length(oracle, segment):
+    import torch
+    words = weight_like(np.random.default_rng(segment), 96, 768)
+    frame, t = _tensor(words, fused_segment=segment)
+    assert t.fused is not None and t.fused_plan["seg_len"] == segment
+    assert np.array_equal(t.decode().view(torch.uint16).cpu().numpy(), words)
+
+
+def test_fused_decode_rare_symbols_forward_scan(oracle):
+    import torch
+    words = _wide_range(np.random.default_rng(3), 128, 512)
+    frame, t = _tensor(words)
+    print("mode", t.mode, "fused", t.fused is not None, t.fused_reason, getattr(t, "fused_plan", None), flush=True)
+    if t.fused is None:
+        pytest.skip("frame not eligible: " + t.fused_reason)
+    assert np.array_equal(t.decode().view(torch.uint16).cpu().numpy(), words)
+
+
+@pytest.mark.parametrize("shape", [(64, 256), (512, 1280), (100, 384), (16, 2176)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_gemv_matches_float64_and_is_m_invariant(oracle, shape):
+    import torch
+    rng = np.random.default_rng(shape[1])
+    words = weight_like(rng, *shape)
+    frame, t = _tensor(words)
+    assert t.fused is not None, t.fused_reason
+    w64 = words_to_float(oracle.bctx_decode(frame)).astype(np.float64)
+    xw = bf16_words(rng.normal(0, 1, size=(8, shape[1])))
+    x = torch.from_numpy(xw).view(torch.bfloat16).cuda()
+    ref = words_to_float(xw).astype(np.float64) @ w64.T
+    scale = np.abs(words_to_float(xw).astype(np.float64)) @ np.abs(w64).T
+    y8 = t.linear(x, check=True)
+    got = words_to_float(y8.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    # relative to the magnitude of the terms: 1e-2 is the stated bar, BF16 rounding is ~4e-3 of |y|
+    assert np.all(np.abs(got - ref) <= 1e-2 * np.maximum(np.abs(ref), 1e-3 * scale) + 1e-30)
+    dense = torch.nn.functional.linear(x.float(), t.decode().float()).double().cpu().numpy()
+    assert np.all(np.abs(got - dense) <= 1e-2 * np.maximum(np.abs(dense), 1e-3 * scale) + 1e-30)
+    for m in (1, 2, 3, 5, 8):
+        ym = t.linear(x[:m], check=True)
+        assert torch.equal(ym.view(torch.uint16), y8[:m].view(torch.uint16)), f"M={m} rows differ from M=8"
+    y1 = torch.cat([t.linear(x[i:i + 1]) for i in range(8)])
+    assert torch.equal(y1.view(torch.uint16), y8.view(torch.uint16))
+
+
+def test_gemv_bias_and_batched_input(oracle):
+    import torch
+    rng = np.random.default_rng(17)
+    words = weight_like(rng, 96, 512)
+    frame, t = _tensor(words)
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(2, 3, 512)))).view(torch.bfloat16).cuda()
+    bias = torch.from_numpy(bf16_words(rng.normal(0, 1, size=96))).view(torch.bfloat16).cuda()
+    y = t.linear(x, bias, check=True)
+    assert y.shape == (2, 3, 96)
+    ref = torch.nn.functional.linear(x.double(), t.decode().double(), bias.double())
+    assert torch.allclose(y.double(), ref, rtol=1e-2, atol=1e-2)
+
+
+def test_fused_checkpoint_mismatch_sets_error(oracle):
+    import torch
+    from georefine_amd import bitexact_context_codec as codec
+    words = weight_like(np.random.default_rng(23), 64, 512)
+    frame, t = _tensor(words)
+    t.buffers["fused_seg_state"].view(torch.int32)[5] += 1  # forced from the host; the kernel finishes normally
+    x = torch.zeros(1, 512, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(codec.CodecError):
+        t.linear(x, check=True)
+    assert t.linear(x).shape == (1, 64)
+    assert t.error.item() != 0
