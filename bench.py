@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Headline benchmark: fused decode-GEMV at batch 1 on Qwen-27B-like MLP shapes.
+
+One step = one pass of the hot path over the three coded MLP matrices of a layer
+(gate and up: 17408x5120, down: 5120x17408), i.e. three fused decode-GEMV
+launches on seeded synthetic BF16 weights (N(0,0.02) with per-row log-normal(0,0.5)
+scale and 0.1% outliers at 10x) against an N(0,1) BF16 activation vector.  The
+three matrices together are ~354 MB coded, more than L2 + Infinity Cache, so
+every step streams its compressed bytes from HBM.
+
+Prints ONE JSON line: metric = compressed bytes consumed per second (GB/s), with
+the achieved fraction of the 8 TB/s HBM roofline for the dominant kernel and a
+CPU baseline (the CPU oracle's decode + matvec on the host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0
+MODEL_BF16_BYTES = 55_586_113_293  # dense BF16 bytes of the 27B model one token has to read at batch 1
+SHAPES = {"gate": (17408, 5120), "up": (17408, 5120), "down": (5120, 17408)}
+
+
+def log(*a):
+    print("[bench]", *a, file=sys.stderr, flush=True)
+
+
+def bf16_words(values):
+    u = np.ascontiguousarray(values, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def synth_weights(index, rows, cols):
+    rng = np.random.default_rng(1000 + index)
+    out = np.empty((rows, cols), dtype=np.uint16)
+    scale = rng.lognormal(0.0, 0.5, size=(rows, 1)).astype(np.float32)
+    step = 2048
+    for lo in range(0, rows, step):  # chunked so the float temporaries stay small
+        hi = min(rows, lo + step)
+        w = rng.normal(0.0, 0.02, size=(hi - lo, cols)).astype(np.float32) * scale[lo:hi]
+        mask = rng.random((hi - lo, cols)) < 1e-3
+        w = np.where(mask, w * np.float32(10.0), w)
+        out[lo:hi] = bf16_words(w)
+    return out
+
+
+def algorithmic_bytes(t, m):
+    """Bytes one fused GEMV launch has to touch once: both streams, the fused index,
+    the per-class lookup tables, labels, activations and outputs."""
+    b = t.buffers
+    n = lambda k: b[k].numel() * b[k].element_size()
+    rows, cols = t.shape
+    payload = t._main_bytes + n("residual_stream")
+    _, tile_rows, tile_class, _ = t._tiling(m)
+    index = (n("fused_seg_state") + n("fused_seg_offset") + tile_rows.numel() * tile_rows.element_size()
+             + tile_class.numel() * tile_class.element_size())
+    tables = n("fused_lut") + n("fused_tab")
+    labels = cols
+    io = m * cols * 2 + m * rows * 2
+    return dict(total=payload + index + tables + labels + io, payload=payload, index=index, tables=tables)
+
+
+def cpu_baseline(frame, words, x_words, sample_rows):
+    """The CPU oracle (full 65536-slot lookup, one thread, as the reference decodes a
+    frame) on a row slab of the same matrix, plus an fp32 matvec on the host."""
+    from oracle import codec_oracle as orc
+    from georefine_amd import bitexact_context_codec as codec
+    sub = np.ascontiguousarray(words[:sample_rows])
+    sub_frame = codec.encode(sub)
+    t0 = time.perf_counter()
+    dec = orc.bctx_decode(sub_frame)
+    wf = (dec.astype(np.uint32) << 16).view(np.float32)
+    xf = (x_words.astype(np.uint32) << 16).view(np.float32)
+    y = wf @ xf
+    dt = time.perf_counter() - t0
+    assert np.array_equal(dec, sub), "CPU oracle decode is not bit-exact"
+    coded = len(sub_frame)
+    return dict(value=coded / dt / 1e9, unit="GB/s", cores=1, kind="port",
+                sample=f"first {sample_rows} rows of gate ({sample_rows}x{sub.shape[1]}, {coded} coded bytes): "
+                       f"frame parse + sha256 + full-LUT rANS decode + 6-bit unpack + fp32 matvec in {dt:.2f}s "
+                       f"({sub.nbytes / dt / 1e6:.1f} MB/s of BF16 produced)",
+                checksum=float(np.sum(y)))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=1, help="activation rows per GEMV (1..8)")
+    ap.add_argument("--segment", type=int, default=0, help="fused segment length (0 = automatic)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-rows", type=int, default=4096)
+    ap.add_argument("--only", default="", help="comma list of gate,up,down (profiling aid)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this decode path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists)")
+
+    import torch
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd.bitexact_context_gpu import HipContextTensor
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs a ROCm GPU")
+    names = [s for s in args.only.split(",") if s] or list(SHAPES)
+    tensors, frames, words_of = {}, {}, {}
+    t_setup = time.perf_counter()
+    for i, name in enumerate(SHAPES):
+        if name not in names:
+            continue
+        rows, cols = SHAPES[name]
+        w = synth_weights(i, rows, cols)
+        t0 = time.perf_counter()
+        frame = codec.encode(w)
+        t1 = time.perf_counter()
+        tensors[name] = HipContextTensor(frame, stride=1024, device="cuda:0",
+                                         fused_segment=args.segment or None)
+        t2 = time.perf_counter()
+        if tensors[name].fused is None:
+            sys.exit(f"bench.py: {name} is not eligible for the fused kernel: {tensors[name].fused_reason}")
+        log(f"{name}: {rows}x{cols} mode {tensors[name].mode} frame {len(frame)} B "
+            f"({8 * len(frame) / w.size:.3f} bit/weight) encode {t1 - t0:.1f}s index+upload {t2 - t1:.1f}s "
+            f"plan {tensors[name].fused_plan} tiling {tensors[name]._tiling(args.batch)[3]}")
+        frames[name] = frame
+        if name == "gate":
+            words_of[name] = w
+    log(f"setup {time.perf_counter() - t_setup:.1f}s")
+
+    m = args.batch
+    rng = np.random.default_rng(7)
+    x_words = {k: bf16_words(rng.normal(0, 1, size=(m, k))) for k in (5120, 17408)}
+    x = {k: torch.from_numpy(v).view(torch.bfloat16).cuda() for k, v in x_words.items()}
+
+    def step():
+        outs = []
+        for name in names:
+            outs.append(tensors[name].linear(x[SHAPES[name][1]]))
+        return outs
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    for name in names:
+        if tensors[name].error.item():
+            sys.exit(f"bench.py: decoder error word set for {name}")
+
+    # per-launch durations with events on the stream the kernels run on
+    starts = [[torch.cuda.Event(enable_timing=True) for _ in names] for _ in range(args.steps)]
+    ends = [[torch.cuda.Event(enable_timing=True) for _ in names] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    wall0 = time.perf_counter()
+    for s in range(args.steps):
+        for j, name in enumerate(names):
+            starts[s][j].record()
+            tensors[name].linear(x[SHAPES[name][1]])
+            ends[s][j].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    for name in names:
+        if tensors[name].error.item():
+            sys.exit(f"bench.py: decoder error word set for {name}")
+
+    per_kernel_ms = {name: float(np.mean([starts[s][j].elapsed_time(ends[s][j]) for s in range(args.steps)]))
+                     for j, name in enumerate(names)}
+    alg = {name: algorithmic_bytes(tensors[name], m) for name in names}
+    step_bytes = sum(a["total"] for a in alg.values())
+    dense_bytes = sum(2 * SHAPES[n][0] * SHAPES[n][1] for n in names)
+    ms_per_step = wall / args.steps * 1e3
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    eff_bf16 = dense_bytes / (ms_per_step * 1e-3) / 1e9
+
+    dom = max(names, key=lambda n_: per_kernel_ms[n_])
+    achieved = alg[dom]["total"] / (per_kernel_ms[dom] * 1e-3) / 1e9
+    result = {
+        "metric": "compressed-weight decode-GEMV GB/s",
+        "value": round(value, 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": "fused decode-GEMV, batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
+                               "BCTX (16,4) mode-0 frames" % m,
+                   "batch": m, "matrices": names,
+                   "segment": tensors[names[0]].fused_plan["seg_len"]},
+        "effective_bf16_GBps": round(eff_bf16, 2),
+        "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3),
+        "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
+        "per_kernel": {n_: {"ms": round(per_kernel_ms[n_], 4), "alg_bytes": alg[n_]["total"],
+                            "payload_bytes": alg[n_]["payload"], "index_bytes": alg[n_]["index"],
+                            "table_bytes": alg[n_]["tables"],
+                            "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in names},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": f"fused_walk_kernel<{m},false> on {dom}"},
+    }
+    if not args.no_cpu_baseline and "gate" in words_of:
+        log("timing the CPU oracle on a row slab of gate ...")
+        result["cpu_baseline"] = cpu_baseline(frames["gate"], words_of["gate"], x_words[5120][0], args.cpu_rows)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

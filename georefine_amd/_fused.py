@@ -12,7 +12,6 @@ import os
 
 import numpy as np
 
-THREADS = 256
 MAX_LDS = 160 * 1024
 LUT_BUDGET = int(os.environ.get("GEOREFINE_FUSED_LUT_BYTES", 16 * 1024))
 
@@ -40,12 +39,10 @@ def choose_shift(nc, budget=LUT_BUDGET):
 
 
 def sparse_tables(freq, nr, nc, shift):
-    """Per row class: u8 lookup [nc << lognb] and u64 entries [(tabn+1)*nc].
+    """Per row class: u8 lookup [nc << lognb] and u64 entries [nc][tabn+1].
 
-    Entry(sparse i, column class c) sits at i*nc + c:
-    low32 = start | (freq-1) << 16, high32 = next_start | symbol << 21 | (freq < 2^shift) << 31.
-    Unused slots hold next_start = 65536 so a forward scan always stops there."""
-    vocab = freq.shape[1]
+    Entry(column class c, sparse i): low32 = start | (freq-1) << 16, high32 = symbol << 21.
+    Unused entries are (start 0, freq 65536): a forward scan always stops on them."""
     nz = freq > 0
     tabn = int(nz.sum(axis=1).max())
     if tabn == 0:
@@ -55,8 +52,7 @@ def sparse_tables(freq, nr, nc, shift):
     lognb = 16 - shift
     nb = 1 << lognb
     lut = np.zeros((nr, nc, nb), dtype=np.uint8)
-    filler = np.uint64(65536) << np.uint64(32)
-    tab = np.full((nr, tabn + 1, nc), filler, dtype=np.uint64)
+    tab = np.full((nr, nc, tabn + 1), np.uint64(0xFFFF0000), dtype=np.uint64)
     first_slots = (np.arange(nb, dtype=np.int64) << shift)
     for rho in range(nr):
         for c in range(nc):
@@ -66,22 +62,23 @@ def sparse_tables(freq, nr, nc, shift):
                 continue
             fs = f[syms]
             starts = np.concatenate(([0], np.cumsum(fs)[:-1]))
-            nxt = starts + fs
             lo = starts | ((fs - 1) << 16)
-            hi = nxt | (syms << 21) | ((fs < (1 << shift)).astype(np.int64) << 31)
-            tab[rho, :syms.size, c] = (lo.astype(np.uint64) | (hi.astype(np.uint64) << np.uint64(32)))
+            hi = syms << 21
+            tab[rho, c, :syms.size] = (lo.astype(np.uint64) | (hi.astype(np.uint64) << np.uint64(32)))
             lut[rho, c] = (np.searchsorted(starts, first_slots, side="right") - 1).astype(np.uint8)
-    return lut.reshape(nr, nc * nb), tab.reshape(nr, (tabn + 1) * nc), tabn
+    return lut.reshape(nr, nc * nb), tab.reshape(nr, nc * (tabn + 1)), tabn
 
 
-def lds_bytes(nc, lognb, tabn, m, p, s, r, piece_cap):
+X_PAD = 8
+TAB_CAP = 257  # entries reserved per column class in LDS
+
+
+def lds_bytes(nc, lognb, tabn, m, p, s, r, piece_cap, spr):
     a16 = lambda v: (v + 15) // 16 * 16
-    total = a16(nc << lognb)
-    total = a16(total + (tabn + 1) * nc * 8)
-    total = a16(total + m * p * (s + 4) * 4)
-    total = a16(total + p * s)
+    total = a16(nc * (TAB_CAP * 8 + (1 << lognb)))
     total = a16(total + r * piece_cap)
-    total = a16(total + r * p * m * 4)
+    total = a16(total + m * p * (s + X_PAD) * 2)
+    total = a16(total + r * spr * m * 4)
     return total
 
 
@@ -98,30 +95,37 @@ def piece_capacity(offsets, rows, spr, p):
     return (longest + 2 + 15) // 16 * 16
 
 
-def choose_tiling(rows, spr, class_rows, piece_cap_fn, lds_fn, cus=256):
-    """(lanes_per_row P, rows_per_tile R): best modelled throughput.
+def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
+    """(threads T, lanes_per_row P, rows_per_tile R, ...): best modelled throughput.
 
-    Model: lane efficiency (idle lanes in the last slab and in a partly filled
-    workgroup) times how evenly the tiles fill the machine at the occupancy LDS allows."""
+    The walk is a chain of dependent steps per lane, so time ~ steps per lane x rounds
+    of workgroups, at the speed the resident wave count allows.  The model multiplies
+    lane efficiency (idle lanes in the last slab and in a partly filled workgroup), tile
+    fill, how evenly the tiles fill the machine, and a penalty below 16 waves per CU."""
     best = None
-    for p in range(1, min(spr, THREADS) + 1):
-        r = THREADS // p
-        n_slabs = -(-spr // p)
-        lane_eff = spr / (n_slabs * p) * (p * r / THREADS)
-        tiles = sum(-(-int(cnt) // r) for cnt in class_rows if cnt)
-        fill = sum(int(cnt) for cnt in class_rows) / (tiles * r)
-        cap = piece_cap_fn(p)
-        lds = lds_fn(p, r, cap)
-        if lds > MAX_LDS:
-            continue
-        per_cu = max(1, min(8, MAX_LDS // lds))
-        slots = cus * per_cu
-        rounds = -(-tiles // slots)
-        quant = tiles / (rounds * slots)
-        occupancy = min(1.0, per_cu / 4)  # fewer than 4 workgroups per CU hides latency poorly
-        score = lane_eff * fill * quant * (0.5 + 0.5 * occupancy)
-        if best is None or score > best[0] + 1e-9:
-            best = (score, p, r, n_slabs, tiles, cap, lds)
+    total_rows = sum(int(c) for c in class_rows)
+    for threads in (1024, 512, 256):
+        for p in range(1, min(spr, threads) + 1):
+            r = threads // p
+            n_slabs = -(-spr // p)
+            if p > 1 and -(-spr // (p - 1)) == n_slabs:
+                continue  # a narrower slab of the same count wastes fewer lanes; it was scored already
+            lanes = p * r
+            lane_eff = spr / (n_slabs * p) * (lanes / threads)
+            tiles = sum(-(-int(cnt) // r) for cnt in class_rows if cnt)
+            fill = total_rows / (tiles * r)
+            cap = piece_cap_fn(p)
+            lds = lds_fn(p, r, cap)
+            if lds > MAX_LDS:
+                continue
+            per_cu = max(1, min(2048 // threads, MAX_LDS // lds))
+            waves = per_cu * threads // 64
+            slots = cus * per_cu
+            rounds = -(-tiles // slots)
+            quant = tiles / (rounds * slots)
+            score = lane_eff * fill * quant * min(1.0, waves / 16)
+            if best is None or score > best[0] + 1e-9:
+                best = (score, threads, p, r, n_slabs, tiles, cap, lds)
     if best is None:
         raise FusedUnsupported("no tiling fits in LDS")
     return best[1:]
@@ -146,30 +150,41 @@ def build_tiles(row_class, nr, r):
     return np.concatenate(tiles), np.asarray(classes, dtype=np.uint8)
 
 
-def plan(shape, nr, nc, row_class, main_freq, seg_states, seg_offsets, main_bytes, seg_len, m_for_lds=8):
-    """All host arrays and scalars of a ``grf_bctx_fused`` descriptor."""
-    rows, cols = shape
-    if rows * cols > 0xFFFFFFFF:
-        raise FusedUnsupported("matrix too large")
-    spr = cols // seg_len
-    shift = choose_shift(nc)
-    lut, tab, tabn = sparse_tables(main_freq, nr, nc, shift)
-    lognb = 16 - shift
-    states = np.concatenate((seg_states, [1 << 23])).astype(np.uint32)
-    offsets = np.concatenate((seg_offsets, [main_bytes])).astype(np.uint32)
-    counts = np.bincount(row_class, minlength=nr)
-    caps = {}
+class FramePlan:
+    """Frame-level derived arrays (shared by every tiling) and a tiling factory."""
 
-    def cap_of(p):
-        if p not in caps:
-            caps[p] = piece_capacity(offsets, rows, spr, p)
-        return caps[p]
+    def __init__(self, shape, nr, nc, row_class, main_freq, seg_states, seg_offsets, main_bytes, seg_len):
+        rows, cols = shape
+        if rows * cols > 0xFFFFFFFF:
+            raise FusedUnsupported("matrix too large")
+        self.rows, self.cols, self.nr, self.nc, self.seg_len = rows, cols, nr, nc, seg_len
+        self.spr = cols // seg_len
+        self.shift = choose_shift(nc)
+        self.lognb = 16 - self.shift
+        self.lut, self.tab, self.tabn = sparse_tables(main_freq, nr, nc, self.shift)
+        self.seg_state = np.concatenate((seg_states, [1 << 23])).astype(np.uint32)
+        self.seg_offset = np.concatenate((seg_offsets, [main_bytes])).astype(np.uint32)
+        self.row_class = np.asarray(row_class)
+        self.class_rows = np.bincount(self.row_class, minlength=nr)
+        self._caps = {}
 
-    p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
-        rows, spr, counts, cap_of, lambda p_, r_, cap_: lds_bytes(nc, lognb, tabn, m_for_lds, p_, seg_len, r_, cap_))
-    tile_rows, tile_class = build_tiles(row_class, nr, r)
-    assert len(tile_class) == n_tiles
-    return dict(seg_state=states, seg_offset=offsets, tile_rows=tile_rows, tile_class=tile_class, lut=lut, tab=tab,
-                scalars=dict(rows=rows, cols=cols, nr=nr, nc=nc, lognc=int(math.log2(nc)), seg_len=seg_len,
-                             segs_per_row=spr, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs, n_tiles=n_tiles,
-                             shift=shift, lognb=lognb, tabn=tabn, piece_cap=cap))
+    def scalars(self):
+        return dict(rows=self.rows, cols=self.cols, nr=self.nr, nc=self.nc, seg_len=self.seg_len,
+                    segs_per_row=self.spr, shift=self.shift, lognb=self.lognb, tabn=self.tabn)
+
+    def _cap(self, p):
+        if p not in self._caps:
+            self._caps[p] = piece_capacity(self.seg_offset, self.rows, self.spr, p)
+        return self._caps[p]
+
+    def tiling(self, m):
+        """Host arrays and scalars of a ``grf_fused_tiling`` sized for m activation rows
+        (m = 0: the store sink)."""
+        threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
+            self.spr, self.class_rows, self._cap,
+            lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_, self.spr))
+        tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
+        assert len(tile_class) == n_tiles
+        return dict(tile_rows=tile_rows, tile_class=tile_class,
+                    scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
+                                 n_tiles=n_tiles, piece_cap=cap), lds=lds)

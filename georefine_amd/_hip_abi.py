@@ -26,11 +26,16 @@ class GrfPpcxFrame(ctypes.Structure):
 
 class GrfBctxFused(ctypes.Structure):
     _fields_ = [("main_bytes", ctypes.c_void_p), ("raw6", ctypes.c_void_p), ("seg_state", ctypes.c_void_p),
-                ("seg_offset", ctypes.c_void_p), ("tile_rows", ctypes.c_void_p), ("tile_class", ctypes.c_void_p),
-                ("lut", ctypes.c_void_p), ("tab", ctypes.c_void_p), ("col_class", ctypes.c_void_p)] + [
+                ("seg_offset", ctypes.c_void_p), ("lut", ctypes.c_void_p), ("tab", ctypes.c_void_p),
+                ("col_class", ctypes.c_void_p)] + [
         (name, ctypes.c_uint32) for name in (
-            "main_n_bytes", "rows", "cols", "nr", "nc", "lognc", "seg_len", "segs_per_row", "lanes_per_row",
-            "rows_per_tile", "n_slabs", "n_tiles", "shift", "lognb", "tabn", "piece_cap")]
+            "main_n_bytes", "rows", "cols", "nr", "nc", "seg_len", "segs_per_row", "shift", "lognb", "tabn")]
+
+
+class GrfFusedTiling(ctypes.Structure):
+    _fields_ = [("tile_rows", ctypes.c_void_p), ("tile_class", ctypes.c_void_p)] + [
+        (name, ctypes.c_uint32) for name in (
+            "threads", "lanes_per_row", "rows_per_tile", "n_slabs", "n_tiles", "piece_cap")]
 
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
@@ -45,11 +50,12 @@ def declare(L):
     L.grf_ppcx_decode.restype = i
     L.grf_mix_predict.argtypes = [vp, vp, vp, vp, u32, u32, vp, vp]
     L.grf_mix_predict.restype = i
-    L.grf_bctx_gemv.argtypes = [ctypes.POINTER(GrfBctxFused), vp, u32, u32, vp, u32, vp, vp, vp]
+    tiling = ctypes.POINTER(GrfFusedTiling)
+    L.grf_bctx_gemv.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, u32, u32, vp, u32, vp, vp, vp]
     L.grf_bctx_gemv.restype = i
-    L.grf_bctx_fused_decode.argtypes = [ctypes.POINTER(GrfBctxFused), vp, vp, vp]
+    L.grf_bctx_fused_decode.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, vp, vp]
     L.grf_bctx_fused_decode.restype = i
-    L.grf_bctx_fused_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), u32]
+    L.grf_bctx_fused_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, u32]
     L.grf_bctx_fused_lds_bytes.restype = u32
     L.grf_last_error.restype = ctypes.c_char_p
     L.grf_abi_version.restype = i

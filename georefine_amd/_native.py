@@ -108,6 +108,8 @@ def codec():
             L.bcx_unpack6.argtypes = [U8P, _sz, _u64, U16P]
             L.bcx_checkpoint.argtypes = [U8P, _sz, _u64, _u32, _u32, U8P, U8P, _u32, _u32, _u32, U16P, U32P,
                                          _u32, U32P, U32P, U16P]
+            L.grf_bctx_join.argtypes = [U16P, U16P, _u64, U16P]
+            L.grf_bctx_join.restype = _int
             L.p_encode.argtypes = [U16P, U16P, _u64, _u32, _u32, ctypes.POINTER(U32P), ctypes.POINTER(U8P),
                                    ctypes.POINTER(_sz)]
             L.p_decode.argtypes = [U8P, _sz, _u64, U16P, _u32, _u32, U32P, U16P]

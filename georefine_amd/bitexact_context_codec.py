@@ -169,9 +169,13 @@ def _inflate_exact(data, expected):
 
 def recombine(main, residual):
     """10-bit main symbol + 6-bit residual -> BF16 word (GCR/bitexact_context_codec.py:426)."""
-    m = np.asarray(main).astype(np.uint32)
-    r = np.asarray(residual).astype(np.uint32)
-    return ((m << 5) | (r & 31) | ((r >> 5) << 15)).astype("<u2")
+    m = np.ascontiguousarray(main, dtype="<u2").ravel()
+    r = np.ascontiguousarray(residual, dtype="<u2").ravel()
+    out = np.empty(m.size, dtype="<u2")
+    if m.size != r.size or _lib().grf_bctx_join(_native.ptr(m, ctypes.c_uint16), _native.ptr(r, ctypes.c_uint16),
+                                                 m.size, _native.ptr(out, ctypes.c_uint16)):
+        raise CodecError("symbol outside its alphabet")
+    return out
 
 
 def _frame(mode, nr, nc, r, c, meta, table, sy, rs, raw, dig):

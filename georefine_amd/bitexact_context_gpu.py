@@ -44,12 +44,17 @@ def checkpoints(stream, freq, rows, columns, shape, nr, nc, stride, main=None):
     return states, offsets, out
 
 
-def index_frame(frame: bytes, stride: int = 1024, *, fused_segment=None):
+def index_frame(frame: bytes, stride: int = 1024, *, fused_segment=None, raw6_residual=False):
     """Parse, validate and index a frame; the decoded words must hash to the header digest.
 
     With ``fused_segment`` (a segment length dividing the row length) the result also
     carries ``fused_states`` / ``fused_offsets``, the main-stream index at that length.
-    One validated walk serves both indexes when the lengths are multiples of each other."""
+    One validated walk serves both indexes when the lengths are multiples of each other.
+
+    ``raw6_residual``: a mode-128 frame's residual section is validated, decoded and
+    re-packed into the 6-bit raw form (the form the encoder itself emits for mode 0,
+    GCR/bitexact_context_ans.cpp:328-345); the result then carries ``resident_mode`` 0 and
+    no residual index.  The main stream's bytes are never altered."""
     if not isinstance(stride, int) or not 1 <= stride <= 65536:
         raise base.CodecError("invalid checkpoint stride")
     if len(frame) < base.HEADER.size + 32:
@@ -61,10 +66,13 @@ def index_frame(frame: bytes, stride: int = 1024, *, fused_segment=None):
            "frame_bytes": len(frame)}
     if info["mode"] == 1:
         out["raw"] = info["raw"].reshape(-1).astype(np.uint16)
+        out["resident_mode"] = 1
         return out
     rows, columns, sf = info["rows"], info["columns"], info["main_freq"]
     sy, rs = info["main_stream"], info["residual_stream"]
-    fine = fused_segment if (fused_segment and info["mode"] == 0) else None
+    repack = raw6_residual and info["mode"] == 128
+    out["resident_mode"] = 0 if repack else info["mode"]
+    fine = fused_segment if (fused_segment and out["resident_mode"] == 0) else None
     if fine and stride % fine == 0:
         fs, fo, main = checkpoints(sy, sf, rows, columns, (r, c), info["nr"], info["nc"], fine)
         states, offsets = fs[::stride // fine].copy(), fo[::stride // fine].copy()
@@ -78,12 +86,17 @@ def index_frame(frame: bytes, stride: int = 1024, *, fused_segment=None):
                main_states=states, main_offsets=offsets, residual_stream=np.frombuffer(rs, dtype=np.uint8).copy())
     if info["mode"] == 128:
         rf = info["residual_freq"]
-        states, offsets, residual = checkpoints(rs, rf, rows, columns, (r, c), info["nr"], info["nc"], stride, main)
-        out.update(residual_freq=rf, residual_states=states, residual_offsets=offsets)
+        states, offsets, residual = checkpoints(rs, rf, rows, columns, (r, c), info["nr"], info["nc"],
+                                                r * c if repack else stride, main)
+        if not repack:
+            out.update(residual_freq=rf, residual_states=states, residual_offsets=offsets)
     else:
         residual = base._unpack6(base._lib(), rs, r * c)
-    if hashlib.sha256(base.recombine(main, residual).tobytes()).digest() != info["digest"]:
+    words = base.recombine(main, residual)
+    if hashlib.sha256(words.tobytes()).digest() != info["digest"]:
         raise base.CodecError("indexed source checksum mismatch")
+    if repack:
+        out["residual_stream"] = np.frombuffer(base._pack6(base._lib(), words), dtype=np.uint8).copy()
     return out
 
 
@@ -112,13 +125,15 @@ class HipContextTensor:
         if fused:
             try:
                 segment = _fused.choose_segment(base.HEADER.unpack_from(frame)[6], fused_segment)
-            except (_fused.FusedUnsupported, Exception):
+            except _fused.FusedUnsupported:
                 segment = None
-        indexed = index_frame(frame, stride, fused_segment=segment)
+        indexed = index_frame(frame, stride, fused_segment=segment, raw6_residual=segment is not None)
         self.shape = indexed["shape"]
         self.n = math.prod(self.shape)
         self.stride = stride
         self.mode, self.nr, self.nc = indexed["mode"], indexed["nr"], indexed["nc"]
+        # form of the residual section on the device: 0 = packed 6-bit, 128 = rANS stream
+        self.resident_mode = indexed["resident_mode"]
         self.source_sha256 = indexed["source_sha256"]
         self.frame_sha256 = indexed["frame_sha256"]
         self.frame_bytes = indexed["frame_bytes"]
@@ -129,9 +144,9 @@ class HipContextTensor:
         plan = None
         if "fused_states" in indexed:
             try:
-                plan = _fused.plan(self.shape, self.nr, self.nc, indexed["rows"], indexed["main_freq"],
-                                   indexed.pop("fused_states"), indexed.pop("fused_offsets"),
-                                   len(indexed["main_stream"]), indexed["fused_segment"])
+                plan = _fused.FramePlan(self.shape, self.nr, self.nc, indexed["rows"], indexed["main_freq"],
+                                        indexed.pop("fused_states"), indexed.pop("fused_offsets"),
+                                        len(indexed["main_stream"]), indexed["fused_segment"])
             except _fused.FusedUnsupported as exc:
                 self.fused_reason = str(exc)
                 indexed.pop("fused_states", None)
@@ -139,8 +154,8 @@ class HipContextTensor:
         self._main_bytes = len(indexed["main_stream"]) if "main_stream" in indexed else 0
         if plan is not None:  # the fused kernels read 16-byte vectors: pad the stream's allocation
             indexed["main_stream"] = np.concatenate((indexed["main_stream"], np.zeros(16, dtype=np.uint8)))
-            for key in ("seg_state", "seg_offset", "tile_rows", "tile_class", "lut", "tab"):
-                indexed["fused_" + key] = plan[key]
+            indexed.update(fused_seg_state=plan.seg_state, fused_seg_offset=plan.seg_offset, fused_lut=plan.lut,
+                           fused_tab=plan.tab)
         for name, array in indexed.items():
             if isinstance(array, np.ndarray):
                 self.buffers[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
@@ -160,22 +175,45 @@ class HipContextTensor:
             f.row_class = self.buffers["rows"].data_ptr()
             f.col_class = self.buffers["columns"].data_ptr()
             f.rows, f.cols = self.shape
-            f.nc, f.mode, f.stride = self.nc, self.mode, stride
+            f.nc, f.mode, f.stride = self.nc, self.resident_mode, stride
             f.main.n_bytes = self._main_bytes
             self._frame = f
+        self._plan = plan
+        self._tilings = {}
         if plan is not None:
             d = _hip_abi.GrfBctxFused()
             b = self.buffers
             d.main_bytes, d.raw6 = b["main_stream"].data_ptr(), b["residual_stream"].data_ptr()
             d.seg_state, d.seg_offset = b["fused_seg_state"].data_ptr(), b["fused_seg_offset"].data_ptr()
-            d.tile_rows, d.tile_class = b["fused_tile_rows"].data_ptr(), b["fused_tile_class"].data_ptr()
             d.lut, d.tab, d.col_class = b["fused_lut"].data_ptr(), b["fused_tab"].data_ptr(), b["columns"].data_ptr()
             d.main_n_bytes = self._main_bytes
-            for key, value in plan["scalars"].items():
+            for key, value in plan.scalars().items():
                 setattr(d, key, value)
             self.fused = d
-            self.fused_plan = plan["scalars"]
+            self.fused_plan = plan.scalars()
             self.fused_reason = ""
+            try:
+                self._tiling(1)
+                self._tiling(0)
+            except _fused.FusedUnsupported as exc:
+                self.fused, self.fused_reason = None, str(exc)
+
+    def _tiling(self, m):
+        """Device copy of the tiling used for m activation rows (0 = store sink); tilings
+        are made for m in {0, 1, 2, 4, 8} and shared by the row counts in between."""
+        import torch
+        bucket = 0 if m == 0 else next(v for v in (1, 2, 4, 8) if v >= m)
+        if bucket not in self._tilings:
+            host = self._plan.tiling(bucket)
+            rows = torch.from_numpy(host["tile_rows"]).to(self.device)
+            classes = torch.from_numpy(host["tile_class"]).to(self.device)
+            g = _hip_abi.GrfFusedTiling()
+            g.tile_rows, g.tile_class = rows.data_ptr(), classes.data_ptr()
+            for key, value in host["scalars"].items():
+                setattr(g, key, value)
+            self._tilings[bucket] = (g, rows, classes, dict(host["scalars"], lds=host["lds"]))
+            self.resident_bytes += rows.numel() * 4 + classes.numel()
+        return self._tilings[bucket]
 
     # ------------------------------------------------------------------ decode
     def _decode_blocks(self, blocks=None, *, check=True):
@@ -222,7 +260,8 @@ class HipContextTensor:
             return self._decode_blocks(check=check)[:self.n].reshape(self.shape)
         out = torch.empty(self.n, device=self.device, dtype=torch.uint16)
         self.error.zero_()
-        self._launch(self._lib.grf_bctx_fused_decode, ctypes.byref(self.fused), out.data_ptr(), self.error.data_ptr())
+        self._launch(self._lib.grf_bctx_fused_decode, ctypes.byref(self.fused), ctypes.byref(self._tiling(0)[0]),
+                     out.data_ptr(), self.error.data_ptr())
         self._check(check)
         return out.view(torch.bfloat16).reshape(self.shape)
 
@@ -247,7 +286,10 @@ class HipContextTensor:
         if bias is not None:
             bias = bias.to(device=self.device, dtype=torch.bfloat16).contiguous()
         self.error.zero_()
-        self._launch(self._lib.grf_bctx_gemv, ctypes.byref(self.fused), x2.data_ptr(), x2.stride(0), m,
+        if x2.stride(0) % 2 or x2.data_ptr() % 4:
+            x2 = x2.clone(memory_format=torch.contiguous_format)
+        self._launch(self._lib.grf_bctx_gemv, ctypes.byref(self.fused), ctypes.byref(self._tiling(m)[0]),
+                     x2.data_ptr(), x2.stride(0), m,
                      y.data_ptr(), y.stride(0), bias.data_ptr() if bias is not None else None,
                      self.error.data_ptr())
         self._check(check)

@@ -1,9 +1,11 @@
 // The fused decoder: one walker over a checkpointed segment whose decoded BF16
-// words go to a sink (FMA chain for the GEMV, LDS tile for the GEMM, global
-// store for decode()).  Because every sink is fed by the same walker, words
-// proven bit-exact through the store sink are the words the fused sinks consume.
+// words go to a sink (dot-product chain for the GEMV, LDS tile for the GEMM,
+// global store for decode()).  Because every sink is fed by the same walker,
+// words proven bit-exact through the store sink are the words the fused sinks
+// consume.
 //
-// Work decomposition (mode 0 frames, segment length S divides the row length K):
+// Work decomposition (packed-residual frames, segment length S divides the row
+// length K):
 //   * rows are grouped by row class; a workgroup ("tile") owns up to R rows of
 //     ONE class, so only that class's nc column contexts are live and their
 //     lookup tables fit in LDS;
@@ -14,14 +16,15 @@
 //     they are copied to LDS with 16-byte coalesced loads and each lane then
 //     consumes its own sub-range with byte-granular LDS reads;
 //   * the packed 6-bit residuals of a lane are 12 bytes per 16 symbols at a
-//     position known in advance; they are loaded straight into registers.
+//     position known in advance; they are loaded straight into registers, as are
+//     the 16 column classes of the same columns.
 //
 // Symbol lookup: slot>>shift indexes a u8 table giving the sparse index of the
 // symbol that owns the bucket's first slot; the 8-byte entries of that symbol
 // and of its successor are read together and one compare picks between them.
-// Entry: lo = start | (freq-1)<<16, hi = next_start (bits 0..16) | symbol<<21
-// | small<<31 where `small` marks freq < bucket size (then the successor may
-// still end inside the bucket and a short forward scan finishes the search).
+// Entry: low32 = start | (freq-1)<<16, high32 = symbol<<21 (the symbol's bits in
+// the fp32 image of the BF16 word).  A selected symbol with freq < bucket size
+// may still end before the slot; a short forward scan then finishes the search.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -31,107 +34,173 @@
 
 namespace grf {
 
-constexpr int kFusedThreads = 256;
+constexpr int kFusedMaxThreads = 1024;
 constexpr uint32_t kNoRow = 0xFFFFFFFFu;
-
-struct FusedLds {
-  uint8_t *lut;       // nc << lognb bytes
-  const uint2 *tab;   // (tabn + 1) * nc entries, index = sparse*nc + cc
-  float *xs;          // M * P * (S + 4) floats
-  uint8_t *cc8;       // P * S bytes: column class
-  uint8_t *stream;    // R * piece_cap bytes
-  float *part;        // R * P * M floats
-};
+constexpr uint32_t kXPad = 8;  // BF16 elements of padding per x segment in LDS (16 bytes)
 
 __host__ __device__ inline uint32_t align_up(uint32_t v, uint32_t a) { return (v + a - 1) / a * a; }
 
-// byte offsets of the LDS regions; shared by host (size) and device (carve)
+// Per column class the LDS holds one block: the sparse symbol table first (kTabCap
+// 8-byte entries), then the class's lookup bytes.  With the block base in a register
+// the table read needs no further address arithmetic and the lookup read folds the
+// constant table size into its offset field.
+constexpr uint32_t kTabCap = 257;  // up to 256 symbols + the entry a forward scan stops on
+constexpr uint32_t kTabBytes = kTabCap * 8;
+
+// byte offsets of the LDS regions; shared by host (size) and device (carve).
 struct FusedLdsLayout {
-  uint32_t lut, tab, xs, cc8, stream, part, total;
-  __host__ __device__ FusedLdsLayout(const grf_bctx_fused &f, uint32_t m) {
+  uint32_t blocks, block_pitch, stream, xs, part, total;
+  __host__ __device__ FusedLdsLayout(const grf_bctx_fused &f, const grf_fused_tiling &g, uint32_t m) {
     uint32_t at = 0;
-    lut = at;
-    at = align_up(at + (f.nc << f.lognb), 16);
-    tab = at;
-    at = align_up(at + (f.tabn + 1) * f.nc * 8, 16);
-    xs = at;
-    at = align_up(at + m * f.lanes_per_row * (f.seg_len + 4) * 4, 16);
-    cc8 = at;
-    at = align_up(at + f.lanes_per_row * f.seg_len, 16);
+    blocks = at;
+    block_pitch = kTabBytes + (1u << f.lognb);
+    at = align_up(at + f.nc * block_pitch, 16);
     stream = at;
-    at = align_up(at + f.rows_per_tile * f.piece_cap, 16);
+    at = align_up(at + g.rows_per_tile * g.piece_cap, 16);
+    xs = at;
+    at = align_up(at + m * g.lanes_per_row * (f.seg_len + kXPad) * 2, 16);
     part = at;
-    at = align_up(at + f.rows_per_tile * f.lanes_per_row * m * 4, 16);
+    at = align_up(at + g.rows_per_tile * f.segs_per_row * m * 4, 16);
     total = at;
   }
 };
 
-// One decode step of the main stream against LDS tables.
-// Returns the selected table entry's hi word (symbol<<21 among other bits).
-__device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, const uint8_t *lds_base,
-                                                 uint32_t lut_off, uint32_t tab_off, uint32_t cc, uint32_t shift,
-                                                 uint32_t lognb, uint32_t lognc) {
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+typedef uint32_t v2u32 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) v2u32 lds_v2u32;
+
+// LDS accesses by absolute byte offset (dynamic LDS starts at address 0 here:
+// the kernels declare no static LDS)
+__device__ __forceinline__ uint8_t lds_load_u8(uint32_t off) { return *reinterpret_cast<lds_u8 *>(off); }
+
+struct FusedParams {  // uniform values the step needs, kept in scalar registers
+  uint32_t shift, block_pitch, small_limit;
+};
+
+// Slow twin of the step for the rare case that the selected symbol is smaller than a
+// bucket: scan forward from table address `ta` to the symbol that holds the slot, then
+// update and refill in plain C.  Returns the entry's high word.
+__device__ __forceinline__ uint32_t fused_symbol_scan(uint32_t &state, uint32_t &ip, uint32_t ta, uint32_t byte0,
+                                                      uint32_t byte1) {
   const uint32_t slot = state & 0xFFFFu;
-  const uint32_t la = (cc << lognb) | (slot >> shift);
-  uint32_t idx = lds_base[lut_off + la];
-  const uint2 *tab = reinterpret_cast<const uint2 *>(lds_base + tab_off);
-  uint32_t ta = (idx << lognc) | cc;
-  const uint2 e0 = tab[ta];
-  const uint2 e1 = tab[ta + (1u << lognc)];
-  const bool take1 = slot >= (e0.y & 0x1FFFFu);
-  uint32_t lo = take1 ? e1.x : e0.x;
-  uint32_t hi = take1 ? e1.y : e0.y;
-  if (__builtin_expect((int32_t)hi < 0, 0)) {  // small symbol: successor may also end before slot
-    ta += take1 ? (1u << lognc) : 0u;
-    while (slot >= (hi & 0x1FFFFu)) {
-      ta += 1u << lognc;
-      const uint2 e = tab[ta];
-      lo = e.x;
-      hi = e.y;
-    }
+  v2u32 e = *reinterpret_cast<lds_v2u32 *>(ta);
+  while ((slot - (e.x & 0xFFFFu)) > (e.x >> 16)) {
+    ta += 8;
+    e = *reinterpret_cast<lds_v2u32 *>(ta);
   }
   const uint32_t h = state >> 16;
-  uint32_t x = (lo >> 16) * h + (slot + h - (lo & 0xFFFFu));
-  // refill: at most two bytes; both are read unconditionally (the region has slack)
-  uint16_t two;
-  __builtin_memcpy(&two, lds_base + ip, 2);
-  const uint32_t b0 = two & 0xFFu, b1 = two >> 8;
-  const bool n1 = x < kLow;
-  x = n1 ? ((x << 8) | b0) : x;
-  ip += n1;
-  const bool n2 = x < kLow;
-  x = n2 ? ((x << 8) | b1) : x;
-  ip += n2;
+  uint32_t x = (e.x >> 16) * h + (slot + h - (e.x & 0xFFFFu));
+  if (x < kLow) {
+    x = (x << 8) | byte0;
+    ++ip;
+    if (x < kLow) {
+      x = (x << 8) | byte1;
+      ++ip;
+    }
+  }
   state = x;
+  return e.y;
+}
+
+// One decode step of the main stream against LDS tables.  Returns the fp32 image
+// of the symbol's bits (symbol << 21).
+__device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, uint32_t cc, const FusedParams &q) {
+  // the two possible refill bytes, fetched ahead of need with byte reads: an unaligned
+  // 16-bit LDS read stalls the LDS pipeline for tens of cycles on this hardware
+  uint32_t byte0, byte1;
+#if defined(__HIP_DEVICE_COMPILE__)
+  // issued as raw instructions so that no mask is applied to the zero-extended result; the
+  // compiler does not count these two LDS reads, the block below waits for them itself
+  asm volatile("ds_read_u8 %0, %2\n\tds_read_u8 %1, %2 offset:1" : "=&v"(byte0), "=&v"(byte1) : "v"(ip));
+#else
+  byte0 = byte1 = 0;
+#endif
+  const uint32_t block = __umul24(cc, q.block_pitch);
+  const uint32_t bucket = (state & 0xFFFFu) >> q.shift;
+  const uint32_t idx = lds_load_u8(block + bucket + kTabBytes);
+  const uint32_t ta = (idx << 3) + block;
+  const v2u32 e0 = *reinterpret_cast<lds_v2u32 *>(ta);
+  const v2u32 e1 = *reinterpret_cast<lds_v2u32 *>(ta + 8);
+  const uint32_t state_in = state, ip_in = ip;
+  uint32_t lo, hi, x, ipn;
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t t, a;
+  // Pick entry 0 or 1 (slot past entry 0's range), x = (freq-1)*h + (slot + h - start)
+  // with h = state>>16, then up to two refills (x << 8) | byte while x < 2^23, ip counting
+  // the bytes taken.  Operand halves are addressed with SDWA selects instead of shifts and
+  // masks; v_perm builds (x << 8) | byte from the byte register's low byte only.  gfx950
+  // needs two wait states between a VALU write of VCC and a VALU read of it.
+  asm volatile(
+      "s_waitcnt lgkmcnt(0)\n\t"
+      "v_sub_u32_sdwa %[t], %[st], %[e0lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_0\n\t"
+      "v_cmp_gt_u32_sdwa vcc, %[t], %[e0lo] src0_sel:DWORD src1_sel:WORD_1\n\t"
+      "v_add_u32_sdwa %[a], %[st], %[st] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
+      "s_nop 0\n\t"
+      "v_cndmask_b32 %[lo], %[e0lo], %[e1lo], vcc\n\t"
+      "v_cndmask_b32 %[hi], %[e0hi], %[e1hi], vcc\n\t"
+      "v_mul_u32_u24_sdwa %[x], %[lo], %[st] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_1 src1_sel:WORD_1\n\t"
+      "v_sub_u32_sdwa %[a], %[a], %[lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_0\n\t"
+      "v_add_u32 %[x], %[x], %[a]\n\t"
+      "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
+      "v_perm_b32 %[t], %[x], %[b0], %[sel]\n\t"
+      "s_nop 0\n\t"
+      "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
+      "v_addc_co_u32 %[ipo], vcc, 0, %[ipi], vcc\n\t"
+      "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
+      "v_perm_b32 %[t], %[x], %[b1], %[sel]\n\t"
+      "s_nop 0\n\t"
+      "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
+      "v_addc_co_u32 %[ipo], vcc, 0, %[ipo], vcc\n\t"
+      : [x] "=&v"(x), [t] "=&v"(t), [a] "=&v"(a), [lo] "=&v"(lo), [hi] "=&v"(hi), [ipo] "=&v"(ipn)
+      : [st] "v"(state), [e0lo] "v"(e0.x), [e0hi] "v"(e0.y), [e1lo] "v"(e1.x), [e1hi] "v"(e1.y),
+        [b0] "v"(byte0), [b1] "v"(byte1), [sel] "s"(0x06050400u), [ipi] "v"(ip)
+      : "vcc");
+#else
+  lo = e0.x + e1.x + byte0 + byte1;  // host pass only parses this
+  hi = e0.y + e1.y;
+  x = state;
+  ipn = ip;
+#endif
+  state = x;
+  ip = ipn;
+  if (__builtin_expect((lo >> 16) < q.small_limit, 0)) {
+    // freq < bucket size: the slot may lie beyond the picked entry.  Redo the step from the
+    // saved state with a forward scan starting at the picked entry.
+    state = state_in;
+    ip = ip_in;
+    const bool took1 = ((state_in & 0xFFFFu) - (e0.x & 0xFFFFu)) > (e0.x >> 16);
+    hi = fused_symbol_scan(state, ip, ta + (took1 ? 8u : 0u), byte0 & 0xFFu, byte1 & 0xFFu);
+  }
   return hi;
 }
 
 // Sixteen packed 6-bit residuals (12 bytes, MSB first) -> field k, k compile-time.
 struct Raw6x16 {
   uint32_t w0, w1, w2;  // big-endian dwords
-  __device__ __forceinline__ void load(const uint8_t *p) {
-    const uint32_t *q = reinterpret_cast<const uint32_t *>(p);
-    w0 = __builtin_bswap32(q[0]);
-    w1 = __builtin_bswap32(q[1]);
-    w2 = __builtin_bswap32(q[2]);
+  __device__ __forceinline__ void set(uint32_t a, uint32_t b, uint32_t c) {
+    w0 = __builtin_bswap32(a);
+    w1 = __builtin_bswap32(b);
+    w2 = __builtin_bswap32(c);
   }
   template <int K>
   __device__ __forceinline__ uint32_t field() const {
-    constexpr int bit = K * 6;          // position from the MSB of the 96-bit group
+    constexpr int bit = K * 6;  // position from the MSB of the 96-bit group
     constexpr int word = bit / 32, off = bit % 32;
     const uint32_t a = word == 0 ? w0 : (word == 1 ? w1 : w2);
     if constexpr (off + 6 <= 32) {
-      return (a >> (32 - 6 - off)) & 63u;
+      return __builtin_amdgcn_ubfe(a, 32 - 6 - off, 6);
     } else {
       const uint32_t b = word == 0 ? w1 : w2;
-      return (uint32_t)((((uint64_t)a << 32 | b) >> (64 - 6 - off)) & 63u);
+      return __builtin_amdgcn_ubfe(__builtin_amdgcn_alignbit(a, b, 64 - 6 - off), 0, 6);
     }
   }
 };
 
-// fp32 bit pattern of the BF16 word (word << 16) from the entry's hi field and the residual
+// fp32 image of the BF16 word: symbol bits | mantissa low 5 bits << 16 | sign << 31.
+// r6 * (1 + 2^10) puts the five mantissa bits at 0..4 and the sign at 15 (a 24-bit
+// multiply); the mask drops the copies that land elsewhere.
 __device__ __forceinline__ uint32_t fused_value_bits(uint32_t hi, uint32_t r6) {
-  return (hi & 0x7FE00000u) | ((r6 & 31u) << 16) | ((r6 >> 5) << 31);
+  return (((r6 * 0x401u) & 0x801Fu) << 16) | hi;
 }
 
 }  // namespace grf

@@ -453,6 +453,18 @@ int bcx_checkpoint(const uint8_t *stream, size_t stream_bytes, uint64_t n, uint3
       5, 6);
 }
 
+// 10-bit main symbols + 6-bit residuals -> BF16 words (no reference counterpart:
+// the reference recombines in numpy, GCR/bitexact_context_codec.py:426).
+int grf_bctx_join(const uint16_t *main_sym, const uint16_t *res_sym, uint64_t n, uint16_t *out) {
+  if (!main_sym || !res_sym || !out) return 1;
+  for (uint64_t i = 0; i < n; ++i) {
+    const uint32_t m = main_sym[i], r = res_sym[i];
+    if (m > 1023u || r > 63u) return 2;
+    out[i] = (uint16_t)((m << 5) | (r & 31u) | ((r >> 5) << 15));
+  }
+  return 0;
+}
+
 // ---------------------------------------------------------------- PPCX
 int p_encode(const uint16_t *v, const uint16_t *cx, uint64_t n, uint32_t nc, uint32_t vocab, uint32_t **freqp,
              uint8_t **streamp, size_t *sn) {

@@ -58,6 +58,9 @@ int bcx_checkpoint(const uint8_t *stream, size_t stream_bytes, uint64_t n, uint3
                    const uint8_t *rc, const uint8_t *cc, uint32_t nr, uint32_t nc, uint32_t kind,
                    const uint16_t *resctx, const uint32_t *freq, uint32_t stride, uint32_t *states,
                    uint32_t *offsets, uint16_t *out);
+/* Symbol pair -> BF16 word, the inverse of the split at GCR/bitexact_context_ans.cpp:9-12
+ * (the reference does this step in numpy, GCR/bitexact_context_codec.py:426). 2 = symbol out of range. */
+int grf_bctx_join(const uint16_t *main_sym, const uint16_t *res_sym, uint64_t n, uint16_t *out);
 /* GCR/bitexact_predictive_ans.cpp:10-12  generic context coder of the predictive frames */
 int p_encode(const uint16_t *v, const uint16_t *cx, uint64_t n, uint32_t nc, uint32_t vocab, uint32_t **freq,
              uint8_t **stream, size_t *stream_n);
@@ -151,18 +154,16 @@ int grf_ppcx_decode(const grf_ppcx_frame *frame, const uint16_t *reference, uint
 int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *coeff, uint16_t *out,
                     uint32_t rows, uint32_t cols, int32_t *error, void *hip_stream);
 
-/* A mode-0 BCTX frame prepared for the fused kernels.  Segments have a length that
- * divides the row length, rows are grouped by row class into tiles, and the
- * per-class lookup tables are laid out for LDS:
+/* A BCTX frame prepared for the fused kernels: main rANS stream as in the frame,
+ * residuals in the packed 6-bit form, segments of a length that divides the row
+ * length, and per-row-class lookup tables laid out for LDS:
  *   seg_state / seg_offset  u32 [rows*segs_per_row + 1]; the extra last entry is
  *                           (2^23, main_n_bytes)
- *   tile_rows   u32 [n_tiles*rows_per_tile]  row of each slot, 0xFFFFFFFF = empty
- *   tile_class  u8  [n_tiles]                row class shared by the tile's rows
  *   lut         u8  [nr][nc << lognb]        lognb = 16 - shift; sparse index of the
  *                                            symbol owning the bucket's first slot
- *   tab         u64 [nr][(tabn+1)*nc]        entry(sparse, cc) at sparse*nc + cc:
- *                 low32 = start | (freq-1)<<16
- *                 high32 = next_start (bits 0..16) | symbol<<21 | (freq < 2^shift)<<31
+ *   tab         u64 [nr][nc][tabn+1]         entry(cc, sparse): low32 = start |
+ *                                            (freq-1)<<16, high32 = symbol<<21;
+ *                                            unused entries: start 0, freq 65536
  *   col_class   u8  [cols]
  * main_bytes must be readable for 16 bytes past main_n_bytes. */
 typedef struct grf_bctx_fused {
@@ -170,19 +171,30 @@ typedef struct grf_bctx_fused {
   const uint8_t *raw6;
   const uint32_t *seg_state;
   const uint32_t *seg_offset;
-  const uint32_t *tile_rows;
-  const uint8_t *tile_class;
   const uint8_t *lut;
   const uint64_t *tab;
   const uint8_t *col_class;
   uint32_t main_n_bytes;
   uint32_t rows, cols;
-  uint32_t nr, nc, lognc;
+  uint32_t nr, nc;
   uint32_t seg_len, segs_per_row;
-  uint32_t lanes_per_row, rows_per_tile, n_slabs, n_tiles;
   uint32_t shift, lognb, tabn;
-  uint32_t piece_cap; /* LDS bytes reserved per row piece (multiple of 16) */
 } grf_bctx_fused;
+
+/* How a launch cuts the frame into workgroups.  A tile is up to rows_per_tile rows of
+ * one row class; lane (r, p) of the workgroup walks segment b*lanes_per_row + p of the
+ * tile's row r in slab b.  threads >= rows_per_tile*lanes_per_row, a multiple of 64,
+ * at most 1024.
+ *   tile_rows   u32 [n_tiles*rows_per_tile]  row of each slot, 0xFFFFFFFF = empty
+ *   tile_class  u8  [n_tiles]                row class shared by the tile's rows
+ *   piece_cap   LDS bytes reserved per row piece of one slab (multiple of 16) */
+typedef struct grf_fused_tiling {
+  const uint32_t *tile_rows;
+  const uint8_t *tile_class;
+  uint32_t threads;
+  uint32_t lanes_per_row, rows_per_tile, n_slabs, n_tiles;
+  uint32_t piece_cap;
+} grf_fused_tiling;
 
 /* Fused decode-GEMV, the slot the reference leaves for "a backend with a fused GEMM"
  * behind the CudaContextTensor contract (GCR/bitexact_context_serving.py:3-5; it replaces
@@ -190,14 +202,16 @@ typedef struct grf_bctx_fused {
  * W[n][k] + bias[n]) for 1 <= m_rows <= 8, fp32 accumulation in an order that does not
  * depend on m_rows (the M-invariance contract of GS/miv_gemv.py:10-29).
  * x: BF16 [m_rows][ldx], y: BF16 [m_rows][ldy], bias: BF16 [rows] or NULL. */
-int grf_bctx_gemv(const grf_bctx_fused *frame, const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint16_t *y,
-                  uint32_t ldy, const uint16_t *bias, int32_t *error, void *hip_stream);
+int grf_bctx_gemv(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, const uint16_t *x, uint32_t ldx,
+                  uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
+                  void *hip_stream);
 
 /* Same walker with a store sink: out[rows*cols] BF16 words (decode() for fused frames). */
-int grf_bctx_fused_decode(const grf_bctx_fused *frame, uint16_t *out, int32_t *error, void *hip_stream);
+int grf_bctx_fused_decode(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint16_t *out,
+                          int32_t *error, void *hip_stream);
 
-/* LDS bytes a launch on this frame needs for the given m_rows (0 for the store sink). */
-uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, uint32_t m_rows);
+/* LDS bytes a launch needs for the given m_rows (0 for the store sink). */
+uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint32_t m_rows);
 
 const char *grf_last_error(void);
 int grf_abi_version(void);
