@@ -23,7 +23,7 @@ class FusedUnsupported(ValueError):
 def choose_segment(cols, preferred=None):
     """Largest supported segment length that divides the row length."""
     order = [preferred] if preferred else []
-    order += [128, 64, 256, 32, 16]
+    order += [64, 128, 32, 256, 16]
     for s in order:
         if s and s % 16 == 0 and cols % s == 0:
             return s
@@ -41,7 +41,7 @@ def choose_shift(nc, budget=LUT_BUDGET):
 def sparse_tables(freq, nr, nc, shift):
     """Per row class: u8 lookup [nc << lognb] and u64 entries [nc][tabn+1].
 
-    Entry(column class c, sparse i): low32 = start | (freq-1) << 16, high32 = symbol << 21.
+    Entry(column class c, sparse i): low32 = start | (freq-1) << 16, high32 = symbol << 5.
     Unused entries are (start 0, freq 65536): a forward scan always stops on them."""
     nz = freq > 0
     tabn = int(nz.sum(axis=1).max())
@@ -63,7 +63,7 @@ def sparse_tables(freq, nr, nc, shift):
             fs = f[syms]
             starts = np.concatenate(([0], np.cumsum(fs)[:-1]))
             lo = starts | ((fs - 1) << 16)
-            hi = syms << 21
+            hi = syms << 5
             tab[rho, c, :syms.size] = (lo.astype(np.uint64) | (hi.astype(np.uint64) << np.uint64(32)))
             lut[rho, c] = (np.searchsorted(starts, first_slots, side="right") - 1).astype(np.uint8)
     return lut.reshape(nr, nc * nb), tab.reshape(nr, nc * (tabn + 1)), tabn
@@ -101,14 +101,21 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
     The walk is a chain of dependent steps per lane, so time ~ steps per lane x rounds
     of workgroups, at the speed the resident wave count allows.  The model multiplies
     lane efficiency (idle lanes in the last slab and in a partly filled workgroup), tile
-    fill, how evenly the tiles fill the machine, and a penalty below 16 waves per CU."""
+    fill, how evenly the tiles fill the machine, and a penalty below 24 waves per CU
+    (measured: the dependent LDS round trips of a step need that many waves to overlap)."""
     best = None
     total_rows = sum(int(c) for c in class_rows)
-    for threads in (1024, 512, 256):
-        for p in range(1, min(spr, threads) + 1):
+    forced = os.environ.get("GEOREFINE_FUSED_TILING")  # "threads,lanes_per_row": experiments only
+    thread_choices = range(1024, 0, -64)
+    lane_choices = None
+    if forced:
+        t_, p_ = (int(v) for v in forced.split(","))
+        thread_choices, lane_choices = [t_], [min(p_, spr)]
+    for threads in thread_choices:
+        for p in (lane_choices or range(1, min(spr, threads) + 1)):
             r = threads // p
             n_slabs = -(-spr // p)
-            if p > 1 and -(-spr // (p - 1)) == n_slabs:
+            if not forced and p > 1 and -(-spr // (p - 1)) == n_slabs:
                 continue  # a narrower slab of the same count wastes fewer lanes; it was scored already
             lanes = p * r
             lane_eff = spr / (n_slabs * p) * (lanes / threads)
@@ -118,12 +125,13 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
             lds = lds_fn(p, r, cap)
             if lds > MAX_LDS:
                 continue
-            per_cu = max(1, min(2048 // threads, MAX_LDS // lds))
+            # the kernels use up to 72 vector registers: 7 waves per SIMD, 28 per CU
+            per_cu = max(1, min(28 // (threads // 64), MAX_LDS // lds))
             waves = per_cu * threads // 64
             slots = cus * per_cu
             rounds = -(-tiles // slots)
             quant = tiles / (rounds * slots)
-            score = lane_eff * fill * quant * min(1.0, waves / 16)
+            score = lane_eff * fill * quant * min(1.0, waves / 24)
             if best is None or score > best[0] + 1e-9:
                 best = (score, threads, p, r, n_slabs, tiles, cap, lds)
     if best is None:

@@ -22,8 +22,8 @@
 // Symbol lookup: slot>>shift indexes a u8 table giving the sparse index of the
 // symbol that owns the bucket's first slot; the 8-byte entries of that symbol
 // and of its successor are read together and one compare picks between them.
-// Entry: low32 = start | (freq-1)<<16, high32 = symbol<<21 (the symbol's bits in
-// the fp32 image of the BF16 word).  A selected symbol with freq < bucket size
+// Entry: low32 = start | (freq-1)<<16, high32 = symbol<<5 (the symbol's bits in
+// the BF16 word).  A selected symbol with freq < bucket size
 // may still end before the slot; a short forward scan then finishes the search.
 #pragma once
 #include <hip/hip_runtime.h>
@@ -66,6 +66,7 @@ struct FusedLdsLayout {
 };
 
 typedef __attribute__((address_space(3))) uint8_t lds_u8;
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
 typedef uint32_t v2u32 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) v2u32 lds_v2u32;
 
@@ -102,19 +103,15 @@ __device__ __forceinline__ uint32_t fused_symbol_scan(uint32_t &state, uint32_t 
   return e.y;
 }
 
-// One decode step of the main stream against LDS tables.  Returns the fp32 image
-// of the symbol's bits (symbol << 21).
+// One decode step of the main stream against LDS tables.  Returns the image
+// of the symbol's bits in the BF16 word (symbol << 5).
 __device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, uint32_t cc, const FusedParams &q) {
-  // the two possible refill bytes, fetched ahead of need with byte reads: an unaligned
-  // 16-bit LDS read stalls the LDS pipeline for tens of cycles on this hardware
-  uint32_t byte0, byte1;
-#if defined(__HIP_DEVICE_COMPILE__)
-  // issued as raw instructions so that no mask is applied to the zero-extended result; the
-  // compiler does not count these two LDS reads, the block below waits for them itself
-  asm volatile("ds_read_u8 %0, %2\n\tds_read_u8 %1, %2 offset:1" : "=&v"(byte0), "=&v"(byte1) : "v"(ip));
-#else
-  byte0 = byte1 = 0;
-#endif
+  // The two possible refill bytes, fetched ahead of need: the aligned dword that holds
+  // byte `ip` and the dword after it, shifted so that the bytes sit in bits 0..15.
+  // (An unaligned 16-bit LDS read stalls the LDS pipeline for tens of cycles on this
+  // hardware, and two byte reads cost two bank-conflicted accesses.)
+  const v2u32 dw = {*reinterpret_cast<lds_u32 *>(ip & ~3u), *reinterpret_cast<lds_u32 *>((ip & ~3u) + 4)};
+  const uint32_t bytes = __builtin_amdgcn_alignbyte(dw.y, dw.x, ip);
   const uint32_t block = __umul24(cc, q.block_pitch);
   const uint32_t bucket = (state & 0xFFFFu) >> q.shift;
   const uint32_t idx = lds_load_u8(block + bucket + kTabBytes);
@@ -131,7 +128,6 @@ __device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, 
   // masks; v_perm builds (x << 8) | byte from the byte register's low byte only.  gfx950
   // needs two wait states between a VALU write of VCC and a VALU read of it.
   asm volatile(
-      "s_waitcnt lgkmcnt(0)\n\t"
       "v_sub_u32_sdwa %[t], %[st], %[e0lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_0\n\t"
       "v_cmp_gt_u32_sdwa vcc, %[t], %[e0lo] src0_sel:DWORD src1_sel:WORD_1\n\t"
       "v_add_u32_sdwa %[a], %[st], %[st] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
@@ -142,21 +138,21 @@ __device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, 
       "v_sub_u32_sdwa %[a], %[a], %[lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_0\n\t"
       "v_add_u32 %[x], %[x], %[a]\n\t"
       "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
-      "v_perm_b32 %[t], %[x], %[b0], %[sel]\n\t"
+      "v_perm_b32 %[t], %[x], %[b], %[sel0]\n\t"
       "s_nop 0\n\t"
       "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
       "v_addc_co_u32 %[ipo], vcc, 0, %[ipi], vcc\n\t"
       "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
-      "v_perm_b32 %[t], %[x], %[b1], %[sel]\n\t"
+      "v_perm_b32 %[t], %[x], %[b], %[sel1]\n\t"
       "s_nop 0\n\t"
       "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
       "v_addc_co_u32 %[ipo], vcc, 0, %[ipo], vcc\n\t"
       : [x] "=&v"(x), [t] "=&v"(t), [a] "=&v"(a), [lo] "=&v"(lo), [hi] "=&v"(hi), [ipo] "=&v"(ipn)
       : [st] "v"(state), [e0lo] "v"(e0.x), [e0hi] "v"(e0.y), [e1lo] "v"(e1.x), [e1hi] "v"(e1.y),
-        [b0] "v"(byte0), [b1] "v"(byte1), [sel] "s"(0x06050400u), [ipi] "v"(ip)
+        [b] "v"(bytes), [sel0] "s"(0x06050400u), [sel1] "s"(0x06050401u), [ipi] "v"(ip)
       : "vcc");
 #else
-  lo = e0.x + e1.x + byte0 + byte1;  // host pass only parses this
+  lo = e0.x + e1.x + bytes;  // host pass only parses this
   hi = e0.y + e1.y;
   x = state;
   ipn = ip;
@@ -169,7 +165,7 @@ __device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, 
     state = state_in;
     ip = ip_in;
     const bool took1 = ((state_in & 0xFFFFu) - (e0.x & 0xFFFFu)) > (e0.x >> 16);
-    hi = fused_symbol_scan(state, ip, ta + (took1 ? 8u : 0u), byte0 & 0xFFu, byte1 & 0xFFu);
+    hi = fused_symbol_scan(state, ip, ta + (took1 ? 8u : 0u), bytes & 0xFFu, (bytes >> 8) & 0xFFu);
   }
   return hi;
 }
@@ -196,11 +192,11 @@ struct Raw6x16 {
   }
 };
 
-// fp32 image of the BF16 word: symbol bits | mantissa low 5 bits << 16 | sign << 31.
-// r6 * (1 + 2^10) puts the five mantissa bits at 0..4 and the sign at 15 (a 24-bit
-// multiply); the mask drops the copies that land elsewhere.
-__device__ __forceinline__ uint32_t fused_value_bits(uint32_t hi, uint32_t r6) {
-  return (((r6 * 0x401u) & 0x801Fu) << 16) | hi;
+// BF16 word in bits 0..15 (bits above are unspecified): symbol bits | mantissa low 5 bits
+// | sign << 15.  r6 * (1 + 2^10) puts the five mantissa bits at 0..4 and the sign at 15
+// (a 24-bit multiply); the mask drops the copies that land elsewhere.
+__device__ __forceinline__ uint32_t fused_word_bits(uint32_t hi, uint32_t r6) {
+  return ((r6 * 0x401u) & 0x801Fu) | hi;
 }
 
 }  // namespace grf

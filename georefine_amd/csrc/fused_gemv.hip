@@ -127,14 +127,14 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   {                                                                       \
     const uint32_t cc = __builtin_amdgcn_ubfe(cw[(k) / 4], 8 * ((k) % 4), 8); \
     const uint32_t hi = grf::fused_symbol(state, ip, cc, q);              \
-    bits[k] = grf::fused_value_bits(hi, rr.field<k>());                   \
+    bits[k] = grf::fused_word_bits(hi, rr.field<k>());                   \
   }
         GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
         GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
 #undef GRF_STEP
         uint32_t pair[8];  // BF16 words k (low half) and k+1 (high half)
 #pragma unroll
-        for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x07060302u);
+        for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
         if (STORE) {
           uint4 *dst = reinterpret_cast<uint4 *>(out + elem0 + t);
           dst[0] = make_uint4(pair[0], pair[1], pair[2], pair[3]);
