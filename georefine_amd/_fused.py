@@ -82,6 +82,16 @@ def lds_bytes(nc, lognb, tabn, m, p, s, r, piece_cap, spr):
     return total
 
 
+def lds_bytes_gemm(nc, lognb, m16, p, r, piece_cap):
+    a16 = lambda v: (v + 15) // 16 * 16
+    pitch = p * 32 + 8
+    total = a16(nc * (TAB_CAP * 8 + (1 << lognb)))
+    total = a16(total + r * piece_cap)
+    total = a16(total + a16(r) * pitch)
+    total = a16(total + m16 * pitch)
+    return total
+
+
 def piece_capacity(offsets, rows, spr, p):
     """LDS bytes one row piece may need: the longest (16-byte aligned start .. end) span
     over every (row, slab), plus two bytes the refill reads ahead, rounded to 16."""
@@ -95,7 +105,7 @@ def piece_capacity(offsets, rows, spr, p):
     return (longest + 2 + 15) // 16 * 16
 
 
-def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
+def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
     """(threads T, lanes_per_row P, rows_per_tile R, ...): best modelled throughput.
 
     The walk is a chain of dependent steps per lane, so time ~ steps per lane x rounds
@@ -114,9 +124,18 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
     for threads in thread_choices:
         for p in (lane_choices or range(1, min(spr, threads) + 1)):
             r = threads // p
+            if gemm:  # see below: at most waves/2 column blocks of 16 rows
+                r = min(r, (threads // 128) * 16)
+                if r == 0:
+                    continue
             n_slabs = -(-spr // p)
             if not forced and p > 1 and -(-spr // (p - 1)) == n_slabs:
                 continue  # a narrower slab of the same count wastes fewer lanes; it was scored already
+            if gemm:
+                # every 16-row column block needs a wave, and a wave owns at most 4 of the 8 row tiles
+                waves_wg, col_blocks = threads // 64, -(-r // 16)
+                if col_blocks > waves_wg or -(-8 // (waves_wg // col_blocks)) > 4:
+                    continue
             lanes = p * r
             lane_eff = spr / (n_slabs * p) * (lanes / threads)
             tiles = sum(-(-int(cnt) // r) for cnt in class_rows if cnt)
@@ -191,6 +210,18 @@ class FramePlan:
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
             self.spr, self.class_rows, self._cap,
             lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_, self.spr))
+        tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
+        assert len(tile_class) == n_tiles
+        return dict(tile_rows=tile_rows, tile_class=tile_class,
+                    scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
+                                 n_tiles=n_tiles, piece_cap=cap), lds=lds)
+
+    def gemm_tiling(self):
+        """The one tiling every fused GEMM launch uses, whatever its row count: the order in
+        which an output element accumulates follows the tiling, so it must not change with M."""
+        threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
+            self.spr, self.class_rows, self._cap,
+            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, 128, p_, r_, cap_), gemm=True)
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,

@@ -39,7 +39,7 @@ class GrfFusedTiling(ctypes.Structure):
 
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
-                  "grf_bctx_fused_decode", "grf_bctx_fused_lds_bytes", "grf_last_error", "grf_abi_version")
+                  "grf_bctx_fused_decode", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes", "grf_last_error", "grf_abi_version")
 
 
 def declare(L):
@@ -53,6 +53,10 @@ def declare(L):
     tiling = ctypes.POINTER(GrfFusedTiling)
     L.grf_bctx_gemv.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, u32, u32, vp, u32, vp, vp, vp]
     L.grf_bctx_gemv.restype = i
+    L.grf_bctx_gemm.argtypes = L.grf_bctx_gemv.argtypes
+    L.grf_bctx_gemm.restype = i
+    L.grf_bctx_gemm_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, u32]
+    L.grf_bctx_gemm_lds_bytes.restype = u32
     L.grf_bctx_fused_decode.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, vp, vp]
     L.grf_bctx_fused_decode.restype = i
     L.grf_bctx_fused_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, u32]

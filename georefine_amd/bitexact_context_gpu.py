@@ -265,35 +265,75 @@ class HipContextTensor:
         self._check(check)
         return out.view(torch.bfloat16).reshape(self.shape)
 
-    def linear(self, x, bias=None, *, check=False):
-        """y = x @ W.T (+ bias) with W decoded inside the kernel; x is BF16 [..., K].
-
-        Up to 8 activation rows run the fused decode-GEMV; other cases decode and call
-        the dense matmul.  ``check=True`` reads the error word back (a host sync)."""
+    def _gemm_tiling(self):
         import torch
-        import torch.nn.functional as F
+        if "gemm" not in self._tilings:
+            host = self._plan.gemm_tiling()
+            rows = torch.from_numpy(host["tile_rows"]).to(self.device)
+            classes = torch.from_numpy(host["tile_class"]).to(self.device)
+            g = _hip_abi.GrfFusedTiling()
+            g.tile_rows, g.tile_class = rows.data_ptr(), classes.data_ptr()
+            for key, value in host["scalars"].items():
+                setattr(g, key, value)
+            self._tilings["gemm"] = (g, rows, classes, dict(host["scalars"], lds=host["lds"]))
+            self.resident_bytes += rows.numel() * 4 + classes.numel()
+        return self._tilings["gemm"]
+
+    def _prepare_activations(self, x, bias, align):
+        import torch
         if x.dtype != torch.bfloat16 or x.shape[-1] != self.shape[1]:
             raise ValueError("activation must be bfloat16 with the weight's input width")
-        lead = x.shape[:-1]
-        x2 = x.reshape(-1, self.shape[1])
-        m = x2.shape[0]
-        if self.fused is None or not 1 <= m <= 8:
-            return F.linear(x, self.decode(check=check), bias)
-        if x2.stride(-1) != 1:
-            x2 = x2.contiguous()
-        x2 = x2.to(self.device)
-        y = torch.empty((m, self.shape[0]), device=self.device, dtype=torch.bfloat16)
+        x2 = x.reshape(-1, self.shape[1]).to(self.device)
+        if x2.stride(-1) != 1 or x2.stride(0) % align or x2.data_ptr() % (2 * align):
+            x2 = x2.clone(memory_format=torch.contiguous_format)
         if bias is not None:
             bias = bias.to(device=self.device, dtype=torch.bfloat16).contiguous()
-        self.error.zero_()
-        if x2.stride(0) % 2 or x2.data_ptr() % 4:
-            x2 = x2.clone(memory_format=torch.contiguous_format)
-        self._launch(self._lib.grf_bctx_gemv, ctypes.byref(self.fused), ctypes.byref(self._tiling(m)[0]),
-                     x2.data_ptr(), x2.stride(0), m,
-                     y.data_ptr(), y.stride(0), bias.data_ptr() if bias is not None else None,
-                     self.error.data_ptr())
-        self._check(check)
+        y = torch.empty((x2.shape[0], self.shape[0]), device=self.device, dtype=torch.bfloat16)
+        return x2, bias, y
+
+    def _fused_call(self, fn, tiling, x, bias, check):
+        lead = x.shape[:-1]
+        x2, bias, y = self._prepare_activations(x, bias, 4)
+        if x2.shape[0]:
+            self.error.zero_()
+            self._launch(fn, ctypes.byref(self.fused), ctypes.byref(tiling), x2.data_ptr(), x2.stride(0),
+                         x2.shape[0], y.data_ptr(), y.stride(0), bias.data_ptr() if bias is not None else None,
+                         self.error.data_ptr())
+            self._check(check)
         return y.reshape(*lead, self.shape[0])
+
+    def gemv(self, x, bias=None, *, check=False):
+        """Fused decode-GEMV (vector ALUs) for 1..8 activation rows; the result of a row does
+        not depend on how many rows the call carries."""
+        if self.fused is None:
+            raise base.CodecError("frame is not eligible for the fused kernels: " + self.fused_reason)
+        m = math.prod(x.shape[:-1])
+        if not 1 <= m <= 8:
+            raise ValueError("gemv takes 1..8 activation rows")
+        return self._fused_call(self._lib.grf_bctx_gemv, self._tiling(m)[0], x, bias, check)
+
+    def gemm(self, x, bias=None, *, check=False):
+        """Fused decode-GEMM (matrix cores) for any number of activation rows, batch-invariant:
+        a row's output bits are the same whatever else is in the batch."""
+        if self.fused is None:
+            raise base.CodecError("frame is not eligible for the fused kernels: " + self.fused_reason)
+        return self._fused_call(self._lib.grf_bctx_gemm, self._gemm_tiling()[0], x, bias, check)
+
+    def linear(self, x, bias=None, *, check=False, batch_invariant=False):
+        """y = x @ W.T (+ bias) with W decoded inside the kernel; x is BF16 [..., K].
+
+        Up to 8 activation rows run the fused decode-GEMV, more run the fused decode-GEMM;
+        ``batch_invariant=True`` sends every row count through the GEMM so that a row's
+        output never depends on the batch it arrives in.  Frames the fused kernels cannot
+        take are decoded on the device and multiplied densely.  ``check=True`` reads the
+        error word back (a host sync)."""
+        import torch.nn.functional as F
+        if self.fused is None:
+            return F.linear(x.to(self.device), self.decode(check=check), bias)
+        m = math.prod(x.shape[:-1])
+        if batch_invariant or m > 8 or m == 0:
+            return self.gemm(x, bias, check=check)
+        return self.gemv(x, bias, check=check)
 
     def gather_rows(self, ids, *, check=True):
         import torch

@@ -192,11 +192,100 @@ struct Raw6x16 {
   }
 };
 
+// ---- pieces of the tile walk shared by the GEMV and GEMM kernels ----
+
+// this row class's lookup tables -> LDS, one block per column class: table, then lookup bytes
+__device__ __forceinline__ void fused_load_tables(uint8_t *lds, uint32_t blocks, uint32_t block_pitch,
+                                                  const grf_bctx_fused &f, uint32_t cls, uint32_t tid,
+                                                  uint32_t nthreads) {
+  const uint32_t nb = 1u << f.lognb, entries = f.tabn + 1;
+  for (uint32_t c = 0; c < f.nc; ++c) {
+    const uint4 *src = reinterpret_cast<const uint4 *>(f.lut + ((size_t)cls * f.nc + c) * nb);
+    uint4 *dst = reinterpret_cast<uint4 *>(lds + blocks + c * block_pitch + kTabBytes);
+    for (uint32_t i = tid; i < nb / 16; i += nthreads) dst[i] = src[i];
+    const uint2 *ts = reinterpret_cast<const uint2 *>(f.tab) + ((size_t)cls * f.nc + c) * entries;
+    uint2 *td = reinterpret_cast<uint2 *>(lds + blocks + c * block_pitch);
+    for (uint32_t i = tid; i < entries; i += nthreads) td[i] = ts[i];
+  }
+}
+
+// Copy the main-stream bytes of one row piece (segments [seg_base, seg_base+nseg)) to LDS
+// at piece_off, keeping the 16-byte phase of the global address.  The P lanes of the row
+// share the copy.  Returns the aligned global start so lanes can place their cursors.
+__device__ __forceinline__ uint32_t fused_stage_piece(uint8_t *lds, uint32_t piece_off, const grf_bctx_fused &f,
+                                                      uint32_t seg_base, uint32_t nseg, uint32_t p, uint32_t P) {
+  const uint32_t g0 = f.seg_offset[seg_base], g1 = f.seg_offset[seg_base + nseg];
+  const uint32_t a0 = g0 & ~15u;
+  for (uint32_t o = a0 + p * 16; o < g1; o += P * 16)
+    *reinterpret_cast<uint4 *>(lds + piece_off + (o - a0)) = *reinterpret_cast<const uint4 *>(f.main_bytes + o);
+  return a0;
+}
+
+// A lane's position in its segment: rANS state, LDS cursor, and the registers that hold
+// the packed residuals and column classes of the next 16 symbols.
+struct SegmentWalk {
+  uint32_t state, ip, ip0, gofs, seg;
+  const uint32_t *rawp;
+  const uint4 *ccp;
+  uint32_t n0, n1, n2;
+  uint4 nc4;
+
+  __device__ __forceinline__ void open(const grf_bctx_fused &f, uint32_t seg_, uint32_t piece_off, uint32_t a0,
+                                       uint64_t elem0, uint32_t col0) {
+    seg = seg_;
+    state = f.seg_state[seg];
+    gofs = f.seg_offset[seg];
+    ip0 = piece_off + (gofs - a0);
+    ip = ip0;
+    rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
+    ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
+    n0 = rawp[0];
+    n1 = rawp[1];
+    n2 = rawp[2];
+    nc4 = ccp[0];
+  }
+
+  // Decode symbols [t, t+16) of the segment into eight BF16 pairs (word k in the low half,
+  // k+1 in the high half); loads the registers for the following group meanwhile.
+  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const FusedParams &q, uint32_t (&pair)[8]);
+
+  // the segment must end exactly on the next checkpoint
+  __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
+    return state == f.seg_state[seg + 1] && gofs + (ip - ip0) == f.seg_offset[seg + 1];
+  }
+};
+
 // BF16 word in bits 0..15 (bits above are unspecified): symbol bits | mantissa low 5 bits
 // | sign << 15.  r6 * (1 + 2^10) puts the five mantissa bits at 0..4 and the sign at 15
 // (a 24-bit multiply); the mask drops the copies that land elsewhere.
 __device__ __forceinline__ uint32_t fused_word_bits(uint32_t hi, uint32_t r6) {
   return ((r6 * 0x401u) & 0x801Fu) | hi;
+}
+
+__device__ __forceinline__ void SegmentWalk::decode16(uint32_t t, uint32_t S, const FusedParams &q,
+                                                     uint32_t (&pair)[8]) {
+  Raw6x16 rr;
+  rr.set(n0, n1, n2);
+  const uint32_t cw[4] = {nc4.x, nc4.y, nc4.z, nc4.w};
+  if (t + 16 < S) {
+    const uint32_t *nx = rawp + (t / 16 + 1) * 3;
+    n0 = nx[0];
+    n1 = nx[1];
+    n2 = nx[2];
+    nc4 = ccp[t / 16 + 1];
+  }
+  uint32_t bits[16];
+#define GRF_STEP(k)                                                            \
+  {                                                                            \
+    const uint32_t cc = __builtin_amdgcn_ubfe(cw[(k) / 4], 8 * ((k) % 4), 8);  \
+    const uint32_t hi = fused_symbol(state, ip, cc, q);                        \
+    bits[k] = fused_word_bits(hi, rr.field<k>());                              \
+  }
+  GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
+  GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
+#undef GRF_STEP
+#pragma unroll
+  for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
 }
 
 }  // namespace grf

@@ -49,17 +49,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
 
-  {  // this row class's lookup tables -> LDS, one block per column class: table, then lookup bytes
-    const uint32_t nb = 1u << f.lognb, entries = f.tabn + 1;
-    for (uint32_t c = 0; c < f.nc; ++c) {
-      const uint4 *src = reinterpret_cast<const uint4 *>(f.lut + ((size_t)cls * f.nc + c) * nb);
-      uint4 *dst = reinterpret_cast<uint4 *>(lds + L.blocks + c * L.block_pitch + grf::kTabBytes);
-      for (uint32_t i = tid; i < nb / 16; i += nthreads) dst[i] = src[i];
-      const uint2 *ts = reinterpret_cast<const uint2 *>(f.tab) + ((size_t)cls * f.nc + c) * entries;
-      uint2 *td = reinterpret_cast<uint2 *>(lds + L.blocks + c * L.block_pitch);
-      for (uint32_t i = tid; i < entries; i += nthreads) td[i] = ts[i];
-    }
-  }
+  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   const grf::FusedParams q{f.shift, L.block_pitch, (1u << f.shift) - 1u};
 
   const uint32_t r = tid / P, p = tid % P;
@@ -88,53 +78,21 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
     const uint32_t piece_off = L.stream + r * g.piece_cap;
     if (row != grf::kNoRow) {
       seg_base = row * f.segs_per_row + first_seg;
-      const uint32_t g0 = f.seg_offset[seg_base], g1 = f.seg_offset[seg_base + nseg];
-      a0 = g0 & ~15u;
-      for (uint32_t o = a0 + p * 16; o < g1; o += P * 16)
-        *reinterpret_cast<uint4 *>(lds + piece_off + (o - a0)) = *reinterpret_cast<const uint4 *>(f.main_bytes + o);
+      a0 = grf::fused_stage_piece(lds, piece_off, f, seg_base, nseg, p, P);
     }
     __syncthreads();
     if (row != grf::kNoRow && p < nseg) {
-      const uint32_t seg = seg_base + p;
-      uint32_t state = f.seg_state[seg];
-      const uint32_t gofs = f.seg_offset[seg];
-      const uint32_t ip0 = piece_off + (gofs - a0);
-      uint32_t ip = ip0;
       const uint32_t col0 = (first_seg + p) * S;
       const uint64_t elem0 = (uint64_t)row * K + col0;
-      const uint32_t *rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
-      const uint4 *ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
+      grf::SegmentWalk w;
+      w.open(f, seg_base + p, piece_off, a0, elem0, col0);
       const uint16_t *xr = xs + p * xpitch;
-      // registers for the next group of 16 are loaded while the current one is decoded
-      uint32_t n0 = rawp[0], n1 = rawp[1], n2 = rawp[2];
-      uint4 nc4 = ccp[0];
       float acc[M];
 #pragma unroll
       for (int m = 0; m < M; ++m) acc[m] = 0.f;
       for (uint32_t t = 0; t < S; t += 16) {
-        grf::Raw6x16 rr;
-        rr.set(n0, n1, n2);
-        const uint32_t cw[4] = {nc4.x, nc4.y, nc4.z, nc4.w};
-        if (t + 16 < S) {
-          const uint32_t *nx = rawp + (t / 16 + 1) * 3;
-          n0 = nx[0];
-          n1 = nx[1];
-          n2 = nx[2];
-          nc4 = ccp[t / 16 + 1];
-        }
-        uint32_t bits[16];
-#define GRF_STEP(k)                                                       \
-  {                                                                       \
-    const uint32_t cc = __builtin_amdgcn_ubfe(cw[(k) / 4], 8 * ((k) % 4), 8); \
-    const uint32_t hi = grf::fused_symbol(state, ip, cc, q);              \
-    bits[k] = grf::fused_word_bits(hi, rr.field<k>());                   \
-  }
-        GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
-        GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
-#undef GRF_STEP
-        uint32_t pair[8];  // BF16 words k (low half) and k+1 (high half)
-#pragma unroll
-        for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
+        uint32_t pair[8];
+        w.decode16(t, S, q, pair);
         if (STORE) {
           uint4 *dst = reinterpret_cast<uint4 *>(out + elem0 + t);
           dst[0] = make_uint4(pair[0], pair[1], pair[2], pair[3]);
@@ -154,8 +112,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
 #pragma unroll
         for (int m = 0; m < M; ++m) part[(r * f.segs_per_row + first_seg + p) * M + m] = acc[m];
       }
-      // the segment must end exactly on the next checkpoint
-      if (state != f.seg_state[seg + 1] || gofs + (ip - ip0) != f.seg_offset[seg + 1]) bad |= GRF_ERR_CHECKPOINT;
+      if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
     }
   }
 
@@ -175,7 +132,10 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   if (bad) atomicOr(error, (int)bad);
 }
 
-int check_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who) {
+}  // namespace
+
+namespace grf {
+int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who) {
   auto bad = [&](const char *why) { return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": " + why); };
   if (!f.main_bytes || !f.raw6 || !f.seg_state || !f.seg_offset || !g.tile_rows || !g.tile_class || !f.lut ||
       !f.tab || !f.col_class)
@@ -194,6 +154,10 @@ int check_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *
   if ((uint64_t)f.rows * f.cols > 0xFFFFFFFFull) return bad("matrix too large");
   return GRF_OK;
 }
+}  // namespace grf
+
+namespace {
+using grf::check_fused_frame;
 
 template <int M, bool STORE>
 int launch(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint16_t *y,
@@ -226,7 +190,7 @@ int grf_bctx_gemv(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
                   void *hip_stream) {
   if (!frame || !tiling || !x || !y || !error)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemv: null argument");
-  if (int rc = check_frame(*frame, *tiling, "grf_bctx_gemv")) return rc;
+  if (int rc = check_fused_frame(*frame, *tiling, "grf_bctx_gemv")) return rc;
   if (m_rows < 1 || m_rows > 8) return grf::set_error(GRF_UNSUPPORTED, "grf_bctx_gemv: 1 <= m_rows <= 8");
   if (ldx < frame->cols || ldy < frame->rows || (ldx & 1) || ((uintptr_t)x & 3))
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemv: x must be 4-byte aligned with an even leading dimension");
@@ -249,7 +213,7 @@ int grf_bctx_fused_decode(const grf_bctx_fused *frame, const grf_fused_tiling *t
                           int32_t *error, void *hip_stream) {
   if (!frame || !tiling || !out || !error)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_fused_decode: null argument");
-  if (int rc = check_frame(*frame, *tiling, "grf_bctx_fused_decode")) return rc;
+  if (int rc = check_fused_frame(*frame, *tiling, "grf_bctx_fused_decode")) return rc;
   return launch<1, true>(*frame, *tiling, nullptr, 0, nullptr, 0, nullptr, out, error, (hipStream_t)hip_stream);
 }
 

@@ -210,6 +210,15 @@ int grf_bctx_gemv(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
 int grf_bctx_fused_decode(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint16_t *out,
                           int32_t *error, void *hip_stream);
 
+/* Fused decode-GEMM on the matrix cores for any number of activation rows; same operand
+ * meaning as grf_bctx_gemv.  Batch-invariant in the sense of GS/bi_csrc/bi_gemm.cuh:1-17:
+ * with one tiling, row m of y is a function of row m of x and of W only.  x must be
+ * 8-byte aligned with ldx a multiple of 4.  More than 128 rows run as several launches. */
+int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, const uint16_t *x, uint32_t ldx,
+                  uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
+                  void *hip_stream);
+uint32_t grf_bctx_gemm_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint32_t m_rows);
+
 /* LDS bytes a launch needs for the given m_rows (0 for the store sink). */
 uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint32_t m_rows);
 

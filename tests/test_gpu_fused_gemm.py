@@ -1,0 +1,71 @@
+"""Fused decode-GEMM on the matrix cores: accuracy, batch invariance, edge shapes."""
+import numpy as np
+import pytest
+
+from conftest import bf16_words, weight_like, words_to_float
+
+pytestmark = pytest.mark.gpu
+
+
+def _tensor(words, nr=16, nc=4, **kw):
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd.bitexact_context_gpu import HipContextTensor
+    frame = codec.encode(words, row_classes=nr, col_classes=nc)
+    return frame, HipContextTensor(frame, stride=1024, device="cuda:0", **kw)
+
+
+@pytest.mark.parametrize("shape", [(64, 256), (512, 1280), (100, 384), (48, 2176), (1024, 1024)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
+def test_gemm_matches_float64_and_rows_do_not_depend_on_batch(oracle, shape):
+    import torch
+    rng = np.random.default_rng(shape[0] + shape[1])
+    words = weight_like(rng, *shape)
+    frame, t = _tensor(words)
+    assert t.fused is not None, t.fused_reason
+    print("gemm tiling", t._gemm_tiling()[3], flush=True)
+    w64 = words_to_float(oracle.bctx_decode(frame)).astype(np.float64)
+    xw = bf16_words(rng.normal(0, 1, size=(160, shape[1])))
+    x = torch.from_numpy(xw).view(torch.bfloat16).cuda()
+    xf = words_to_float(xw).astype(np.float64)
+    ref = xf @ w64.T
+    scale = np.abs(xf) @ np.abs(w64).T
+    y_all = t.gemm(x, check=True)
+    got = words_to_float(y_all.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    # 1e-2 relative to the result (bar of the task), measured against the magnitude of the terms
+    assert np.all(np.abs(got - ref) <= 1e-2 * np.maximum(np.abs(ref), 1e-3 * scale) + 1e-30)
+    for m in (1, 8, 16, 17, 32, 64, 128, 129):
+        ym = t.gemm(x[:m], check=True)
+        assert torch.equal(ym.view(torch.uint16), y_all[:m].view(torch.uint16)), f"batch {m} changed a row"
+    # a row keeps its bits wherever it sits in the batch
+    perm = torch.randperm(160, generator=torch.Generator().manual_seed(1)).cuda()
+    y_perm = t.gemm(x[perm], check=True)
+    assert torch.equal(y_perm.view(torch.uint16), y_all[perm].view(torch.uint16))
+    # linear() routes through the same kernel when asked to be batch-invariant
+    y1 = t.linear(x[:1], batch_invariant=True)
+    assert torch.equal(y1.view(torch.uint16), y_all[:1].view(torch.uint16))
+
+
+def test_gemm_bias_strided_input_and_dense_agreement(oracle):
+    import torch
+    rng = np.random.default_rng(5)
+    words = weight_like(rng, 192, 768)
+    frame, t = _tensor(words)
+    base = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(40, 2, 768)))).view(torch.bfloat16).cuda()
+    x = base[:, 1, :]  # row stride 1536: a strided view
+    bias = torch.from_numpy(bf16_words(rng.normal(0, 1, size=192))).view(torch.bfloat16).cuda()
+    y = t.linear(x, bias, check=True)
+    assert y.shape == (40, 192)
+    dense = torch.nn.functional.linear(x.float(), t.decode().float(), bias.float())
+    assert torch.allclose(y.float(), dense, rtol=1e-2, atol=2e-2)
+    assert t.gemm(x[:0]).shape == (0, 192)
+
+
+def test_gemm_checkpoint_mismatch_sets_error(oracle):
+    import torch
+    from georefine_amd import bitexact_context_codec as codec
+    words = weight_like(np.random.default_rng(29), 64, 512)
+    frame, t = _tensor(words)
+    t.buffers["fused_seg_state"].view(torch.int32)[7] += 1  # forced from the host; the kernel finishes normally
+    x = torch.zeros(32, 512, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(codec.CodecError):
+        t.gemm(x, check=True)
