@@ -1,0 +1,157 @@
+"""Indexed device decoding of PPCX frames on MI355X.
+
+``_read_frame`` and ``HipPredictiveTensor`` keep the contract of the reference's
+``_read_frame`` / ``CudaPredictiveTensor`` (GCR/bitexact_predictive_gpu.py:87-136 and
+:138-174): ``factory(frame, reference_uint16_numpy, stride=..., device=...)``, then
+``shape``, ``frame_sha256``, ``source_sha256``, ``resident_bytes`` and
+``decode(reference_bf16_device, check=)``.  The reference words are an input of every
+decode: the kernel derives each symbol's context from the reference word at the same
+position (sign alignment per row, ordinal key, threshold bin).
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import math
+import os
+
+import numpy as np
+
+from . import _hip_abi, _native, _tables
+from . import bitexact_predictive_codec as codec
+
+
+def _ptr(a, t):
+    return a.ctypes.data_as(ctypes.POINTER(t))
+
+
+def _checkpoints(stream, ctx, freq, vocab, stride):
+    """(states, offsets, symbols) of one stream via ``ppcx_checkpoint``."""
+    ctx = np.ascontiguousarray(ctx, dtype="<u2")
+    freq = np.ascontiguousarray(freq, dtype="<u4")
+    n = len(ctx)
+    states = np.empty((n + stride - 1) // stride, dtype="<u4")
+    offsets = np.empty_like(states)
+    symbols = np.empty(n, dtype="<u2")
+    data = np.frombuffer(stream, dtype=np.uint8)
+    backend = os.environ.get("BITEXACT_PREDICTIVE_FAST_INDEX", "0")
+    if backend not in ("0", "1"):
+        raise codec.CodecError("BITEXACT_PREDICTIVE_FAST_INDEX must be 0 or 1")
+    lib = _native.codec()
+    fn = lib.ppcx_checkpoint_binary if backend == "1" else lib.ppcx_checkpoint
+    status = fn(_ptr(data, ctypes.c_uint8), len(data), n, _ptr(ctx, ctypes.c_uint16), freq.size // vocab, vocab,
+                _ptr(freq, ctypes.c_uint32), stride, _ptr(states, ctypes.c_uint32), _ptr(offsets, ctypes.c_uint32),
+                _ptr(symbols, ctypes.c_uint16))
+    if status:
+        raise codec.CodecError(f"PPCX checkpoint validation failed ({status})")
+    return states, offsets, symbols
+
+
+def _read_frame(frame, reference, stride):
+    """Parse, validate and index a frame against its reference words."""
+    if not isinstance(frame, (bytes, bytearray, memoryview)):
+        raise codec.CodecError("frame must be bytes")
+    info = codec.parse(frame, reference)
+    r, c = info["shape"]
+    n = r * c
+    target_hash = info["target_sha256"]
+    result = dict(shape=(r, c), mode=info["mode"], frame_bytes=len(frame),
+                  frame_sha256=hashlib.sha256(bytes(frame)).hexdigest(), source_sha256=target_hash.hex(),
+                  target_sha256=target_hash.hex(), reference_sha256=info["reference_sha256"].hex())
+    if info["mode"] == 2:
+        target = np.frombuffer(info["data"], dtype="<u2").copy().reshape(r, c)
+        if hashlib.sha256(target.tobytes()).digest() != target_hash:
+            raise codec.CodecError("target checksum mismatch")
+        result["raw"] = target
+        return result
+    freq = info["main_freq"].reshape(codec.MAIN_CONTEXTS, codec.MAIN_VOCAB)
+    ctx = codec.contexts(info["reference"], info["labels"], info["flips"], info["thresholds"])
+    states, offsets, main = _checkpoints(info["stream"], ctx, freq, codec.MAIN_VOCAB, stride)
+    result.update(labels=info["labels"], flips=info["flips"], thresholds=info["thresholds"], main_freq=freq,
+                  main_stream=np.frombuffer(info["stream"], dtype=np.uint8).copy(), main_states=states,
+                  main_offsets=offsets)
+    if info["mode"] == 0:
+        residual = codec._unpackbits(info["data"], 5, n, "raw5")
+        result.update(raw5=np.frombuffer(info["data"], dtype=np.uint8).copy(), residual_symbols=residual)
+    else:
+        rf = info["residual_freq"].reshape(codec.RES_CONTEXTS, codec.RES_VOCAB)
+        rs, ro, residual = _checkpoints(info["residual_stream"], main, rf, codec.RES_VOCAB, stride)
+        result.update(residual_freq=rf, residual_stream=np.frombuffer(info["residual_stream"], dtype=np.uint8).copy(),
+                      residual_states=rs, residual_offsets=ro)
+    if hashlib.sha256(codec.join_symbols(main, residual).tobytes()).digest() != target_hash:
+        raise codec.CodecError("target checksum mismatch")
+    return result
+
+
+class HipPredictiveTensor:
+    """A PPCX-coded BF16 matrix resident on one MI355X; decoding needs the reference matrix."""
+
+    def __init__(self, frame, reference_uint16_numpy, stride=1024, device="cuda:0"):
+        if not isinstance(stride, int) or not 1 <= stride <= 65536:
+            raise codec.CodecError("invalid checkpoint stride")
+        ix = _read_frame(frame, reference_uint16_numpy, stride)
+        import torch
+        if not torch.cuda.is_available():
+            raise RuntimeError("a ROCm GPU is required")
+        self._lib = _native.hip()
+        self.shape = ix["shape"]
+        self.n = math.prod(self.shape)
+        self.stride, self.mode = stride, ix["mode"]
+        self.device = torch.device(device)
+        for key in ("source_sha256", "target_sha256", "reference_sha256", "frame_sha256", "frame_bytes"):
+            setattr(self, key, ix[key])
+        self.buffers = {}
+        for name, array in ix.items():
+            if isinstance(array, np.ndarray) and name != "residual_symbols":
+                self.buffers[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
+        for name in ("main", "residual"):
+            if name + "_freq" in ix:
+                cum = _tables.cumulative(ix[name + "_freq"])
+                self.buffers[name + "_cum"] = torch.from_numpy(cum).to(self.device)
+                self.buffers[name + "_bucket"] = torch.from_numpy(_tables.coarse_buckets(cum)).to(self.device)
+        self.error = torch.zeros((), device=self.device, dtype=torch.int32)
+        self.resident_bytes = int(sum(t.numel() * t.element_size() for t in self.buffers.values()) + 4)
+        self._frame = None
+        if self.mode != 2:
+            b = self.buffers
+            f = _hip_abi.GrfPpcxFrame()
+            f.main.bytes, f.main.n_bytes = b["main_stream"].data_ptr(), b["main_stream"].numel()
+            f.main.vocab, f.main.nctx = codec.MAIN_VOCAB, codec.MAIN_CONTEXTS
+            f.main.cum, f.main.bucket = b["main_cum"].data_ptr(), b["main_bucket"].data_ptr()
+            f.main.states, f.main.offsets = b["main_states"].data_ptr(), b["main_offsets"].data_ptr()
+            if self.mode == 0:
+                f.residual.bytes, f.residual.n_bytes = b["raw5"].data_ptr(), b["raw5"].numel()
+            else:
+                f.residual.bytes, f.residual.n_bytes = b["residual_stream"].data_ptr(), b["residual_stream"].numel()
+                f.residual.vocab, f.residual.nctx = codec.RES_VOCAB, codec.RES_CONTEXTS
+                f.residual.cum, f.residual.bucket = b["residual_cum"].data_ptr(), b["residual_bucket"].data_ptr()
+                f.residual.states = b["residual_states"].data_ptr()
+                f.residual.offsets = b["residual_offsets"].data_ptr()
+            f.labels, f.flips, f.thresholds = b["labels"].data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr()
+            f.rows, f.cols = self.shape
+            f.mode, f.stride = self.mode, stride
+            self._frame = f
+
+    def decode(self, reference_bf16_device, check=True):
+        import torch
+        if self.mode == 2:
+            return self.buffers["raw"].view(torch.bfloat16).reshape(self.shape)
+        ref = reference_bf16_device.to(device=self.device).contiguous()
+        if tuple(ref.shape) != tuple(self.shape) or ref.dtype != torch.bfloat16:
+            raise ValueError("reference device tensor shape/dtype mismatch")
+        count = (self.n + self.stride - 1) // self.stride
+        out = torch.empty(count * self.stride, device=self.device, dtype=torch.uint16)
+        self.error.zero_()
+        with torch.cuda.device(self.device):
+            status = self._lib.grf_ppcx_decode(ctypes.byref(self._frame), ref.data_ptr(), out.data_ptr(),
+                                               self.error.data_ptr(),
+                                               torch.cuda.current_stream(self.device).cuda_stream)
+        if status:
+            raise codec.CodecError(f"device decode launch failed ({status}): "
+                                   + self._lib.grf_last_error().decode(errors="replace"))
+        if check and self.error.item():
+            raise codec.CodecError("HIP PPCX checkpoint/context mismatch")
+        return out[:self.n].view(torch.bfloat16).reshape(self.shape)
+
+
+CudaPredictiveTensor = HipPredictiveTensor
