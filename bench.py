@@ -102,6 +102,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-rows", type=int, default=4096)
     ap.add_argument("--only", default="", help="comma list of gate,up,down (profiling aid)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 128 MiB read + 128 MiB write elementwise kernel three times, so that a "
+                         "counter profile of this command holds a kernel of known traffic to scale by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this decode path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists)")
@@ -170,6 +173,13 @@ def main():
         if tensors[name].error.item():
             sys.exit(f"bench.py: decoder error word set for {name}")
 
+    if args.calibrate_copy:
+        src = torch.ones(32 * 1024 * 1024, dtype=torch.int32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+
     per_kernel_ms = {name: float(np.mean([starts[s][j].elapsed_time(ends[s][j]) for s in range(args.steps)]))
                      for j, name in enumerate(names)}
     alg = {name: algorithmic_bytes(tensors[name], m) for name in names}
@@ -178,6 +188,13 @@ def main():
     ms_per_step = wall / args.steps * 1e3
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     eff_bf16 = dense_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # HBM bytes per launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE (scaled by a copy
+    # kernel of known size); a recorded figure, bench.py cannot read hardware counters itself
+    traffic = None
+    recorded = ROOT / "profiles" / "fused_gemv_m1_qwen27b_mlp_traffic.json"
+    if m == 1 and recorded.exists():
+        traffic = json.loads(recorded.read_text()).get("traffic_bytes_per_launch")
 
     dom = max(names, key=lambda n_: per_kernel_ms[n_])
     achieved = alg[dom]["total"] / (per_kernel_ms[dom] * 1e-3) / 1e9
@@ -195,7 +212,7 @@ def main():
         "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": "fused decode-GEMV, batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
-                               "BCTX (16,4) mode-0 frames" % m,
+                               "BCTX (16,4) frames, residuals resident in packed 6-bit form" % m,
                    "batch": m, "matrices": names,
                    "segment": tensors[names[0]].fused_plan["seg_len"]},
         "effective_bf16_GBps": round(eff_bf16, 2),
@@ -206,7 +223,7 @@ def main():
                             "table_bytes": alg[n_]["tables"],
                             "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in names},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "kernel": f"fused_walk_kernel<{m},false> on {dom}"},
     }
     if not args.no_cpu_baseline and "gate" in words_of:
