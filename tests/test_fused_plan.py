@@ -1,0 +1,97 @@
+"""Host-side preparation for the fused kernels, checked without a GPU: the lookup tables
+resolve every slot to the right symbol, tilings cover every row once, LDS budgets hold."""
+import numpy as np
+import pytest
+
+from conftest import bf16_words, weight_like
+from georefine_amd import _fused
+from georefine_amd import bitexact_context_codec as codec
+from georefine_amd.bitexact_context_gpu import index_frame
+
+
+def _plan(words, nr=16, nc=4, segment=64):
+    frame = codec.encode(words, row_classes=nr, col_classes=nc)
+    ix = index_frame(frame, 1024, fused_segment=segment, raw6_residual=True)
+    plan = _fused.FramePlan(ix["shape"], ix["nr"], ix["nc"], ix["rows"], ix["main_freq"], ix["fused_states"],
+                            ix["fused_offsets"], len(ix["main_stream"]), segment)
+    return ix, plan
+
+
+def emulate_lookup(plan, rho, cc, slots):
+    """The device step's symbol search, in numpy: bucket -> sparse index, pick entry 0 or 1,
+    scan forward while the slot lies beyond the picked entry."""
+    nb = 1 << plan.lognb
+    lut = plan.lut[rho].reshape(plan.nc, nb)[cc]
+    tab = plan.tab[rho].reshape(plan.nc, plan.tabn + 1)[cc]
+    lo, hi = (tab & 0xFFFFFFFF).astype(np.int64), (tab >> 32).astype(np.int64)
+    start, fm1 = lo & 0xFFFF, lo >> 16
+    idx = lut[slots >> plan.shift].astype(np.int64)
+    idx = np.where(slots - start[idx] > fm1[idx], idx + 1, idx)
+    for _ in range(plan.tabn + 1):
+        beyond = slots - start[idx] > fm1[idx]
+        if not beyond.any():
+            break
+        idx = np.where(beyond, idx + 1, idx)
+    return hi[idx] >> 5, start[idx], fm1[idx] + 1
+
+
+@pytest.mark.parametrize("classes", [(16, 4), (1, 1), (64, 16), (4, 16)])
+def test_lookup_tables_resolve_every_slot(classes):
+    rng = np.random.default_rng(classes[0])
+    wide = bf16_words(np.exp2(rng.uniform(-30, 10, size=(128, 256))) * rng.choice([-1.0, 1.0], size=(128, 256)))
+    for words in (weight_like(rng, 128, 256), wide):
+        if codec.encode(words, row_classes=classes[0], col_classes=classes[1])[5] == 1:
+            continue  # the encoder fell back to raw words: nothing to look up
+        ix, plan = _plan(words, *classes)
+        freq = ix["main_freq"]
+        slots = np.arange(65536, dtype=np.int64)
+        for ctx in range(freq.shape[0]):
+            f = freq[ctx].astype(np.int64)
+            if not f.any():
+                continue
+            cum = np.concatenate(([0], np.cumsum(f)))
+            want = np.searchsorted(cum, slots, side="right") - 1
+            sym, start, fr = emulate_lookup(plan, ctx // plan.nc, ctx % plan.nc, slots)
+            assert np.array_equal(sym, want)
+            assert np.array_equal(start, cum[want]) and np.array_equal(fr, f[want])
+
+
+@pytest.mark.parametrize("shape", [(100, 384), (512, 1280), (37, 1024), (16, 2176)])
+def test_tilings_cover_each_row_once_with_one_class_per_tile(shape):
+    words = weight_like(np.random.default_rng(shape[0]), *shape)
+    ix, plan = _plan(words)
+    tilings = [plan.tiling(m) for m in (0, 1, 8)] + [plan.gemm_tiling()]
+    for t in tilings:
+        s = t["scalars"]
+        rows = t["tile_rows"].reshape(s["n_tiles"], s["rows_per_tile"])
+        real = rows[rows != 0xFFFFFFFF]
+        assert sorted(real.tolist()) == list(range(shape[0]))
+        for tile, cls in zip(rows, t["tile_class"]):
+            members = tile[tile != 0xFFFFFFFF]
+            assert members.size and np.all(ix["rows"][members] == cls)
+        assert s["threads"] % 64 == 0 and s["lanes_per_row"] * s["rows_per_tile"] <= s["threads"] <= 1024
+        assert s["n_slabs"] == -(-plan.spr // s["lanes_per_row"])
+        assert t["lds"] <= _fused.MAX_LDS
+        # a row piece of any slab fits its LDS slot together with the two bytes read ahead
+        off = plan.seg_offset.astype(np.int64)
+        for b in range(s["n_slabs"]):
+            first = np.arange(shape[0]) * plan.spr + b * s["lanes_per_row"]
+            last = first + min(s["lanes_per_row"], plan.spr - b * s["lanes_per_row"])
+            assert np.max(off[last] - (off[first] & ~15)) + 2 <= s["piece_cap"]
+    g = tilings[-1]["scalars"]
+    waves, blocks = g["threads"] // 64, -(-g["rows_per_tile"] // 16)
+    assert blocks <= waves and -(-8 // (waves // blocks)) <= 4
+
+
+def test_unsupported_frames_are_reported():
+    with pytest.raises(_fused.FusedUnsupported):
+        _fused.choose_segment(67)
+    assert _fused.choose_segment(5120) == 64 and _fused.choose_segment(48) == 16
+    assert _fused.choose_segment(5120, 128) == 128
+    words = np.arange(65536, dtype=np.uint16).reshape(256, 256)  # 1024 distinct symbols in one context
+    frame = codec.encode(words, row_classes=1, col_classes=1)
+    if frame[5] != 1:
+        ix = index_frame(frame, 1024, fused_segment=64, raw6_residual=True)
+        with pytest.raises(_fused.FusedUnsupported):
+            _fused.FramePlan(ix["shape"], ix["nr"], ix["nc"], ix["rows"], ix["main_freq"], ix["fused_states"],
+                             ix["fused_offsets"], len(ix["main_stream"]), 64)

@@ -1,0 +1,124 @@
+"""Device decode of PPCX frames, the mixed-reference predictor and the serving modules."""
+import hashlib
+import struct
+import zlib
+
+import numpy as np
+import pytest
+
+from conftest import bf16_words, weight_like
+
+pytestmark = pytest.mark.gpu
+
+
+def _frame_for_mode(codec, target, ref, mode):
+    labels, flips, th = codec._fit(target, ref)
+    main, residual = codec.split_symbols(target)
+    table, stream = codec._rans_encode(main.ravel(), codec.contexts(ref, labels, flips, th), 256, 2048)
+    meta = zlib.compress(labels.tobytes() + flips.tobytes() + th.tobytes(), 6)
+    hashes = (hashlib.sha256(ref.tobytes()).digest(), hashlib.sha256(target.tobytes()).digest())
+    if mode == 2:
+        body = codec.HEADER.pack(b"PPCX", 1, 2, 0, *target.shape, 0, 0, 0, *hashes) + target.tobytes()
+    else:
+        if mode == 0:
+            data = codec._packbits(residual.ravel(), 5)
+        else:
+            rt, rs = codec._rans_encode(residual.ravel(), main.ravel(), 2048, 32)
+            data = struct.pack("<I", len(rt)) + rt + rs
+        body = codec.HEADER.pack(b"PPCX", 1, mode, 0, *target.shape, len(meta), len(table), len(stream), *hashes)
+        body += meta + table + stream + data
+    return body + hashlib.sha256(body).digest()
+
+
+def _pairs():
+    rng = np.random.default_rng(77)
+    t = weight_like(rng, 96, 160)
+    tf = (t.astype(np.uint32) << 16).view(np.float32)
+    yield "near-reference", t, bf16_words(tf + rng.normal(0, 0.002, t.shape).astype(np.float32))
+    yield "random", rng.integers(0, 65536, (5, 71), dtype=np.uint16), rng.integers(0, 65536, (5, 71), dtype=np.uint16)
+    allw = np.arange(65536, dtype=np.uint16).reshape(256, 256)
+    yield "all-words", allw, np.roll(allw, 7, axis=1)
+    yield "negated", t, t ^ np.uint16(0x8000)
+
+
+@pytest.mark.parametrize("name,target,ref", list(_pairs()), ids=[p[0] for p in _pairs()])
+@pytest.mark.parametrize("mode", [0, 1, 2])
+@pytest.mark.parametrize("stride", [1, 17, 128, 1024])
+def test_ppcx_decode_matches_oracle(oracle, name, target, ref, mode, stride):
+    import torch
+    from georefine_amd import bitexact_predictive_codec as codec
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
+    if stride == 1 and target.size > 20000:
+        pytest.skip("one checkpoint per symbol is only exercised on the small cases")
+    frame = _frame_for_mode(codec, target, ref, mode)
+    expect = oracle.ppcx_decode(frame, ref)
+    assert np.array_equal(expect, target)
+    print(f"case={name} mode={mode} stride={stride}", flush=True)
+    t = HipPredictiveTensor(frame, ref, stride=stride, device="cuda:0")
+    ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
+    got = t.decode(ref_dev).view(torch.uint16).cpu().numpy()
+    assert np.array_equal(got, expect)
+    assert t.frame_sha256 == hashlib.sha256(frame).hexdigest()
+    assert t.source_sha256 == hashlib.sha256(target.tobytes()).hexdigest()
+    assert isinstance(t.resident_bytes, int) and t.resident_bytes > 0
+
+
+def test_ppcx_wrong_reference_on_device_sets_error(oracle):
+    import torch
+    from georefine_amd import bitexact_predictive_codec as codec
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
+    _, target, ref = next(_pairs())
+    t = HipPredictiveTensor(_frame_for_mode(codec, target, ref, 0), ref, stride=64)
+    other = torch.from_numpy(np.roll(ref, 3, axis=1).copy()).view(torch.bfloat16).cuda()
+    with pytest.raises(codec.CodecError):  # contexts differ: segments miss their checkpoints
+        t.decode(other)
+    with pytest.raises(ValueError):
+        t.decode(other[:, :8])
+
+
+def test_mix_predict_device_matches_host_bits(oracle):
+    import torch
+    from georefine_amd.bitexact_predictive_mix import PredictiveMixError, predict
+    rng = np.random.default_rng(12)
+    up, gate = bf16_words(rng.normal(size=(64, 300))), bf16_words(rng.normal(size=(64, 300)))
+    coeff = bf16_words(rng.normal(size=(64, 3)))
+    host = predict(up, gate, coeff)
+    assert np.array_equal(host, oracle.mix_predict(up, gate, coeff))
+    dev = predict(*(torch.from_numpy(a).view(torch.bfloat16).cuda() for a in (up, gate, coeff)))
+    assert np.array_equal(dev.view(torch.uint16).cpu().numpy(), host)
+    one = lambda v: torch.tensor([[v]], dtype=torch.float32).bfloat16().cuda()
+    exact = predict(one(1.0), one(0.01171875), torch.tensor([[1.0, 1.0, 0.0]]).bfloat16().cuda())
+    assert exact.view(torch.uint16).item() == 0x3F81  # truncated, not rounded
+    with pytest.raises(PredictiveMixError):
+        predict(one(float("nan")), one(1.0), torch.tensor([[1.0, 1.0, 0.0]]).bfloat16().cuda())
+
+
+def test_serving_modules_with_fused_and_predictive_weights(oracle):
+    import torch
+    from georefine_amd import bitexact_context_codec as bctx
+    from georefine_amd import bitexact_predictive_codec as ppcx
+    from georefine_amd import serving
+    rng = np.random.default_rng(31)
+    w = weight_like(rng, 128, 256)
+    tensor = serving.hip_tensor_factory(bctx.encode(w), stride=1024, device="cuda:0")
+    bias = torch.nn.Parameter(torch.from_numpy(bf16_words(rng.normal(size=128))).view(torch.bfloat16).cuda(),
+                              requires_grad=False)
+    layer = serving.BctxLinear(tensor, bias)
+    x = torch.from_numpy(bf16_words(rng.normal(size=(3, 5, 256)))).view(torch.bfloat16).cuda()
+    y = layer(x)
+    dense = torch.nn.functional.linear(x.float(), layer.weight.float(), bias.float())
+    assert y.shape == (3, 5, 128) and torch.allclose(y.float(), dense, rtol=1e-2, atol=2e-2)
+    assert layer.forward_calls == 1 and layer.weight_materializations == 1
+    emb = serving.BctxEmbedding(tensor)
+    ids = torch.tensor([[0, 127], [5, 5]], device="cuda")
+    assert np.array_equal(emb(ids).view(torch.uint16).cpu().numpy(), w[ids.cpu().numpy()])
+    # a predictive weight coded against the first one, stored transposed
+    tf = (w.astype(np.uint32) << 16).view(np.float32)
+    target = bf16_words(tf * 0.9 + rng.normal(0, 0.001, w.shape).astype(np.float32))
+    native = serving.hip_predictive_factory(ppcx.encode(target, w), w, stride=256, device="cuda:0")
+    wrapped = serving.PredictiveContextTensor(native, [tensor], transform="target transpose", shape=(256, 128),
+                                              source_sha256=native.source_sha256, frame_sha256=native.frame_sha256,
+                                              resident_bytes=native.resident_bytes)
+    assert np.array_equal(wrapped.decode().view(torch.uint16).cpu().numpy(), target.T)
+    out = serving.BctxLinear(wrapped)(torch.ones(2, 128, dtype=torch.bfloat16, device="cuda"))
+    assert out.shape == (2, 256)
