@@ -20,11 +20,10 @@
 //     the 16 column classes of the same columns.
 //
 // Symbol lookup: slot>>shift indexes a u8 table giving the sparse index of the
-// symbol that owns the bucket's first slot; the 8-byte entries of that symbol
-// and of its successor are read together and one compare picks between them.
-// Entry: low32 = start | (freq-1)<<16, high32 = symbol<<5 (the symbol's bits in
-// the BF16 word).  A selected symbol with freq < bucket size
-// may still end before the slot; a short forward scan then finishes the search.
+// symbol that owns the bucket's first slot; that symbol's 8-byte entry is read and
+// assumed to own the slot.  Entry: low32 = start | (freq-1)<<16, high32 = symbol<<5
+// (the symbol's bits in the BF16 word).  When a symbol boundary falls inside the
+// bucket before the slot, a forward scan over the following entries finishes the search.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -75,12 +74,12 @@ typedef __attribute__((address_space(3))) v2u32 lds_v2u32;
 __device__ __forceinline__ uint8_t lds_load_u8(uint32_t off) { return *reinterpret_cast<lds_u8 *>(off); }
 
 struct FusedParams {  // uniform values the step needs, kept in scalar registers
-  uint32_t shift, block_pitch, small_limit;
+  uint32_t shift, block_pitch;
 };
 
-// Slow twin of the step for the rare case that the selected symbol is smaller than a
-// bucket: scan forward from table address `ta` to the symbol that holds the slot, then
-// update and refill in plain C.  Returns the entry's high word.
+// Slow twin of the step for the rare case that the slot lies beyond the looked-up symbol:
+// scan forward from table address `ta` to the symbol that holds the slot, then update and
+// refill in plain C.  Returns the entry's high word.
 __device__ __forceinline__ uint32_t fused_symbol_scan(uint32_t &state, uint32_t &ip, uint32_t ta, uint32_t byte0,
                                                       uint32_t byte1) {
   const uint32_t slot = state & 0xFFFFu;
@@ -105,6 +104,11 @@ __device__ __forceinline__ uint32_t fused_symbol_scan(uint32_t &state, uint32_t 
 
 // One decode step of the main stream against LDS tables.  Returns the image
 // of the symbol's bits in the BF16 word (symbol << 5).
+//
+// The lookup byte names the symbol that owns the first slot of the slot's bucket.  With
+// buckets finer than almost every symbol, that symbol nearly always owns the slot itself,
+// so the step reads only its entry and assumes it; a lane whose slot lies beyond the entry
+// (a symbol boundary inside the bucket) redoes the step with a forward scan.
 __device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, uint32_t cc, const FusedParams &q) {
   // The two possible refill bytes, fetched ahead of need: the aligned dword that holds
   // byte `ip` and the dword after it, shifted so that the bytes sit in bits 0..15.
@@ -117,25 +121,19 @@ __device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, 
   const uint32_t idx = lds_load_u8(block + bucket + kTabBytes);
   const uint32_t ta = (idx << 3) + block;
   const v2u32 e0 = *reinterpret_cast<lds_v2u32 *>(ta);
-  const v2u32 e1 = *reinterpret_cast<lds_v2u32 *>(ta + 8);
   const uint32_t state_in = state, ip_in = ip;
-  uint32_t lo, hi, x, ipn;
+  uint32_t x, ipn, rel;
 #if defined(__HIP_DEVICE_COMPILE__)
   uint32_t t, a;
-  // Pick entry 0 or 1 (slot past entry 0's range), x = (freq-1)*h + (slot + h - start)
-  // with h = state>>16, then up to two refills (x << 8) | byte while x < 2^23, ip counting
-  // the bytes taken.  Operand halves are addressed with SDWA selects instead of shifts and
-  // masks; v_perm builds (x << 8) | byte from the byte register's low byte only.  gfx950
-  // needs two wait states between a VALU write of VCC and a VALU read of it.
+  // rel = slot - start; x = (freq-1)*h + (slot + h - start) with h = state>>16; then up to
+  // two refills (x << 8) | byte while x < 2^23, ip counting the bytes taken.  Operand halves
+  // are addressed with SDWA selects instead of shifts and masks; v_perm builds (x << 8) | byte.
+  // gfx950 needs two wait states between a VALU write of VCC and a VALU read of it.
   asm volatile(
-      "v_sub_u32_sdwa %[t], %[st], %[e0lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_0\n\t"
-      "v_cmp_gt_u32_sdwa vcc, %[t], %[e0lo] src0_sel:DWORD src1_sel:WORD_1\n\t"
+      "v_sub_u32_sdwa %[rel], %[st], %[e0lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_0\n\t"
       "v_add_u32_sdwa %[a], %[st], %[st] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-      "s_nop 0\n\t"
-      "v_cndmask_b32 %[lo], %[e0lo], %[e1lo], vcc\n\t"
-      "v_cndmask_b32 %[hi], %[e0hi], %[e1hi], vcc\n\t"
-      "v_mul_u32_u24_sdwa %[x], %[lo], %[st] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_1 src1_sel:WORD_1\n\t"
-      "v_sub_u32_sdwa %[a], %[a], %[lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_0\n\t"
+      "v_mul_u32_u24_sdwa %[x], %[e0lo], %[st] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_1 src1_sel:WORD_1\n\t"
+      "v_sub_u32_sdwa %[a], %[a], %[e0lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_0\n\t"
       "v_add_u32 %[x], %[x], %[a]\n\t"
       "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
       "v_perm_b32 %[t], %[x], %[b], %[sel0]\n\t"
@@ -147,25 +145,23 @@ __device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, 
       "s_nop 0\n\t"
       "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
       "v_addc_co_u32 %[ipo], vcc, 0, %[ipo], vcc\n\t"
-      : [x] "=&v"(x), [t] "=&v"(t), [a] "=&v"(a), [lo] "=&v"(lo), [hi] "=&v"(hi), [ipo] "=&v"(ipn)
-      : [st] "v"(state), [e0lo] "v"(e0.x), [e0hi] "v"(e0.y), [e1lo] "v"(e1.x), [e1hi] "v"(e1.y),
-        [b] "v"(bytes), [sel0] "s"(0x06050400u), [sel1] "s"(0x06050401u), [ipi] "v"(ip)
+      : [x] "=&v"(x), [t] "=&v"(t), [a] "=&v"(a), [rel] "=&v"(rel), [ipo] "=&v"(ipn)
+      : [st] "v"(state), [e0lo] "v"(e0.x), [b] "v"(bytes), [sel0] "s"(0x06050400u), [sel1] "s"(0x06050401u),
+        [ipi] "v"(ip)
       : "vcc");
 #else
-  lo = e0.x + e1.x + bytes;  // host pass only parses this
-  hi = e0.y + e1.y;
+  rel = e0.x + bytes;  // host pass only parses this
   x = state;
   ipn = ip;
 #endif
   state = x;
   ip = ipn;
-  if (__builtin_expect((lo >> 16) < q.small_limit, 0)) {
-    // freq < bucket size: the slot may lie beyond the picked entry.  Redo the step from the
-    // saved state with a forward scan starting at the picked entry.
+  uint32_t hi = e0.y;
+  if (__builtin_expect(rel > (e0.x >> 16), 0)) {
+    // the slot lies beyond the entry: redo the step from the saved state with a forward scan
     state = state_in;
     ip = ip_in;
-    const bool took1 = ((state_in & 0xFFFFu) - (e0.x & 0xFFFFu)) > (e0.x >> 16);
-    hi = fused_symbol_scan(state, ip, ta + (took1 ? 8u : 0u), bytes & 0xFFu, (bytes >> 8) & 0xFFu);
+    hi = fused_symbol_scan(state, ip, ta + 8, bytes & 0xFFu, (bytes >> 8) & 0xFFu);
   }
   return hi;
 }

@@ -50,7 +50,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   const uint32_t cls = g.tile_class[tile];
 
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
-  const grf::FusedParams q{f.shift, L.block_pitch, (1u << f.shift) - 1u};
+  const grf::FusedParams q{f.shift, L.block_pitch};
 
   const uint32_t r = tid / P, p = tid % P;
   const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
