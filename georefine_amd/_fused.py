@@ -41,8 +41,9 @@ def choose_shift(nc, budget=LUT_BUDGET):
 def sparse_tables(freq, nr, nc, shift):
     """Per row class: u8 lookup [nc << lognb] and u64 entries [nc][tabn+1].
 
-    Entry(column class c, sparse i): low32 = start | (freq-1) << 16, high32 = symbol << 5.
-    Unused entries are (start 0, freq 65536): a forward scan always stops on them."""
+    Entry(column class c, sparse i): low32 = start | (freq & 0xFFFF) << 16 with 0 standing for
+    65536, high32 = symbol << 5.  Unused entries are (start 0, freq 65536): a forward scan
+    always stops on them."""
     nz = freq > 0
     tabn = int(nz.sum(axis=1).max())
     if tabn == 0:
@@ -52,7 +53,7 @@ def sparse_tables(freq, nr, nc, shift):
     lognb = 16 - shift
     nb = 1 << lognb
     lut = np.zeros((nr, nc, nb), dtype=np.uint8)
-    tab = np.full((nr, nc, tabn + 1), np.uint64(0xFFFF0000), dtype=np.uint64)
+    tab = np.zeros((nr, nc, tabn + 1), dtype=np.uint64)
     first_slots = (np.arange(nb, dtype=np.int64) << shift)
     for rho in range(nr):
         for c in range(nc):
@@ -62,7 +63,7 @@ def sparse_tables(freq, nr, nc, shift):
                 continue
             fs = f[syms]
             starts = np.concatenate(([0], np.cumsum(fs)[:-1]))
-            lo = starts | ((fs - 1) << 16)
+            lo = starts | ((fs & 0xFFFF) << 16)
             hi = syms << 5
             tab[rho, c, :syms.size] = (lo.astype(np.uint64) | (hi.astype(np.uint64) << np.uint64(32)))
             lut[rho, c] = (np.searchsorted(starts, first_slots, side="right") - 1).astype(np.uint8)

@@ -21,7 +21,7 @@
 //
 // Symbol lookup: slot>>shift indexes a u8 table giving the sparse index of the
 // symbol that owns the bucket's first slot; that symbol's 8-byte entry is read and
-// assumed to own the slot.  Entry: low32 = start | (freq-1)<<16, high32 = symbol<<5
+// assumed to own the slot.  Entry: low32 = start | (freq & 0xFFFF)<<16 (0 stands for 65536), high32 = symbol<<5
 // (the symbol's bits in the BF16 word).  When a symbol boundary falls inside the
 // bucket before the slot, a forward scan over the following entries finishes the search.
 #pragma once
@@ -78,18 +78,20 @@ struct FusedParams {  // uniform values the step needs, kept in scalar registers
 };
 
 // Slow twin of the step for the rare case that the slot lies beyond the looked-up symbol:
-// scan forward from table address `ta` to the symbol that holds the slot, then update and
-// refill in plain C.  Returns the entry's high word.
-__device__ __forceinline__ uint32_t fused_symbol_scan(uint32_t &state, uint32_t &ip, uint32_t ta, uint32_t byte0,
-                                                      uint32_t byte1) {
+// scan forward from entry `e` at table address `ta` to the symbol that holds the slot, then
+// update and refill in plain C.  Returns the entry's high word.
+__device__ __forceinline__ uint32_t fused_symbol_scan(uint32_t &state, uint32_t &ip, uint32_t ta, v2u32 e,
+                                                      uint32_t byte0, uint32_t byte1) {
   const uint32_t slot = state & 0xFFFFu;
-  v2u32 e = *reinterpret_cast<lds_v2u32 *>(ta);
-  while ((slot - (e.x & 0xFFFFu)) > (e.x >> 16)) {
+  uint32_t freq = e.x >> 16;
+  freq = freq ? freq : 65536u;
+  while (slot - (e.x & 0xFFFFu) >= freq) {
     ta += 8;
     e = *reinterpret_cast<lds_v2u32 *>(ta);
+    freq = e.x >> 16;
+    freq = freq ? freq : 65536u;
   }
-  const uint32_t h = state >> 16;
-  uint32_t x = (e.x >> 16) * h + (slot + h - (e.x & 0xFFFFu));
+  uint32_t x = freq * (state >> 16) + (slot - (e.x & 0xFFFFu));
   if (x < kLow) {
     x = (x << 8) | byte0;
     ++ip;
@@ -102,66 +104,101 @@ __device__ __forceinline__ uint32_t fused_symbol_scan(uint32_t &state, uint32_t 
   return e.y;
 }
 
-// One decode step of the main stream against LDS tables.  Returns the image
-// of the symbol's bits in the BF16 word (symbol << 5).
+// cc * pitch with cc = byte BYTE of `ccw`: one multiply whose operand select does the extraction
+template <int BYTE>
+__device__ __forceinline__ uint32_t fused_block_offset(uint32_t ccw, uint32_t pitch) {
+  uint32_t block;
+#if defined(__HIP_DEVICE_COMPILE__)
+#define GRF_BLOCK(sel)                                                                                       \
+  asm("v_mul_u32_u24_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:" sel \
+      : "=v"(block)                                                                                          \
+      : "s"(pitch), "v"(ccw))
+  if constexpr (BYTE == 0) GRF_BLOCK("BYTE_0");
+  if constexpr (BYTE == 1) GRF_BLOCK("BYTE_1");
+  if constexpr (BYTE == 2) GRF_BLOCK("BYTE_2");
+  if constexpr (BYTE == 3) GRF_BLOCK("BYTE_3");
+#undef GRF_BLOCK
+#else
+  block = ((ccw >> (8 * BYTE)) & 0xFFu) * pitch;
+#endif
+  return block;
+}
+
+__device__ __forceinline__ uint32_t fused_lshl3_add(uint32_t a, uint32_t b) {  // (a << 3) + b in one instruction
+#if defined(__HIP_DEVICE_COMPILE__)
+  uint32_t r;
+  asm("v_lshl_add_u32 %0, %1, 3, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+#else
+  return (a << 3) + b;
+#endif
+}
+
+// One decode step of the main stream against LDS tables, for the column class held in byte
+// BYTE of `ccw`.  Returns the image of the symbol's bits in the BF16 word (symbol << 5).
 //
 // The lookup byte names the symbol that owns the first slot of the slot's bucket.  With
 // buckets finer than almost every symbol, that symbol nearly always owns the slot itself,
 // so the step reads only its entry and assumes it; a lane whose slot lies beyond the entry
-// (a symbol boundary inside the bucket) redoes the step with a forward scan.
-__device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, uint32_t cc, const FusedParams &q) {
-  // The two possible refill bytes, fetched ahead of need: the aligned dword that holds
-  // byte `ip` and the dword after it, shifted so that the bytes sit in bits 0..15.
-  // (An unaligned 16-bit LDS read stalls the LDS pipeline for tens of cycles on this
-  // hardware, and two byte reads cost two bank-conflicted accesses.)
-  const v2u32 dw = {*reinterpret_cast<lds_u32 *>(ip & ~3u), *reinterpret_cast<lds_u32 *>((ip & ~3u) + 4)};
-  const uint32_t bytes = __builtin_amdgcn_alignbyte(dw.y, dw.x, ip);
-  const uint32_t block = __umul24(cc, q.block_pitch);
+// (a symbol boundary inside the bucket, or the 16-bit frequency field's 0 = 65536) redoes
+// the step with a forward scan.
+template <int BYTE>
+__device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, uint32_t ccw, const FusedParams &q) {
+  // The two possible refill bytes, fetched ahead of need with two byte reads.  (An unaligned
+  // 16-bit LDS read stalls the LDS pipeline for tens of cycles on this hardware; aligned
+  // dwords cost two vector instructions to address and shift.)
+  const uint32_t b0 = lds_load_u8(ip), b1 = lds_load_u8(ip + 1);
+  const uint32_t block = fused_block_offset<BYTE>(ccw, q.block_pitch);
   const uint32_t bucket = (state & 0xFFFFu) >> q.shift;
   const uint32_t idx = lds_load_u8(block + bucket + kTabBytes);
-  const uint32_t ta = (idx << 3) + block;
+  const uint32_t ta = fused_lshl3_add(idx, block);
   const v2u32 e0 = *reinterpret_cast<lds_v2u32 *>(ta);
   const uint32_t state_in = state, ip_in = ip;
   uint32_t x, ipn, rel;
+  uint64_t miss;  // lanes whose slot lies beyond the entry
 #if defined(__HIP_DEVICE_COMPILE__)
-  uint32_t t, a;
-  // rel = slot - start; x = (freq-1)*h + (slot + h - start) with h = state>>16; then up to
-  // two refills (x << 8) | byte while x < 2^23, ip counting the bytes taken.  Operand halves
-  // are addressed with SDWA selects instead of shifts and masks; v_perm builds (x << 8) | byte.
+  uint32_t t;
+  // rel = slot - start; x = freq * (state >> 16) + rel; then up to two refills
+  // (x << 8) | byte while x < 2^23, ip counting the bytes taken.  Operand halves are
+  // addressed with operand selects instead of shifts and masks; v_perm builds (x << 8) | byte.
   // gfx950 needs two wait states between a VALU write of VCC and a VALU read of it.
   asm volatile(
       "v_sub_u32_sdwa %[rel], %[st], %[e0lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_0\n\t"
-      "v_add_u32_sdwa %[a], %[st], %[st] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_1\n\t"
-      "v_mul_u32_u24_sdwa %[x], %[e0lo], %[st] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_1 src1_sel:WORD_1\n\t"
-      "v_sub_u32_sdwa %[a], %[a], %[e0lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:WORD_0\n\t"
-      "v_add_u32 %[x], %[x], %[a]\n\t"
+      "v_mad_u32_u16 %[x], %[e0lo], %[st], %[rel] op_sel:[1,1,0,0]\n\t"
       "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
-      "v_perm_b32 %[t], %[x], %[b], %[sel0]\n\t"
+      "v_perm_b32 %[t], %[x], %[b0], %[sel]\n\t"
       "s_nop 0\n\t"
       "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
       "v_addc_co_u32 %[ipo], vcc, 0, %[ipi], vcc\n\t"
       "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
-      "v_perm_b32 %[t], %[x], %[b], %[sel1]\n\t"
+      "v_perm_b32 %[t], %[x], %[b1], %[sel]\n\t"
       "s_nop 0\n\t"
       "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
       "v_addc_co_u32 %[ipo], vcc, 0, %[ipo], vcc\n\t"
-      : [x] "=&v"(x), [t] "=&v"(t), [a] "=&v"(a), [rel] "=&v"(rel), [ipo] "=&v"(ipn)
-      : [st] "v"(state), [e0lo] "v"(e0.x), [b] "v"(bytes), [sel0] "s"(0x06050400u), [sel1] "s"(0x06050401u),
+      "v_cmp_ge_u32_sdwa %[miss], %[rel], %[e0lo] src0_sel:DWORD src1_sel:WORD_1\n\t"
+      : [x] "=&v"(x), [t] "=&v"(t), [rel] "=&v"(rel), [ipo] "=&v"(ipn), [miss] "=&s"(miss)
+      : [st] "v"(state), [e0lo] "v"(e0.x), [b0] "v"(b0), [b1] "v"(b1), [sel] "s"(0x06050400u),
         [ipi] "v"(ip)
       : "vcc");
 #else
-  rel = e0.x + bytes;  // host pass only parses this
+  rel = e0.x + b0 + b1;  // host pass only parses this
   x = state;
   ipn = ip;
+  miss = rel;
 #endif
   state = x;
   ip = ipn;
   uint32_t hi = e0.y;
-  if (__builtin_expect(rel > (e0.x >> 16), 0)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const bool redo = __builtin_amdgcn_inverse_ballot_w64(miss);
+#else
+  const bool redo = miss != 0;
+#endif
+  if (__builtin_expect(redo, 0)) {
     // the slot lies beyond the entry: redo the step from the saved state with a forward scan
     state = state_in;
     ip = ip_in;
-    hi = fused_symbol_scan(state, ip, ta + 8, bytes & 0xFFu, (bytes >> 8) & 0xFFu);
+    hi = fused_symbol_scan(state, ip, ta, e0, b0, b1);
   }
   return hi;
 }
@@ -273,8 +310,7 @@ __device__ __forceinline__ void SegmentWalk::decode16(uint32_t t, uint32_t S, co
   uint32_t bits[16];
 #define GRF_STEP(k)                                                            \
   {                                                                            \
-    const uint32_t cc = __builtin_amdgcn_ubfe(cw[(k) / 4], 8 * ((k) % 4), 8);  \
-    const uint32_t hi = fused_symbol(state, ip, cc, q);                        \
+    const uint32_t hi = fused_symbol<(k) % 4>(state, ip, cw[(k) / 4], q);      \
     bits[k] = fused_word_bits(hi, rr.field<k>());                              \
   }
   GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)

@@ -162,8 +162,8 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  *   lut         u8  [nr][nc << lognb]        lognb = 16 - shift; sparse index of the
  *                                            symbol owning the bucket's first slot
  *   tab         u64 [nr][nc][tabn+1]         entry(cc, sparse): low32 = start |
- *                                            (freq-1)<<16, high32 = symbol<<5;
- *                                            unused entries: start 0, freq 65536
+ *                                            (freq & 0xFFFF)<<16 (0 stands for 65536),
+ *                                            high32 = symbol<<5; unused entries: 0
  *   col_class   u8  [cols]
  * main_bytes must be readable for 16 bytes past main_n_bytes. */
 typedef struct grf_bctx_fused {

@@ -18,21 +18,21 @@ def _plan(words, nr=16, nc=4, segment=64):
 
 
 def emulate_lookup(plan, rho, cc, slots):
-    """The device step's symbol search, in numpy: bucket -> sparse index, pick entry 0 or 1,
-    scan forward while the slot lies beyond the picked entry."""
+    """The device step's symbol search, in numpy: bucket -> sparse index, then scan forward
+    while the slot lies beyond the entry (frequency field 0 stands for 65536)."""
     nb = 1 << plan.lognb
     lut = plan.lut[rho].reshape(plan.nc, nb)[cc]
     tab = plan.tab[rho].reshape(plan.nc, plan.tabn + 1)[cc]
     lo, hi = (tab & 0xFFFFFFFF).astype(np.int64), (tab >> 32).astype(np.int64)
-    start, fm1 = lo & 0xFFFF, lo >> 16
+    start, freq = lo & 0xFFFF, lo >> 16
+    freq = np.where(freq == 0, 65536, freq)
     idx = lut[slots >> plan.shift].astype(np.int64)
-    idx = np.where(slots - start[idx] > fm1[idx], idx + 1, idx)
     for _ in range(plan.tabn + 1):
-        beyond = slots - start[idx] > fm1[idx]
+        beyond = slots - start[idx] >= freq[idx]
         if not beyond.any():
             break
         idx = np.where(beyond, idx + 1, idx)
-    return hi[idx] >> 5, start[idx], fm1[idx] + 1
+    return hi[idx] >> 5, start[idx], freq[idx]
 
 
 @pytest.mark.parametrize("classes", [(16, 4), (1, 1), (64, 16), (4, 16)])
