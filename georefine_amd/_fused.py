@@ -13,7 +13,7 @@ import os
 import numpy as np
 
 MAX_LDS = 160 * 1024
-LUT_BUDGET = int(os.environ.get("GEOREFINE_FUSED_LUT_BYTES", 16 * 1024))
+LUT_BUDGET = int(os.environ.get("GEOREFINE_FUSED_LUT_BYTES", 32 * 1024))
 
 
 class FusedUnsupported(ValueError):
@@ -70,23 +70,24 @@ def sparse_tables(freq, nr, nc, shift):
     return lut.reshape(nr, nc * nb), tab.reshape(nr, nc * (tabn + 1)), tabn
 
 
+WALK_KNEE = int(os.environ.get("GEOREFINE_FUSED_WALK_KNEE", 32))
 X_PAD = 8
-TAB_CAP = 257  # entries reserved per column class in LDS
 
 
-def lds_bytes(nc, lognb, tabn, m, p, s, r, piece_cap, spr):
+def lds_bytes(nc, lognb, tabn, m, p, s, r, piece_cap):
     a16 = lambda v: (v + 15) // 16 * 16
-    total = a16(nc * (TAB_CAP * 8 + (1 << lognb)))
+    total = a16(nc * (a16((tabn + 1) * 8) + (1 << lognb)))
     total = a16(total + r * piece_cap)
     total = a16(total + m * p * (s + X_PAD) * 2)
-    total = a16(total + r * spr * m * 4)
+    total = a16(total + r * p * m * 4)
+    total = a16(total + r * m * 4)
     return total
 
 
-def lds_bytes_gemm(nc, lognb, m16, p, r, piece_cap):
+def lds_bytes_gemm(nc, lognb, tabn, m16, p, r, piece_cap):
     a16 = lambda v: (v + 15) // 16 * 16
     pitch = p * 32 + 8
-    total = a16(nc * (TAB_CAP * 8 + (1 << lognb)))
+    total = a16(nc * (a16((tabn + 1) * 8) + (1 << lognb)))
     total = a16(total + r * piece_cap)
     total = a16(total + a16(r) * pitch)
     total = a16(total + m16 * pitch)
@@ -106,14 +107,15 @@ def piece_capacity(offsets, rows, spr, p):
     return (longest + 2 + 15) // 16 * 16
 
 
-def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
+def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False, rows_per_lane=1):
     """(threads T, lanes_per_row P, rows_per_tile R, ...): best modelled throughput.
 
     The walk is a chain of dependent steps per lane, so time ~ steps per lane x rounds
     of workgroups, at the speed the resident wave count allows.  The model multiplies
     lane efficiency (idle lanes in the last slab and in a partly filled workgroup), tile
-    fill, how evenly the tiles fill the machine, and a penalty below 24 waves per CU
-    (measured: the dependent LDS round trips of a step need that many waves to overlap)."""
+    fill, how evenly the tiles fill the machine, and a penalty below WALK_KNEE independent
+    walks per CU (measured: the dependent LDS round trips of a step need about that many
+    to overlap with two rows per lane, 24 with one)."""
     best = None
     total_rows = sum(int(c) for c in class_rows)
     forced = os.environ.get("GEOREFINE_FUSED_TILING")  # "threads,lanes_per_row": experiments only
@@ -124,11 +126,11 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
         thread_choices, lane_choices = [t_], [min(p_, spr)]
     for threads in thread_choices:
         for p in (lane_choices or range(1, min(spr, threads) + 1)):
-            r = threads // p
+            r = (threads // p) * rows_per_lane
             if gemm:  # see below: at most waves/2 column blocks of 16 rows
                 r = min(r, (threads // 128) * 16)
-                if r == 0:
-                    continue
+            if r == 0:
+                continue
             n_slabs = -(-spr // p)
             if not forced and p > 1 and -(-spr // (p - 1)) == n_slabs:
                 continue  # a narrower slab of the same count wastes fewer lanes; it was scored already
@@ -137,7 +139,7 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
                 waves_wg, col_blocks = threads // 64, -(-r // 16)
                 if col_blocks > waves_wg or -(-8 // (waves_wg // col_blocks)) > 4:
                     continue
-            lanes = p * r
+            lanes = p * -(-r // rows_per_lane)
             lane_eff = spr / (n_slabs * p) * (lanes / threads)
             tiles = sum(-(-int(cnt) // r) for cnt in class_rows if cnt)
             fill = total_rows / (tiles * r)
@@ -145,13 +147,15 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
             lds = lds_fn(p, r, cap)
             if lds > MAX_LDS:
                 continue
-            # the kernels use up to 72 vector registers: 7 waves per SIMD, 28 per CU
-            per_cu = max(1, min(28 // (threads // 64), MAX_LDS // lds))
-            waves = per_cu * threads // 64
+            # A workgroup's waves are dealt round-robin to the CU's four SIMDs.  The one-row
+            # kernels use up to 72 vector registers (7 waves per SIMD), the two-row ones 128 (4).
+            per_simd = -(-(threads // 64) // 4)
+            per_cu = max(1, min((7 if rows_per_lane == 1 else 4) // per_simd, MAX_LDS // lds))
+            walks = per_cu * (threads // 64) * rows_per_lane  # independent 64-lane walks per CU
             slots = cus * per_cu
             rounds = -(-tiles // slots)
             quant = tiles / (rounds * slots)
-            score = lane_eff * fill * quant * min(1.0, waves / 24)
+            score = lane_eff * fill * quant * min(1.0, walks / (WALK_KNEE if rows_per_lane == 2 else 24))
             if best is None or score > best[0] + 1e-9:
                 best = (score, threads, p, r, n_slabs, tiles, cap, lds)
     if best is None:
@@ -207,24 +211,27 @@ class FramePlan:
 
     def tiling(self, m):
         """Host arrays and scalars of a ``grf_fused_tiling`` sized for m activation rows
-        (m = 0: the store sink)."""
+        (m = 0: the store sink).  One row per lane is faster at m <= 2, two rows per lane,
+        which share the activation reads, above (measured on the 17408 x 5120 matrices)."""
+        rows_per_lane = int(os.environ.get("GEOREFINE_FUSED_ROWS_PER_LANE", 1 if m <= 2 else 2))
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
             self.spr, self.class_rows, self._cap,
-            lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_, self.spr))
+            lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_),
+            rows_per_lane=rows_per_lane)
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                 n_tiles=n_tiles, piece_cap=cap), lds=lds)
+                                 n_tiles=n_tiles, piece_cap=cap, rows_per_lane=rows_per_lane), lds=lds)
 
     def gemm_tiling(self):
         """The one tiling every fused GEMM launch uses, whatever its row count: the order in
         which an output element accumulates follows the tiling, so it must not change with M."""
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
             self.spr, self.class_rows, self._cap,
-            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, 128, p_, r_, cap_), gemm=True)
+            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, 128, p_, r_, cap_), gemm=True)
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                 n_tiles=n_tiles, piece_cap=cap), lds=lds)
+                                 n_tiles=n_tiles, piece_cap=cap, rows_per_lane=1), lds=lds)

@@ -39,27 +39,28 @@ constexpr uint32_t kXPad = 8;  // BF16 elements of padding per x segment in LDS 
 
 __host__ __device__ inline uint32_t align_up(uint32_t v, uint32_t a) { return (v + a - 1) / a * a; }
 
-// Per column class the LDS holds one block: the sparse symbol table first (kTabCap
-// 8-byte entries), then the class's lookup bytes.  With the block base in a register
-// the table read needs no further address arithmetic and the lookup read folds the
-// constant table size into its offset field.
-constexpr uint32_t kTabCap = 257;  // up to 256 symbols + the entry a forward scan stops on
-constexpr uint32_t kTabBytes = kTabCap * 8;
+// Per column class the LDS holds one block: the sparse symbol table first (tabn + 1
+// 8-byte entries: the symbols plus the entry a forward scan stops on), then the class's
+// lookup bytes.  With the block base in a register the table read needs no further
+// address arithmetic and the lookup read adds the uniform table size.
+__host__ __device__ inline uint32_t fused_table_bytes(const grf_bctx_fused &f) { return align_up((f.tabn + 1) * 8, 16); }
 
 // byte offsets of the LDS regions; shared by host (size) and device (carve).
 struct FusedLdsLayout {
-  uint32_t blocks, block_pitch, stream, xs, part, total;
+  uint32_t blocks, block_pitch, stream, xs, part, rowsum, total;
   __host__ __device__ FusedLdsLayout(const grf_bctx_fused &f, const grf_fused_tiling &g, uint32_t m) {
     uint32_t at = 0;
     blocks = at;
-    block_pitch = kTabBytes + (1u << f.lognb);
+    block_pitch = fused_table_bytes(f) + (1u << f.lognb);
     at = align_up(at + f.nc * block_pitch, 16);
     stream = at;
     at = align_up(at + g.rows_per_tile * g.piece_cap, 16);
     xs = at;
     at = align_up(at + m * g.lanes_per_row * (f.seg_len + kXPad) * 2, 16);
     part = at;
-    at = align_up(at + g.rows_per_tile * f.segs_per_row * m * 4, 16);
+    at = align_up(at + g.rows_per_tile * g.lanes_per_row * m * 4, 16);
+    rowsum = at;
+    at = align_up(at + g.rows_per_tile * m * 4, 16);
     total = at;
   }
 };
@@ -74,35 +75,8 @@ typedef __attribute__((address_space(3))) v2u32 lds_v2u32;
 __device__ __forceinline__ uint8_t lds_load_u8(uint32_t off) { return *reinterpret_cast<lds_u8 *>(off); }
 
 struct FusedParams {  // uniform values the step needs, kept in scalar registers
-  uint32_t shift, block_pitch;
+  uint32_t shift, block_pitch, table_bytes;
 };
-
-// Slow twin of the step for the rare case that the slot lies beyond the looked-up symbol:
-// scan forward from entry `e` at table address `ta` to the symbol that holds the slot, then
-// update and refill in plain C.  Returns the entry's high word.
-__device__ __forceinline__ uint32_t fused_symbol_scan(uint32_t &state, uint32_t &ip, uint32_t ta, v2u32 e,
-                                                      uint32_t byte0, uint32_t byte1) {
-  const uint32_t slot = state & 0xFFFFu;
-  uint32_t freq = e.x >> 16;
-  freq = freq ? freq : 65536u;
-  while (slot - (e.x & 0xFFFFu) >= freq) {
-    ta += 8;
-    e = *reinterpret_cast<lds_v2u32 *>(ta);
-    freq = e.x >> 16;
-    freq = freq ? freq : 65536u;
-  }
-  uint32_t x = freq * (state >> 16) + (slot - (e.x & 0xFFFFu));
-  if (x < kLow) {
-    x = (x << 8) | byte0;
-    ++ip;
-    if (x < kLow) {
-      x = (x << 8) | byte1;
-      ++ip;
-    }
-  }
-  state = x;
-  return e.y;
-}
 
 // cc * pitch with cc = byte BYTE of `ccw`: one multiply whose operand select does the extraction
 template <int BYTE>
@@ -134,73 +108,153 @@ __device__ __forceinline__ uint32_t fused_lshl3_add(uint32_t a, uint32_t b) {  /
 #endif
 }
 
-// One decode step of the main stream against LDS tables, for the column class held in byte
-// BYTE of `ccw`.  Returns the image of the symbol's bits in the BF16 word (symbol << 5).
+// One decode step of the main stream against LDS tables, in parts so that a lane walking
+// two segments can overlap their LDS round trips.
 //
 // The lookup byte names the symbol that owns the first slot of the slot's bucket.  With
 // buckets finer than almost every symbol, that symbol nearly always owns the slot itself,
-// so the step reads only its entry and assumes it; a lane whose slot lies beyond the entry
-// (a symbol boundary inside the bucket, or the 16-bit frequency field's 0 = 65536) redoes
-// the step with a forward scan.
-template <int BYTE>
-__device__ __forceinline__ uint32_t fused_symbol(uint32_t &state, uint32_t &ip, uint32_t ccw, const FusedParams &q) {
-  // The two possible refill bytes, fetched ahead of need with two byte reads.  (An unaligned
-  // 16-bit LDS read stalls the LDS pipeline for tens of cycles on this hardware; aligned
-  // dwords cost two vector instructions to address and shift.)
-  const uint32_t b0 = lds_load_u8(ip), b1 = lds_load_u8(ip + 1);
-  const uint32_t block = fused_block_offset<BYTE>(ccw, q.block_pitch);
-  const uint32_t bucket = (state & 0xFFFFu) >> q.shift;
-  const uint32_t idx = lds_load_u8(block + bucket + kTabBytes);
-  const uint32_t ta = fused_lshl3_add(idx, block);
-  const v2u32 e0 = *reinterpret_cast<lds_v2u32 *>(ta);
-  const uint32_t state_in = state, ip_in = ip;
-  uint32_t x, ipn, rel;
-  uint64_t miss;  // lanes whose slot lies beyond the entry
-#if defined(__HIP_DEVICE_COMPILE__)
-  uint32_t t;
-  // rel = slot - start; x = freq * (state >> 16) + rel; then up to two refills
-  // (x << 8) | byte while x < 2^23, ip counting the bytes taken.  Operand halves are
-  // addressed with operand selects instead of shifts and masks; v_perm builds (x << 8) | byte.
-  // gfx950 needs two wait states between a VALU write of VCC and a VALU read of it.
-  asm volatile(
-      "v_sub_u32_sdwa %[rel], %[st], %[e0lo] dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_0\n\t"
-      "v_mad_u32_u16 %[x], %[e0lo], %[st], %[rel] op_sel:[1,1,0,0]\n\t"
-      "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
-      "v_perm_b32 %[t], %[x], %[b0], %[sel]\n\t"
-      "s_nop 0\n\t"
-      "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
-      "v_addc_co_u32 %[ipo], vcc, 0, %[ipi], vcc\n\t"
-      "v_cmp_gt_u32 vcc, 0x800000, %[x]\n\t"
-      "v_perm_b32 %[t], %[x], %[b1], %[sel]\n\t"
-      "s_nop 0\n\t"
-      "v_cndmask_b32 %[x], %[x], %[t], vcc\n\t"
-      "v_addc_co_u32 %[ipo], vcc, 0, %[ipo], vcc\n\t"
-      "v_cmp_ge_u32_sdwa %[miss], %[rel], %[e0lo] src0_sel:DWORD src1_sel:WORD_1\n\t"
-      : [x] "=&v"(x), [t] "=&v"(t), [rel] "=&v"(rel), [ipo] "=&v"(ipn), [miss] "=&s"(miss)
-      : [st] "v"(state), [e0lo] "v"(e0.x), [b0] "v"(b0), [b1] "v"(b1), [sel] "s"(0x06050400u),
-        [ipi] "v"(ip)
-      : "vcc");
-#else
-  rel = e0.x + b0 + b1;  // host pass only parses this
-  x = state;
-  ipn = ip;
-  miss = rel;
-#endif
-  state = x;
-  ip = ipn;
-  uint32_t hi = e0.y;
-#if defined(__HIP_DEVICE_COMPILE__)
-  const bool redo = __builtin_amdgcn_inverse_ballot_w64(miss);
-#else
-  const bool redo = miss != 0;
-#endif
-  if (__builtin_expect(redo, 0)) {
-    // the slot lies beyond the entry: redo the step from the saved state with a forward scan
-    state = state_in;
-    ip = ip_in;
-    hi = fused_symbol_scan(state, ip, ta, e0, b0, b1);
+// so the step reads only its entry; a lane whose slot lies beyond the entry (a symbol
+// boundary inside the bucket, or the 16-bit frequency field's 0 = 65536) scans forward
+// before the state update, which all lanes then do together.
+struct StepFetch {
+  uint32_t b0, b1, ta;  // the two possible refill bytes, table address of the entry
+  v2u32 e0;
+};
+
+// A lane's position in one segment: rANS state and LDS byte cursor.  The cursor is kept
+// as j = ip - 2k at step k of a 16-step group, so that a step that takes n bytes subtracts
+// 2 - n and the byte reads carry 2k in their offset field.
+struct Cursor {
+  uint32_t state, j;
+  __device__ __forceinline__ void open(uint32_t state_, uint32_t ip_) {
+    state = state_;
+    j = ip_;
   }
-  return hi;
+  __device__ __forceinline__ void end_group() { j += 32; }  // after 16 steps: j is ip again
+};
+
+// `block` is the LDS offset of the column class's block (fused_block_offset).  The LDS
+// returns data in issue order, so the lookup byte, on which the entry read waits, goes first.
+__device__ __forceinline__ uint32_t fused_fetch_index(uint32_t state, uint32_t block, const FusedParams &q) {
+  const uint32_t bucket = (state & 0xFFFFu) >> q.shift;
+  return lds_load_u8(block + bucket + q.table_bytes);
+}
+// Refill bytes are fetched ahead of need with two byte reads.  (An unaligned 16-bit LDS
+// read stalls the LDS pipeline for tens of cycles on this hardware; aligned dwords, or a
+// register window that follows the cursor, cost more instructions than they save.)
+template <int K>
+__device__ __forceinline__ void fused_fetch_bytes(StepFetch &s, const Cursor &c) {
+  s.b0 = lds_load_u8(c.j + 2 * K);
+  s.b1 = lds_load_u8(c.j + 2 * K + 1);
+}
+__device__ __forceinline__ void fused_fetch_entry(StepFetch &s, uint32_t idx, uint32_t block) {
+  s.ta = fused_lshl3_add(idx, block);
+  s.e0 = *reinterpret_cast<lds_v2u32 *>(s.ta);
+}
+
+// rel = slot - start of the entry; `miss` = the lanes whose slot the entry does not hold
+__device__ __forceinline__ uint32_t fused_locate(uint32_t state, uint32_t e_lo, uint64_t &miss) {
+  uint32_t rel;
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm("v_sub_u32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:WORD_0 src1_sel:WORD_0"
+      : "=v"(rel)
+      : "v"(state), "v"(e_lo));
+  asm("v_cmp_ge_u32_sdwa %0, %1, %2 src0_sel:DWORD src1_sel:WORD_1" : "=s"(miss) : "v"(rel), "v"(e_lo));
+#else
+  rel = (state & 0xFFFFu) - (e_lo & 0xFFFFu);
+  miss = rel >= (e_lo >> 16);
+#endif
+  return rel;
+}
+
+__device__ __forceinline__ bool fused_lane_in(uint64_t mask) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_inverse_ballot_w64(mask);
+#else
+  return mask != 0;
+#endif
+}
+
+// For the lanes that missed: scan forward from the entry at `s.ta` to the one that holds the
+// slot.  An entry with frequency 65536 (field 0, start 0) returns rel = state, so that the
+// update freq16 * (state >> 16) + rel leaves the state as it is.
+__device__ __forceinline__ void fused_scan(uint32_t state, StepFetch &s, uint32_t &rel) {
+  const uint32_t slot = state & 0xFFFFu;
+  uint32_t ta = s.ta;
+  v2u32 e = s.e0;
+  for (;;) {
+    const uint32_t freq = e.x >> 16;
+    rel = slot - (e.x & 0xFFFFu);
+    if (freq == 0) rel = state;
+    if (freq == 0 || rel < freq) break;
+    ta += 8;
+    e = *reinterpret_cast<lds_v2u32 *>(ta);
+  }
+  s.e0 = e;
+}
+
+// state' = freq * (state >> 16) + rel, then the refill: n = 0, 1 or 2 bytes are shifted in
+// while the state is below 2^23.  Without branches or condition registers: the state is
+// below 2^31 and at least 2^7, so c = (24 - clz(state')) >> 3 = 2 - n; the byte selector of
+// v_perm that shifts n bytes in is a window, c bytes up, on the constant 00 01 04 05 06 07.
+__device__ __forceinline__ void fused_advance(Cursor &c, const StepFetch &s, uint32_t rel) {
+  uint32_t x;
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm("v_mad_u32_u16 %0, %1, %2, %3 op_sel:[1,1,0,0]" : "=v"(x) : "v"(s.e0.x), "v"(c.state), "v"(rel));
+#else
+  x = (s.e0.x >> 16) * (c.state >> 16) + rel;
+#endif
+  const uint32_t keep = (24u - (uint32_t)__builtin_clz(x)) >> 3;
+  const uint32_t sel = __builtin_amdgcn_alignbyte(0x00000706u, 0x05040100u, keep);
+  uint32_t bytes;  // first byte above the second, as they enter the state
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm("v_lshl_or_b32 %0, %1, 8, %2" : "=v"(bytes) : "v"(s.b0), "v"(s.b1));
+#else
+  bytes = (s.b0 << 8) | s.b1;
+#endif
+  c.state = __builtin_amdgcn_perm(x, bytes, sel);
+  c.j -= keep;
+}
+
+// One step (number K of its group of 16) of one segment, for the column class held in byte
+// BYTE of `ccw`.  Returns the image of the symbol's bits in the BF16 word (symbol << 5).
+template <int K>
+__device__ __forceinline__ uint32_t fused_symbol(Cursor &c, uint32_t ccw, const FusedParams &q) {
+  const uint32_t block = fused_block_offset<K % 4>(ccw, q.block_pitch);
+  StepFetch s;
+  const uint32_t idx = fused_fetch_index(c.state, block, q);
+  fused_fetch_bytes<K>(s, c);
+  fused_fetch_entry(s, idx, block);
+  uint64_t miss;
+  uint32_t rel = fused_locate(c.state, s.e0.x, miss);
+  if (__builtin_expect(fused_lane_in(miss), 0)) fused_scan(c.state, s, rel);
+  fused_advance(c, s, rel);
+  return s.e0.y;
+}
+
+// The same step for two segments that share their columns (hence the column class).
+template <int K>
+__device__ __forceinline__ void fused_symbol2(Cursor &a, Cursor &b, uint32_t ccw, const FusedParams &q,
+                                              uint32_t &hi_a, uint32_t &hi_b) {
+  const uint32_t block = fused_block_offset<K % 4>(ccw, q.block_pitch);
+  StepFetch sa, sb;
+  const uint32_t idx_a = fused_fetch_index(a.state, block, q);
+  const uint32_t idx_b = fused_fetch_index(b.state, block, q);
+  fused_fetch_bytes<K>(sa, a);
+  fused_fetch_entry(sa, idx_a, block);
+  fused_fetch_bytes<K>(sb, b);
+  fused_fetch_entry(sb, idx_b, block);
+  uint64_t miss_a, miss_b;
+  uint32_t rel_a = fused_locate(a.state, sa.e0.x, miss_a);
+  uint32_t rel_b = fused_locate(b.state, sb.e0.x, miss_b);
+  if (__builtin_expect(fused_lane_in(miss_a | miss_b), 0)) {
+    if (fused_lane_in(miss_a)) fused_scan(a.state, sa, rel_a);
+    if (fused_lane_in(miss_b)) fused_scan(b.state, sb, rel_b);
+  }
+  fused_advance(a, sa, rel_a);
+  fused_advance(b, sb, rel_b);
+  hi_a = sa.e0.y;
+  hi_b = sb.e0.y;
 }
 
 // Sixteen packed 6-bit residuals (12 bytes, MSB first) -> field k, k compile-time.
@@ -234,7 +288,7 @@ __device__ __forceinline__ void fused_load_tables(uint8_t *lds, uint32_t blocks,
   const uint32_t nb = 1u << f.lognb, entries = f.tabn + 1;
   for (uint32_t c = 0; c < f.nc; ++c) {
     const uint4 *src = reinterpret_cast<const uint4 *>(f.lut + ((size_t)cls * f.nc + c) * nb);
-    uint4 *dst = reinterpret_cast<uint4 *>(lds + blocks + c * block_pitch + kTabBytes);
+    uint4 *dst = reinterpret_cast<uint4 *>(lds + blocks + c * block_pitch + fused_table_bytes(f));
     for (uint32_t i = tid; i < nb / 16; i += nthreads) dst[i] = src[i];
     const uint2 *ts = reinterpret_cast<const uint2 *>(f.tab) + ((size_t)cls * f.nc + c) * entries;
     uint2 *td = reinterpret_cast<uint2 *>(lds + blocks + c * block_pitch);
@@ -254,40 +308,6 @@ __device__ __forceinline__ uint32_t fused_stage_piece(uint8_t *lds, uint32_t pie
   return a0;
 }
 
-// A lane's position in its segment: rANS state, LDS cursor, and the registers that hold
-// the packed residuals and column classes of the next 16 symbols.
-struct SegmentWalk {
-  uint32_t state, ip, ip0, gofs, seg;
-  const uint32_t *rawp;
-  const uint4 *ccp;
-  uint32_t n0, n1, n2;
-  uint4 nc4;
-
-  __device__ __forceinline__ void open(const grf_bctx_fused &f, uint32_t seg_, uint32_t piece_off, uint32_t a0,
-                                       uint64_t elem0, uint32_t col0) {
-    seg = seg_;
-    state = f.seg_state[seg];
-    gofs = f.seg_offset[seg];
-    ip0 = piece_off + (gofs - a0);
-    ip = ip0;
-    rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
-    ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
-    n0 = rawp[0];
-    n1 = rawp[1];
-    n2 = rawp[2];
-    nc4 = ccp[0];
-  }
-
-  // Decode symbols [t, t+16) of the segment into eight BF16 pairs (word k in the low half,
-  // k+1 in the high half); loads the registers for the following group meanwhile.
-  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const FusedParams &q, uint32_t (&pair)[8]);
-
-  // the segment must end exactly on the next checkpoint
-  __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
-    return state == f.seg_state[seg + 1] && gofs + (ip - ip0) == f.seg_offset[seg + 1];
-  }
-};
-
 // BF16 word in bits 0..15 (bits above are unspecified): symbol bits | mantissa low 5 bits
 // | sign << 15.  r6 * (1 + 2^10) puts the five mantissa bits at 0..4 and the sign at 15
 // (a 24-bit multiply); the mask drops the copies that land elsewhere.
@@ -295,29 +315,89 @@ __device__ __forceinline__ uint32_t fused_word_bits(uint32_t hi, uint32_t r6) {
   return ((r6 * 0x401u) & 0x801Fu) | hi;
 }
 
-__device__ __forceinline__ void SegmentWalk::decode16(uint32_t t, uint32_t S, const FusedParams &q,
-                                                     uint32_t (&pair)[8]) {
-  Raw6x16 rr;
-  rr.set(n0, n1, n2);
-  const uint32_t cw[4] = {nc4.x, nc4.y, nc4.z, nc4.w};
-  if (t + 16 < S) {
-    const uint32_t *nx = rawp + (t / 16 + 1) * 3;
-    n0 = nx[0];
-    n1 = nx[1];
-    n2 = nx[2];
-    nc4 = ccp[t / 16 + 1];
+// A lane's walk over CH segments (CH = 1 or 2) that cover the same columns of CH rows, in
+// lock step: rANS cursors, plus the registers that hold the packed residuals and the
+// (shared) column classes of the next 16 symbols.  With two segments the column classes
+// are loaded once and the two dependent chains of LDS reads overlap.
+template <int CH>
+struct SegmentWalk {
+  static_assert(CH == 1 || CH == 2, "one or two rows per lane");
+  struct Chain {
+    Cursor c;
+    uint32_t ip0, gofs, seg;
+    const uint32_t *rawp;
+    uint32_t n0, n1, n2;
+  } ch[CH];
+  const uint4 *ccp;
+  uint4 nc4;
+
+  __device__ __forceinline__ void open_columns(const grf_bctx_fused &f, uint32_t col0) {
+    ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
+    nc4 = ccp[0];
   }
-  uint32_t bits[16];
-#define GRF_STEP(k)                                                            \
-  {                                                                            \
-    const uint32_t hi = fused_symbol<(k) % 4>(state, ip, cw[(k) / 4], q);      \
-    bits[k] = fused_word_bits(hi, rr.field<k>());                              \
+  // chain i walks segment `seg`, whose row piece was staged at piece_off from global offset a0
+  __device__ __forceinline__ void open_chain(int i, const grf_bctx_fused &f, uint32_t seg, uint32_t piece_off,
+                                             uint32_t a0, uint64_t elem0) {
+    Chain &c = ch[i];
+    c.seg = seg;
+    c.gofs = f.seg_offset[seg];
+    c.ip0 = piece_off + (c.gofs - a0);
+    c.c.open(f.seg_state[seg], c.ip0);
+    c.rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
+    c.n0 = c.rawp[0];
+    c.n1 = c.rawp[1];
+    c.n2 = c.rawp[2];
   }
-  GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
-  GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
+
+  // Decode symbols [t, t+16) of every segment into eight BF16 pairs each (word k in the
+  // low half, k+1 in the high half); loads the registers for the following group meanwhile.
+  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const FusedParams &q, uint32_t (&pair)[CH][8]) {
+    Raw6x16 rr[CH];
+#pragma unroll
+    for (int i = 0; i < CH; ++i) rr[i].set(ch[i].n0, ch[i].n1, ch[i].n2);
+    const uint32_t cw[4] = {nc4.x, nc4.y, nc4.z, nc4.w};
+    if (t + 16 < S) {
+#pragma unroll
+      for (int i = 0; i < CH; ++i) {
+        const uint32_t *nx = ch[i].rawp + (t / 16 + 1) * 3;
+        ch[i].n0 = nx[0];
+        ch[i].n1 = nx[1];
+        ch[i].n2 = nx[2];
+      }
+      nc4 = ccp[t / 16 + 1];
+    }
+    uint32_t bits[CH][16];
+#define GRF_STEP(k)                                                                   \
+  {                                                                                   \
+    uint32_t hi[2];                                                                   \
+    if constexpr (CH == 1) {                                                          \
+      hi[0] = fused_symbol<k>(ch[0].c, cw[(k) / 4], q);                               \
+    } else {                                                                          \
+      fused_symbol2<k>(ch[0].c, ch[CH - 1].c, cw[(k) / 4], q, hi[0], hi[1]);          \
+    }                                                                                 \
+    _Pragma("unroll") for (int i = 0; i < CH; ++i) bits[i][k] = fused_word_bits(hi[i], rr[i].template field<k>()); \
+  }
+    GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
+    GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
 #undef GRF_STEP
 #pragma unroll
-  for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
-}
+    for (int i = 0; i < CH; ++i) ch[i].c.end_group();
+#pragma unroll
+    for (int i = 0; i < CH; ++i)
+#pragma unroll
+      for (int k = 0; k < 8; ++k) pair[i][k] = __builtin_amdgcn_perm(bits[i][2 * k + 1], bits[i][2 * k], 0x05040100u);
+  }
+
+  // every segment must end exactly on the next checkpoint
+  __device__ __forceinline__ bool ended_on_checkpoints(const grf_bctx_fused &f) const {
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+      const Chain &c = ch[i];
+      ok = ok && c.c.state == f.seg_state[c.seg + 1] && c.gofs + (c.c.j - c.ip0) == f.seg_offset[c.seg + 1];
+    }
+    return ok;
+  }
+};
 
 }  // namespace grf

@@ -36,7 +36,7 @@ struct GemmLdsLayout {
   __host__ __device__ GemmLdsLayout(const grf_bctx_fused &f, const grf_fused_tiling &g, uint32_t m16) {
     uint32_t at = 0;
     blocks = at;
-    block_pitch = grf::kTabBytes + (1u << f.lognb);
+    block_pitch = grf::fused_table_bytes(f) + (1u << f.lognb);
     at = grf::align_up(at + f.nc * block_pitch, 16);
     stream = at;
     at = grf::align_up(at + g.rows_per_tile * g.piece_cap, 16);
@@ -69,7 +69,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
-  const grf::FusedParams q{f.shift, L.block_pitch};
+  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
 
   const uint32_t r = tid / P, p = tid % P;
   const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
@@ -98,15 +98,17 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
     }
     __syncthreads();
     const bool active = row != grf::kNoRow && p < nseg;
-    grf::SegmentWalk w;
+    grf::SegmentWalk<1> w;
     if (active) {
       const uint32_t col0 = (first_seg + p) * S;
-      w.open(f, seg_base + p, piece_off, a0, (uint64_t)row * K + col0, col0);
+      w.open_columns(f, col0);
+      w.open_chain(0, f, seg_base + p, piece_off, a0, (uint64_t)row * K + col0);
     }
     for (uint32_t t = 0; t < S; t += kGroup) {
       if (active) {  // 16 words of this lane's segment -> word tile
-        uint32_t pair[8];
-        w.decode16(t, S, q, pair);
+        uint32_t pairs[1][8];
+        w.decode16(t, S, q, pairs);
+        const uint32_t(&pair)[8] = pairs[0];
         uint2 *dst = reinterpret_cast<uint2 *>(lds + L.wt + r * L.wt_pitch + p * 32);
         dst[0] = make_uint2(pair[0], pair[1]);
         dst[1] = make_uint2(pair[2], pair[3]);
@@ -144,7 +146,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
       }
       __syncthreads();  // tiles are overwritten by the next group
     }
-    if (active && !w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
+    if (active && !w.ended_on_checkpoints(f)) bad |= GRF_ERR_CHECKPOINT;
   }
 
   if (contracts) {
@@ -211,6 +213,8 @@ int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
   if (!frame || !tiling || !x || !y || !error)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemm: null argument");
   if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemm")) return rc;
+  if (tiling->rows_per_lane != 1)
+    return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemm: tiling must have one row per lane");
   if (!m_rows) return GRF_OK;
   if (ldx < frame->cols || ldy < frame->rows || (ldx & 3) || ((uintptr_t)x & 7))
     return grf::set_error(GRF_BAD_ARGUMENT,

@@ -183,8 +183,10 @@ typedef struct grf_bctx_fused {
 
 /* How a launch cuts the frame into workgroups.  A tile is up to rows_per_tile rows of
  * one row class; lane (r, p) of the workgroup walks segment b*lanes_per_row + p of the
- * tile's row r in slab b.  threads >= rows_per_tile*lanes_per_row, a multiple of 64,
- * at most 1024.
+ * tile's row r in slab b -- and, with rows_per_lane = 2 (grf_bctx_gemv and
+ * grf_bctx_fused_decode accept 1 or 2), of row r + ceil(rows_per_tile/2) in lock step;
+ * grf_bctx_gemm takes rows_per_lane = 1.  threads >=
+ * ceil(rows_per_tile/rows_per_lane)*lanes_per_row, a multiple of 64, at most 1024.
  *   tile_rows   u32 [n_tiles*rows_per_tile]  row of each slot, 0xFFFFFFFF = empty
  *   tile_class  u8  [n_tiles]                row class shared by the tile's rows
  *   piece_cap   LDS bytes reserved per row piece of one slab (multiple of 16) */
@@ -194,6 +196,7 @@ typedef struct grf_fused_tiling {
   uint32_t threads;
   uint32_t lanes_per_row, rows_per_tile, n_slabs, n_tiles;
   uint32_t piece_cap;
+  uint32_t rows_per_lane;
 } grf_fused_tiling;
 
 /* Fused decode-GEMV, the slot the reference leaves for "a backend with a fused GEMM"

@@ -69,7 +69,9 @@ def test_tilings_cover_each_row_once_with_one_class_per_tile(shape):
         for tile, cls in zip(rows, t["tile_class"]):
             members = tile[tile != 0xFFFFFFFF]
             assert members.size and np.all(ix["rows"][members] == cls)
-        assert s["threads"] % 64 == 0 and s["lanes_per_row"] * s["rows_per_tile"] <= s["threads"] <= 1024
+        lane_rows = -(-s["rows_per_tile"] // s["rows_per_lane"])
+        assert s["rows_per_lane"] in (1, 2)
+        assert s["threads"] % 64 == 0 and s["lanes_per_row"] * lane_rows <= s["threads"] <= 1024
         assert s["n_slabs"] == -(-plan.spr // s["lanes_per_row"])
         assert t["lds"] <= _fused.MAX_LDS
         # a row piece of any slab fits its LDS slot together with the two bytes read ahead
