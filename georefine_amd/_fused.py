@@ -43,7 +43,9 @@ def sparse_tables(freq, nr, nc, shift):
 
     Entry(column class c, sparse i): low32 = start | (freq & 0xFFFF) << 16 with 0 standing for
     65536, high32 = symbol << 5.  Unused entries are (start 0, freq 65536): a forward scan
-    always stops on them."""
+    always stops on them.  The lookup byte of a bucket is the sparse index of the symbol
+    that owns most of the bucket's slots (the first of them on a tie), which minimises the
+    slots whose lookup has to scan to a neighbouring entry."""
     nz = freq > 0
     tabn = int(nz.sum(axis=1).max())
     if tabn == 0:
@@ -54,7 +56,8 @@ def sparse_tables(freq, nr, nc, shift):
     nb = 1 << lognb
     lut = np.zeros((nr, nc, nb), dtype=np.uint8)
     tab = np.zeros((nr, nc, tabn + 1), dtype=np.uint64)
-    first_slots = (np.arange(nb, dtype=np.int64) << shift)
+    lo_slot = (np.arange(nb, dtype=np.int64) << shift)
+    hi_slot = lo_slot + (1 << shift)
     for rho in range(nr):
         for c in range(nc):
             f = freq[rho * nc + c].astype(np.int64)
@@ -63,14 +66,23 @@ def sparse_tables(freq, nr, nc, shift):
                 continue
             fs = f[syms]
             starts = np.concatenate(([0], np.cumsum(fs)[:-1]))
+            ends = starts + fs
             lo = starts | ((fs & 0xFFFF) << 16)
             hi = syms << 5
             tab[rho, c, :syms.size] = (lo.astype(np.uint64) | (hi.astype(np.uint64) << np.uint64(32)))
-            lut[rho, c] = (np.searchsorted(starts, first_slots, side="right") - 1).astype(np.uint8)
+            first = np.searchsorted(starts, lo_slot, side="right") - 1
+            last = np.searchsorted(starts, hi_slot - 1, side="right") - 1
+            best, best_overlap = first.copy(), np.zeros(nb, dtype=np.int64)
+            for k in range(int((last - first).max()) + 1):
+                cand = np.minimum(first + k, last)
+                overlap = np.minimum(ends[cand], hi_slot) - np.maximum(starts[cand], lo_slot)
+                better = overlap > best_overlap
+                best = np.where(better, cand, best)
+                best_overlap = np.where(better, overlap, best_overlap)
+            lut[rho, c] = best.astype(np.uint8)
     return lut.reshape(nr, nc * nb), tab.reshape(nr, nc * (tabn + 1)), tabn
 
 
-WALK_KNEE = int(os.environ.get("GEOREFINE_FUSED_WALK_KNEE", 32))
 X_PAD = 8
 
 
@@ -107,15 +119,14 @@ def piece_capacity(offsets, rows, spr, p):
     return (longest + 2 + 15) // 16 * 16
 
 
-def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False, rows_per_lane=1):
+def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
     """(threads T, lanes_per_row P, rows_per_tile R, ...): best modelled throughput.
 
     The walk is a chain of dependent steps per lane, so time ~ steps per lane x rounds
     of workgroups, at the speed the resident wave count allows.  The model multiplies
     lane efficiency (idle lanes in the last slab and in a partly filled workgroup), tile
-    fill, how evenly the tiles fill the machine, and a penalty below WALK_KNEE independent
-    walks per CU (measured: the dependent LDS round trips of a step need about that many
-    to overlap with two rows per lane, 24 with one)."""
+    fill, how evenly the tiles fill the machine, and a penalty below 24 waves per CU
+    (measured: the dependent LDS round trips of a step need that many waves to overlap)."""
     best = None
     total_rows = sum(int(c) for c in class_rows)
     forced = os.environ.get("GEOREFINE_FUSED_TILING")  # "threads,lanes_per_row": experiments only
@@ -126,7 +137,7 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False, ro
         thread_choices, lane_choices = [t_], [min(p_, spr)]
     for threads in thread_choices:
         for p in (lane_choices or range(1, min(spr, threads) + 1)):
-            r = (threads // p) * rows_per_lane
+            r = threads // p
             if gemm:  # see below: at most waves/2 column blocks of 16 rows
                 r = min(r, (threads // 128) * 16)
             if r == 0:
@@ -139,7 +150,7 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False, ro
                 waves_wg, col_blocks = threads // 64, -(-r // 16)
                 if col_blocks > waves_wg or -(-8 // (waves_wg // col_blocks)) > 4:
                     continue
-            lanes = p * -(-r // rows_per_lane)
+            lanes = p * r
             lane_eff = spr / (n_slabs * p) * (lanes / threads)
             tiles = sum(-(-int(cnt) // r) for cnt in class_rows if cnt)
             fill = total_rows / (tiles * r)
@@ -147,15 +158,15 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False, ro
             lds = lds_fn(p, r, cap)
             if lds > MAX_LDS:
                 continue
-            # A workgroup's waves are dealt round-robin to the CU's four SIMDs.  The one-row
-            # kernels use up to 72 vector registers (7 waves per SIMD), the two-row ones 128 (4).
+            # A workgroup's waves are dealt round-robin to the CU's four SIMDs; the kernels use
+            # up to 72 vector registers, which allows 7 waves per SIMD.
             per_simd = -(-(threads // 64) // 4)
-            per_cu = max(1, min((7 if rows_per_lane == 1 else 4) // per_simd, MAX_LDS // lds))
-            walks = per_cu * (threads // 64) * rows_per_lane  # independent 64-lane walks per CU
+            per_cu = max(1, min(7 // per_simd, MAX_LDS // lds))
+            waves = per_cu * (threads // 64)
             slots = cus * per_cu
             rounds = -(-tiles // slots)
             quant = tiles / (rounds * slots)
-            score = lane_eff * fill * quant * min(1.0, walks / (WALK_KNEE if rows_per_lane == 2 else 24))
+            score = lane_eff * fill * quant * min(1.0, waves / 24)
             if best is None or score > best[0] + 1e-9:
                 best = (score, threads, p, r, n_slabs, tiles, cap, lds)
     if best is None:
@@ -211,18 +222,15 @@ class FramePlan:
 
     def tiling(self, m):
         """Host arrays and scalars of a ``grf_fused_tiling`` sized for m activation rows
-        (m = 0: the store sink).  One row per lane is faster at m <= 2, two rows per lane,
-        which share the activation reads, above (measured on the 17408 x 5120 matrices)."""
-        rows_per_lane = int(os.environ.get("GEOREFINE_FUSED_ROWS_PER_LANE", 1 if m <= 2 else 2))
+        (m = 0: the store sink)."""
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
             self.spr, self.class_rows, self._cap,
-            lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_),
-            rows_per_lane=rows_per_lane)
+            lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_))
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                 n_tiles=n_tiles, piece_cap=cap, rows_per_lane=rows_per_lane), lds=lds)
+                                 n_tiles=n_tiles, piece_cap=cap), lds=lds)
 
     def gemm_tiling(self):
         """The one tiling every fused GEMM launch uses, whatever its row count: the order in
@@ -234,4 +242,4 @@ class FramePlan:
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                 n_tiles=n_tiles, piece_cap=cap, rows_per_lane=1), lds=lds)
+                                 n_tiles=n_tiles, piece_cap=cap), lds=lds)

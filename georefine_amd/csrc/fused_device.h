@@ -20,10 +20,11 @@
 //     the 16 column classes of the same columns.
 //
 // Symbol lookup: slot>>shift indexes a u8 table giving the sparse index of the
-// symbol that owns the bucket's first slot; that symbol's 8-byte entry is read and
+// symbol that owns most of the bucket's slots; that symbol's 8-byte entry is read and
 // assumed to own the slot.  Entry: low32 = start | (freq & 0xFFFF)<<16 (0 stands for 65536), high32 = symbol<<5
-// (the symbol's bits in the BF16 word).  When a symbol boundary falls inside the
-// bucket before the slot, a forward scan over the following entries finishes the search.
+// (the symbol's bits in the BF16 word).  When a symbol boundary inside the bucket
+// separates the slot from that symbol, a scan over the neighbouring entries finishes
+// the search.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -108,14 +109,13 @@ __device__ __forceinline__ uint32_t fused_lshl3_add(uint32_t a, uint32_t b) {  /
 #endif
 }
 
-// One decode step of the main stream against LDS tables, in parts so that a lane walking
-// two segments can overlap their LDS round trips.
+// One decode step of the main stream against LDS tables.
 //
-// The lookup byte names the symbol that owns the first slot of the slot's bucket.  With
+// The lookup byte names the symbol that owns most slots of the slot's bucket.  With
 // buckets finer than almost every symbol, that symbol nearly always owns the slot itself,
-// so the step reads only its entry; a lane whose slot lies beyond the entry (a symbol
-// boundary inside the bucket, or the 16-bit frequency field's 0 = 65536) scans forward
-// before the state update, which all lanes then do together.
+// so the step reads only its entry; a lane whose slot lies outside the entry (a symbol
+// boundary inside the bucket, or the 16-bit frequency field's 0 = 65536) scans to the
+// neighbouring entries before the state update, which all lanes then do together.
 struct StepFetch {
   uint32_t b0, b1, ta;  // the two possible refill bytes, table address of the entry
   v2u32 e0;
@@ -175,9 +175,9 @@ __device__ __forceinline__ bool fused_lane_in(uint64_t mask) {
 #endif
 }
 
-// For the lanes that missed: scan forward from the entry at `s.ta` to the one that holds the
-// slot.  An entry with frequency 65536 (field 0, start 0) returns rel = state, so that the
-// update freq16 * (state >> 16) + rel leaves the state as it is.
+// For the lanes that missed: scan from the entry at `s.ta`, backward or forward, to the one
+// that holds the slot.  An entry with frequency 65536 (field 0, start 0) returns rel = state,
+// so that the update freq16 * (state >> 16) + rel leaves the state as it is.
 __device__ __forceinline__ void fused_scan(uint32_t state, StepFetch &s, uint32_t &rel) {
   const uint32_t slot = state & 0xFFFFu;
   uint32_t ta = s.ta;
@@ -187,7 +187,7 @@ __device__ __forceinline__ void fused_scan(uint32_t state, StepFetch &s, uint32_
     rel = slot - (e.x & 0xFFFFu);
     if (freq == 0) rel = state;
     if (freq == 0 || rel < freq) break;
-    ta += 8;
+    ta += (int32_t)rel < 0 ? -8 : 8;
     e = *reinterpret_cast<lds_v2u32 *>(ta);
   }
   s.e0 = e;
@@ -230,31 +230,6 @@ __device__ __forceinline__ uint32_t fused_symbol(Cursor &c, uint32_t ccw, const 
   if (__builtin_expect(fused_lane_in(miss), 0)) fused_scan(c.state, s, rel);
   fused_advance(c, s, rel);
   return s.e0.y;
-}
-
-// The same step for two segments that share their columns (hence the column class).
-template <int K>
-__device__ __forceinline__ void fused_symbol2(Cursor &a, Cursor &b, uint32_t ccw, const FusedParams &q,
-                                              uint32_t &hi_a, uint32_t &hi_b) {
-  const uint32_t block = fused_block_offset<K % 4>(ccw, q.block_pitch);
-  StepFetch sa, sb;
-  const uint32_t idx_a = fused_fetch_index(a.state, block, q);
-  const uint32_t idx_b = fused_fetch_index(b.state, block, q);
-  fused_fetch_bytes<K>(sa, a);
-  fused_fetch_entry(sa, idx_a, block);
-  fused_fetch_bytes<K>(sb, b);
-  fused_fetch_entry(sb, idx_b, block);
-  uint64_t miss_a, miss_b;
-  uint32_t rel_a = fused_locate(a.state, sa.e0.x, miss_a);
-  uint32_t rel_b = fused_locate(b.state, sb.e0.x, miss_b);
-  if (__builtin_expect(fused_lane_in(miss_a | miss_b), 0)) {
-    if (fused_lane_in(miss_a)) fused_scan(a.state, sa, rel_a);
-    if (fused_lane_in(miss_b)) fused_scan(b.state, sb, rel_b);
-  }
-  fused_advance(a, sa, rel_a);
-  fused_advance(b, sb, rel_b);
-  hi_a = sa.e0.y;
-  hi_b = sb.e0.y;
 }
 
 // Sixteen packed 6-bit residuals (12 bytes, MSB first) -> field k, k compile-time.
@@ -315,88 +290,58 @@ __device__ __forceinline__ uint32_t fused_word_bits(uint32_t hi, uint32_t r6) {
   return ((r6 * 0x401u) & 0x801Fu) | hi;
 }
 
-// A lane's walk over CH segments (CH = 1 or 2) that cover the same columns of CH rows, in
-// lock step: rANS cursors, plus the registers that hold the packed residuals and the
-// (shared) column classes of the next 16 symbols.  With two segments the column classes
-// are loaded once and the two dependent chains of LDS reads overlap.
-template <int CH>
+// A lane's walk over one segment: rANS cursor, plus the registers that hold the packed
+// residuals and the column classes of the next 16 symbols.
 struct SegmentWalk {
-  static_assert(CH == 1 || CH == 2, "one or two rows per lane");
-  struct Chain {
-    Cursor c;
-    uint32_t ip0, gofs, seg;
-    const uint32_t *rawp;
-    uint32_t n0, n1, n2;
-  } ch[CH];
+  Cursor c;
+  uint32_t ip0, gofs, seg;
+  const uint32_t *rawp;
   const uint4 *ccp;
+  uint32_t n0, n1, n2;
   uint4 nc4;
 
-  __device__ __forceinline__ void open_columns(const grf_bctx_fused &f, uint32_t col0) {
+  // walks segment `seg_`, whose row piece was staged at piece_off from global offset a0;
+  // elem0 / col0: the segment's first element / column
+  __device__ __forceinline__ void open(const grf_bctx_fused &f, uint32_t seg_, uint32_t piece_off, uint32_t a0,
+                                       uint64_t elem0, uint32_t col0) {
+    seg = seg_;
+    gofs = f.seg_offset[seg];
+    ip0 = piece_off + (gofs - a0);
+    c.open(f.seg_state[seg], ip0);
+    rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
     ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
+    n0 = rawp[0];
+    n1 = rawp[1];
+    n2 = rawp[2];
     nc4 = ccp[0];
   }
-  // chain i walks segment `seg`, whose row piece was staged at piece_off from global offset a0
-  __device__ __forceinline__ void open_chain(int i, const grf_bctx_fused &f, uint32_t seg, uint32_t piece_off,
-                                             uint32_t a0, uint64_t elem0) {
-    Chain &c = ch[i];
-    c.seg = seg;
-    c.gofs = f.seg_offset[seg];
-    c.ip0 = piece_off + (c.gofs - a0);
-    c.c.open(f.seg_state[seg], c.ip0);
-    c.rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
-    c.n0 = c.rawp[0];
-    c.n1 = c.rawp[1];
-    c.n2 = c.rawp[2];
-  }
 
-  // Decode symbols [t, t+16) of every segment into eight BF16 pairs each (word k in the
-  // low half, k+1 in the high half); loads the registers for the following group meanwhile.
-  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const FusedParams &q, uint32_t (&pair)[CH][8]) {
-    Raw6x16 rr[CH];
-#pragma unroll
-    for (int i = 0; i < CH; ++i) rr[i].set(ch[i].n0, ch[i].n1, ch[i].n2);
+  // Decode symbols [t, t+16) of the segment into eight BF16 pairs (word k in the low half,
+  // k+1 in the high half); loads the registers for the following group meanwhile.
+  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const FusedParams &q, uint32_t (&pair)[8]) {
+    Raw6x16 rr;
+    rr.set(n0, n1, n2);
     const uint32_t cw[4] = {nc4.x, nc4.y, nc4.z, nc4.w};
     if (t + 16 < S) {
-#pragma unroll
-      for (int i = 0; i < CH; ++i) {
-        const uint32_t *nx = ch[i].rawp + (t / 16 + 1) * 3;
-        ch[i].n0 = nx[0];
-        ch[i].n1 = nx[1];
-        ch[i].n2 = nx[2];
-      }
+      const uint32_t *nx = rawp + (t / 16 + 1) * 3;
+      n0 = nx[0];
+      n1 = nx[1];
+      n2 = nx[2];
       nc4 = ccp[t / 16 + 1];
     }
-    uint32_t bits[CH][16];
-#define GRF_STEP(k)                                                                   \
-  {                                                                                   \
-    uint32_t hi[2];                                                                   \
-    if constexpr (CH == 1) {                                                          \
-      hi[0] = fused_symbol<k>(ch[0].c, cw[(k) / 4], q);                               \
-    } else {                                                                          \
-      fused_symbol2<k>(ch[0].c, ch[CH - 1].c, cw[(k) / 4], q, hi[0], hi[1]);          \
-    }                                                                                 \
-    _Pragma("unroll") for (int i = 0; i < CH; ++i) bits[i][k] = fused_word_bits(hi[i], rr[i].template field<k>()); \
-  }
+    uint32_t bits[16];
+#define GRF_STEP(k) bits[k] = fused_word_bits(fused_symbol<k>(c, cw[(k) / 4], q), rr.field<k>());
     GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
     GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
 #undef GRF_STEP
+    c.end_group();
 #pragma unroll
-    for (int i = 0; i < CH; ++i) ch[i].c.end_group();
-#pragma unroll
-    for (int i = 0; i < CH; ++i)
-#pragma unroll
-      for (int k = 0; k < 8; ++k) pair[i][k] = __builtin_amdgcn_perm(bits[i][2 * k + 1], bits[i][2 * k], 0x05040100u);
+    for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
   }
 
-  // every segment must end exactly on the next checkpoint
-  __device__ __forceinline__ bool ended_on_checkpoints(const grf_bctx_fused &f) const {
-    bool ok = true;
-#pragma unroll
-    for (int i = 0; i < CH; ++i) {
-      const Chain &c = ch[i];
-      ok = ok && c.c.state == f.seg_state[c.seg + 1] && c.gofs + (c.c.j - c.ip0) == f.seg_offset[c.seg + 1];
-    }
-    return ok;
+  // the segment must end exactly on the next checkpoint
+  __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
+    return c.state == f.seg_state[seg + 1] && gofs + (c.j - ip0) == f.seg_offset[seg + 1];
   }
 };
 

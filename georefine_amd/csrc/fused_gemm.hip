@@ -98,17 +98,15 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
     }
     __syncthreads();
     const bool active = row != grf::kNoRow && p < nseg;
-    grf::SegmentWalk<1> w;
+    grf::SegmentWalk w;
     if (active) {
       const uint32_t col0 = (first_seg + p) * S;
-      w.open_columns(f, col0);
-      w.open_chain(0, f, seg_base + p, piece_off, a0, (uint64_t)row * K + col0);
+      w.open(f, seg_base + p, piece_off, a0, (uint64_t)row * K + col0, col0);
     }
     for (uint32_t t = 0; t < S; t += kGroup) {
       if (active) {  // 16 words of this lane's segment -> word tile
-        uint32_t pairs[1][8];
-        w.decode16(t, S, q, pairs);
-        const uint32_t(&pair)[8] = pairs[0];
+        uint32_t pair[8];
+        w.decode16(t, S, q, pair);
         uint2 *dst = reinterpret_cast<uint2 *>(lds + L.wt + r * L.wt_pitch + p * 32);
         dst[0] = make_uint2(pair[0], pair[1]);
         dst[1] = make_uint2(pair[2], pair[3]);
@@ -146,7 +144,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
       }
       __syncthreads();  // tiles are overwritten by the next group
     }
-    if (active && !w.ended_on_checkpoints(f)) bad |= GRF_ERR_CHECKPOINT;
+    if (active && !w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
   }
 
   if (contracts) {
@@ -213,8 +211,6 @@ int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
   if (!frame || !tiling || !x || !y || !error)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemm: null argument");
   if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemm")) return rc;
-  if (tiling->rows_per_lane != 1)
-    return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemm: tiling must have one row per lane");
   if (!m_rows) return GRF_OK;
   if (ldx < frame->cols || ldy < frame->rows || (ldx & 3) || ((uintptr_t)x & 7))
     return grf::set_error(GRF_BAD_ARGUMENT,

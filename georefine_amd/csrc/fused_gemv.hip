@@ -38,10 +38,7 @@ __device__ __forceinline__ uint16_t round_bf16(float v) {
   return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
 }
 
-// CH rows per lane: lane (r, p) walks segment b*P + p of the tile's rows r + c*RL,
-// c < CH, RL = ceil(R / CH), in slab b.  The walks of a lane share column classes and
-// activations.
-template <int M, bool STORE, int CH>
+template <int M, bool STORE>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_bctx_fused f, grf_fused_tiling g,
                                                                             const uint16_t *x, uint32_t ldx,
                                                                             uint16_t *y, uint32_t ldy,
@@ -50,19 +47,14 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   extern __shared__ __align__(16) uint8_t lds[];
   const FusedLdsLayout L(f, g, STORE ? 0 : M);
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
-  const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, RL = (R + CH - 1) / CH, S = f.seg_len, K = f.cols;
+  const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
 
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
 
   const uint32_t r = tid / P, p = tid % P;
-  uint32_t slot[CH], row[CH];  // tile slots and matrix rows of this lane; rows fill a tile from slot 0
-#pragma unroll
-  for (int c = 0; c < CH; ++c) {
-    slot[c] = r + c * RL;
-    row[c] = (r < RL && slot[c] < R) ? g.tile_rows[tile * R + slot[c]] : grf::kNoRow;
-  }
+  const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
   uint16_t *xs = reinterpret_cast<uint16_t *>(lds + L.xs);
   const uint32_t xpitch = S + grf::kXPad;
   const uint32_t width = P * S;
@@ -84,47 +76,29 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
     }
     const uint32_t first_seg = b * P;
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
-    uint32_t a0[CH], base[CH], piece[CH];
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      a0[c] = base[c] = 0;
-      piece[c] = L.stream + slot[c] * g.piece_cap;
-      if (row[c] != grf::kNoRow) {
-        base[c] = row[c] * f.segs_per_row + first_seg;
-        a0[c] = grf::fused_stage_piece(lds, piece[c], f, base[c], nseg, p, P);
-      }
+    uint32_t a0 = 0, seg_base = 0;
+    const uint32_t piece_off = L.stream + r * g.piece_cap;
+    if (row != grf::kNoRow) {
+      seg_base = row * f.segs_per_row + first_seg;
+      a0 = grf::fused_stage_piece(lds, piece_off, f, seg_base, nseg, p, P);
     }
     __syncthreads();
-    if (row[0] != grf::kNoRow && p < nseg) {
+    if (row != grf::kNoRow && p < nseg) {
       const uint32_t col0 = (first_seg + p) * S;
-      grf::SegmentWalk<CH> w;
-      w.open_columns(f, col0);
-      uint64_t elem[CH];
-      bool live[CH];  // a lane without a second row walks its first one twice and drops the copy
-#pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        live[c] = row[c] != grf::kNoRow;
-        const int u = live[c] ? c : 0;
-        elem[c] = (uint64_t)row[u] * K + col0;
-        w.open_chain(c, f, base[u] + p, piece[u], a0[u], elem[c]);
-      }
+      const uint64_t elem0 = (uint64_t)row * K + col0;
+      grf::SegmentWalk w;
+      w.open(f, seg_base + p, piece_off, a0, elem0, col0);
       const uint16_t *xr = xs + p * xpitch;
-      float acc[CH][M];
+      float acc[M];
 #pragma unroll
-      for (int c = 0; c < CH; ++c)
-#pragma unroll
-        for (int m = 0; m < M; ++m) acc[c][m] = 0.f;
+      for (int m = 0; m < M; ++m) acc[m] = 0.f;
       for (uint32_t t = 0; t < S; t += 16) {
-        uint32_t pair[CH][8];
+        uint32_t pair[8];
         w.decode16(t, S, q, pair);
         if (STORE) {
-#pragma unroll
-          for (int c = 0; c < CH; ++c) {
-            if (!live[c]) continue;
-            uint4 *dst = reinterpret_cast<uint4 *>(out + elem[c] + t);
-            dst[0] = make_uint4(pair[c][0], pair[c][1], pair[c][2], pair[c][3]);
-            dst[1] = make_uint4(pair[c][4], pair[c][5], pair[c][6], pair[c][7]);
-          }
+          uint4 *dst = reinterpret_cast<uint4 *>(out + elem0 + t);
+          dst[0] = make_uint4(pair[0], pair[1], pair[2], pair[3]);
+          dst[1] = make_uint4(pair[4], pair[5], pair[6], pair[7]);
         } else {
 #pragma unroll
           for (int m = 0; m < M; ++m) {
@@ -132,20 +106,15 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
             const uint4 xa = xm[0], xb = xm[1];
             const uint32_t xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
 #pragma unroll
-            for (int k = 0; k < 8; ++k)
-#pragma unroll
-              for (int c = 0; c < CH; ++c) acc[c][m] = dot2_bf16(pair[c][k], xv[k], acc[c][m]);
+            for (int k = 0; k < 8; ++k) acc[m] = dot2_bf16(pair[k], xv[k], acc[m]);
           }
         }
       }
       if (!STORE) {
 #pragma unroll
-        for (int c = 0; c < CH; ++c)
-#pragma unroll
-          for (int m = 0; m < M; ++m)
-            if (live[c]) part[(slot[c] * P + p) * M + m] = acc[c][m];
+        for (int m = 0; m < M; ++m) part[(r * P + p) * M + m] = acc[m];
       }
-      if (!w.ended_on_checkpoints(f)) bad |= GRF_ERR_CHECKPOINT;
+      if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
     }
     if (!STORE) {  // fold this slab's partials into the running row sums, in segment order
       __syncthreads();
@@ -185,9 +154,7 @@ int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const 
   if (f.seg_len == 0 || f.seg_len % 16 || (uint64_t)f.seg_len * f.segs_per_row != f.cols)
     return bad("segment length must be a multiple of 16 that divides the row length");
   if (!g.threads || g.threads % 64 || g.threads > (uint32_t)grf::kFusedMaxThreads) return bad("thread count");
-  if (g.rows_per_lane != 1 && g.rows_per_lane != 2) return bad("rows per lane");
-  if (!g.lanes_per_row || !g.rows_per_tile ||
-      g.lanes_per_row * ((g.rows_per_tile + g.rows_per_lane - 1) / g.rows_per_lane) > g.threads)
+  if (!g.lanes_per_row || !g.rows_per_tile || g.lanes_per_row * g.rows_per_tile > g.threads)
     return bad("tile does not fit one workgroup");
   if (g.n_slabs != (f.segs_per_row + g.lanes_per_row - 1) / g.lanes_per_row) return bad("slab count mismatch");
   if (f.nc == 0 || f.nc > 16 || (f.nc & (f.nc - 1))) return bad("column class count");
@@ -202,12 +169,12 @@ int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const 
 namespace {
 using grf::check_fused_frame;
 
-template <int M, bool STORE, int CH>
-int launch_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint16_t *y,
-                uint32_t ldy, const uint16_t *bias, uint16_t *out, int32_t *error, hipStream_t s) {
+template <int M, bool STORE>
+int launch(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint16_t *y,
+           uint32_t ldy, const uint16_t *bias, uint16_t *out, int32_t *error, hipStream_t s) {
   const FusedLdsLayout L(f, g, STORE ? 0 : M);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
-  auto kernel = fused_walk_kernel<M, STORE, CH>;
+  auto kernel = fused_walk_kernel<M, STORE>;
   if (L.total > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
@@ -217,13 +184,6 @@ int launch_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
   return GRF_OK;
-}
-
-template <int M, bool STORE>
-int launch(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint16_t *y,
-           uint32_t ldy, const uint16_t *bias, uint16_t *out, int32_t *error, hipStream_t s) {
-  return g.rows_per_lane == 2 ? launch_rows<M, STORE, 2>(f, g, x, ldx, y, ldy, bias, out, error, s)
-                              : launch_rows<M, STORE, 1>(f, g, x, ldx, y, ldy, bias, out, error, s);
 }
 
 }  // namespace

@@ -159,8 +159,9 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  * length, and per-row-class lookup tables laid out for LDS:
  *   seg_state / seg_offset  u32 [rows*segs_per_row + 1]; the extra last entry is
  *                           (2^23, main_n_bytes)
- *   lut         u8  [nr][nc << lognb]        lognb = 16 - shift; sparse index of the
- *                                            symbol owning the bucket's first slot
+ *   lut         u8  [nr][nc << lognb]        lognb = 16 - shift; sparse index of a
+ *                                            symbol with slots in the bucket (best: the
+ *                                            one owning most of them)
  *   tab         u64 [nr][nc][tabn+1]         entry(cc, sparse): low32 = start |
  *                                            (freq & 0xFFFF)<<16 (0 stands for 65536),
  *                                            high32 = symbol<<5; unused entries: 0
@@ -183,10 +184,8 @@ typedef struct grf_bctx_fused {
 
 /* How a launch cuts the frame into workgroups.  A tile is up to rows_per_tile rows of
  * one row class; lane (r, p) of the workgroup walks segment b*lanes_per_row + p of the
- * tile's row r in slab b -- and, with rows_per_lane = 2 (grf_bctx_gemv and
- * grf_bctx_fused_decode accept 1 or 2), of row r + ceil(rows_per_tile/2) in lock step;
- * grf_bctx_gemm takes rows_per_lane = 1.  threads >=
- * ceil(rows_per_tile/rows_per_lane)*lanes_per_row, a multiple of 64, at most 1024.
+ * tile's row r in slab b.  threads >= rows_per_tile*lanes_per_row, a multiple of 64,
+ * at most 1024.
  *   tile_rows   u32 [n_tiles*rows_per_tile]  row of each slot, 0xFFFFFFFF = empty
  *   tile_class  u8  [n_tiles]                row class shared by the tile's rows
  *   piece_cap   LDS bytes reserved per row piece of one slab (multiple of 16) */
@@ -196,7 +195,6 @@ typedef struct grf_fused_tiling {
   uint32_t threads;
   uint32_t lanes_per_row, rows_per_tile, n_slabs, n_tiles;
   uint32_t piece_cap;
-  uint32_t rows_per_lane;
 } grf_fused_tiling;
 
 /* Fused decode-GEMV, the slot the reference leaves for "a backend with a fused GEMM"

@@ -18,8 +18,8 @@ def _plan(words, nr=16, nc=4, segment=64):
 
 
 def emulate_lookup(plan, rho, cc, slots):
-    """The device step's symbol search, in numpy: bucket -> sparse index, then scan forward
-    while the slot lies beyond the entry (frequency field 0 stands for 65536)."""
+    """The device step's symbol search, in numpy: bucket -> sparse index, then scan backward
+    or forward while the slot lies outside the entry (frequency field 0 stands for 65536)."""
     nb = 1 << plan.lognb
     lut = plan.lut[rho].reshape(plan.nc, nb)[cc]
     tab = plan.tab[rho].reshape(plan.nc, plan.tabn + 1)[cc]
@@ -28,10 +28,10 @@ def emulate_lookup(plan, rho, cc, slots):
     freq = np.where(freq == 0, 65536, freq)
     idx = lut[slots >> plan.shift].astype(np.int64)
     for _ in range(plan.tabn + 1):
-        beyond = slots - start[idx] >= freq[idx]
-        if not beyond.any():
+        before, beyond = slots < start[idx], slots - start[idx] >= freq[idx]
+        if not (before | beyond).any():
             break
-        idx = np.where(beyond, idx + 1, idx)
+        idx = np.where(before, idx - 1, np.where(beyond, idx + 1, idx))
     return hi[idx] >> 5, start[idx], freq[idx]
 
 
@@ -69,9 +69,7 @@ def test_tilings_cover_each_row_once_with_one_class_per_tile(shape):
         for tile, cls in zip(rows, t["tile_class"]):
             members = tile[tile != 0xFFFFFFFF]
             assert members.size and np.all(ix["rows"][members] == cls)
-        lane_rows = -(-s["rows_per_tile"] // s["rows_per_lane"])
-        assert s["rows_per_lane"] in (1, 2)
-        assert s["threads"] % 64 == 0 and s["lanes_per_row"] * lane_rows <= s["threads"] <= 1024
+        assert s["threads"] % 64 == 0 and s["lanes_per_row"] * s["rows_per_tile"] <= s["threads"] <= 1024
         assert s["n_slabs"] == -(-plan.spr // s["lanes_per_row"])
         assert t["lds"] <= _fused.MAX_LDS
         # a row piece of any slab fits its LDS slot together with the two bytes read ahead
