@@ -117,7 +117,7 @@ __device__ __forceinline__ uint32_t fused_lshl3_add(uint32_t a, uint32_t b) {  /
 // boundary inside the bucket, or the 16-bit frequency field's 0 = 65536) scans to the
 // neighbouring entries before the state update, which all lanes then do together.
 struct StepFetch {
-  uint32_t b0, b1, ta;  // the two possible refill bytes, table address of the entry
+  uint32_t bytes, ta;  // the two possible refill bytes (first << 8 | second), table address of the entry
   v2u32 e0;
 };
 
@@ -144,8 +144,9 @@ __device__ __forceinline__ uint32_t fused_fetch_index(uint32_t state, uint32_t b
 // register window that follows the cursor, cost more instructions than they save.)
 template <int K>
 __device__ __forceinline__ void fused_fetch_bytes(StepFetch &s, const Cursor &c) {
-  s.b0 = lds_load_u8(c.j + 2 * K);
-  s.b1 = lds_load_u8(c.j + 2 * K + 1);
+  // first byte above the second, as they enter the state (a byte permute: only the low
+  // byte of either register is looked at)
+  s.bytes = __builtin_amdgcn_perm(lds_load_u8(c.j + 2 * K), lds_load_u8(c.j + 2 * K + 1), 0x0c0c0400u);
 }
 __device__ __forceinline__ void fused_fetch_entry(StepFetch &s, uint32_t idx, uint32_t block) {
   s.ta = fused_lshl3_add(idx, block);
@@ -206,13 +207,7 @@ __device__ __forceinline__ void fused_advance(Cursor &c, const StepFetch &s, uin
 #endif
   const uint32_t keep = (24u - (uint32_t)__builtin_clz(x)) >> 3;
   const uint32_t sel = __builtin_amdgcn_alignbyte(0x00000706u, 0x05040100u, keep);
-  uint32_t bytes;  // first byte above the second, as they enter the state
-#if defined(__HIP_DEVICE_COMPILE__)
-  asm("v_lshl_or_b32 %0, %1, 8, %2" : "=v"(bytes) : "v"(s.b0), "v"(s.b1));
-#else
-  bytes = (s.b0 << 8) | s.b1;
-#endif
-  c.state = __builtin_amdgcn_perm(x, bytes, sel);
+  c.state = __builtin_amdgcn_perm(x, s.bytes, sel);
   c.j -= keep;
 }
 
@@ -322,12 +317,13 @@ struct SegmentWalk {
     Raw6x16 rr;
     rr.set(n0, n1, n2);
     const uint32_t cw[4] = {nc4.x, nc4.y, nc4.z, nc4.w};
-    if (t + 16 < S) {
-      const uint32_t *nx = rawp + (t / 16 + 1) * 3;
+    {  // the last group loads itself again rather than branch around the loads
+      const uint32_t next = min(t / 16 + 1, S / 16 - 1);
+      const uint32_t *nx = rawp + next * 3;
       n0 = nx[0];
       n1 = nx[1];
       n2 = nx[2];
-      nc4 = ccp[t / 16 + 1];
+      nc4 = ccp[next];
     }
     uint32_t bits[16];
 #define GRF_STEP(k) bits[k] = fused_word_bits(fused_symbol<k>(c, cw[(k) / 4], q), rr.field<k>());
