@@ -61,7 +61,7 @@ def algorithmic_bytes(t, m):
     n = lambda k: b[k].numel() * b[k].element_size()
     rows, cols = t.shape
     payload = t._main_bytes + n("residual_stream")
-    _, tile_rows, tile_class, _ = t._tiling(m)
+    _, tile_rows, tile_class, _ = t._tiling(m) if m <= 8 else t._gemm_tiling()
     index = (n("fused_seg_state") + n("fused_seg_offset") + tile_rows.numel() * tile_rows.element_size()
              + tile_class.numel() * tile_class.element_size())
     tables = n("fused_lut") + n("fused_tab")
@@ -103,7 +103,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--batch", type=int, default=1, help="activation rows per GEMV (1..8)")
+    ap.add_argument("--batch", type=int, default=1, help="activation rows; 1..8 run the fused GEMV (the headline figure is batch 1), more the fused GEMM")
     ap.add_argument("--segment", type=int, default=0, help="fused segment length (0 = automatic)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--only", default="", help="comma list of gate,up,down (profiling aid)")
@@ -138,7 +138,7 @@ def main():
             sys.exit(f"bench.py: {name} is not eligible for the fused kernel: {tensors[name].fused_reason}")
         log(f"{name}: {rows}x{cols} mode {tensors[name].mode} frame {len(frame)} B "
             f"({8 * len(frame) / w.size:.3f} bit/weight) encode {t1 - t0:.1f}s index+upload {t2 - t1:.1f}s "
-            f"plan {tensors[name].fused_plan} tiling {tensors[name]._tiling(args.batch)[3]}")
+            f"plan {tensors[name].fused_plan} tiling {(tensors[name]._tiling(args.batch) if args.batch <= 8 else tensors[name]._gemm_tiling())[3]}")
         frames[name] = frame
         words_of[name] = w
     log(f"setup {time.perf_counter() - t_setup:.1f}s")
@@ -215,7 +215,7 @@ def main():
         "vs_baseline": None,
         "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
         "data": "synthetic",
-        "config": {"workload": "fused decode-GEMV, batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
+        "config": {"workload": "fused decode-" + ("GEMV" if m <= 8 else "GEMM") + ", batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
                                "BCTX (16,4) frames, residuals resident in packed 6-bit form" % m,
                    "batch": m, "matrices": names,
                    "segment": tensors[names[0]].fused_plan["seg_len"]},
@@ -228,7 +228,7 @@ def main():
                             "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in names},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "kernel": f"fused_walk_kernel<{m},false> on {dom}"},
+                     "kernel": (f"fused_walk_kernel<{m},false>" if m <= 8 else "fused_gemm_kernel") + f" on {dom}"},
     }
     if not args.no_cpu_baseline:
         log("timing the CPU oracle on whole frames ...")

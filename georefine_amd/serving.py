@@ -132,3 +132,197 @@ class PredictiveContextTensor:
     def linear(self, x, bias=None, *, check=False, batch_invariant=False):
         """Decode against the references, then the dense matmul (no fused PPCX kernel yet)."""
         return torch.nn.functional.linear(x, self.decode(check=check), bias)
+
+
+# ----------------------------------------------------------------------------- loader
+
+def _parent_and_attr(model, dotted):
+    parent_name, _, attr = dotted.rpartition(".")
+    return (model.get_submodule(parent_name) if parent_name else model), attr
+
+
+def _runtime_dtype(model, name, parameter, requested):
+    """The requested dtype, except parameters a module pins to fp32 by name pattern
+    (``_keep_in_fp32_modules_strict``; GCR/bitexact_context_serving.py:76-89)."""
+    from fnmatch import fnmatchcase
+    if not parameter.is_floating_point():
+        return parameter.dtype
+    patterns = []
+    for _, module in model.named_modules():
+        patterns.extend(str(p) for p in (getattr(module, "_keep_in_fp32_modules_strict", ()) or ()))
+        if requested == torch.float16:
+            patterns.extend(str(p) for p in (getattr(module, "_keep_in_fp32_modules", ()) or ()))
+    return torch.float32 if any(fnmatchcase(name, p) for p in patterns) else requested
+
+
+def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
+                    tensor_factory=None, host_decoder=None, loader_workers=1, batch_invariant=False,
+                    log=print, progress_callback=None):
+    """Build ``model_factory()`` on the meta device and fill it from a BCTX package without
+    ever holding a dense checkpoint: returns ``(model, receipt)``.
+
+    The procedure and its checks are the reference loader's
+    (GCR/bitexact_context_serving.py:409-712): every ``nn.Linear`` / ``nn.Embedding`` whose
+    weight has a receipt keeps the frame resident on ``device`` behind ``BctxLinear`` /
+    ``BctxEmbedding`` (one ``tensor_factory(frame, stride=, device=)`` call each, from
+    ``loader_workers`` threads); the object's geometry, decoded-source digest, frame digest
+    and ``resident_bytes`` are checked against the receipt.  Every other parameter and every
+    linear bias is decoded on the host, digest checked, and installed dense.  The model must
+    end with no meta tensor left.  What this loader leaves to the caller is the model
+    construction itself (the reference reads a Transformers config and generation config
+    from the package's sidecars): ``model_factory`` returns the module to fill."""
+    import hashlib
+    from concurrent.futures import ThreadPoolExecutor, as_completed
+    from pathlib import Path
+
+    from . import bitexact_context_package as pkg
+    if isinstance(loader_workers, bool) or not isinstance(loader_workers, int) or loader_workers < 1:
+        raise ValueError("loader_workers must be a positive integer")
+    if isinstance(dtype, str):
+        dtype = getattr(torch, dtype)
+    package = Path(package)
+    try:
+        manifest, entries = pkg.read_manifest(package)
+    except pkg.PackageError as exc:
+        raise ContextServingError(str(exc)) from exc
+    if tensor_factory is None:
+        tensor_factory = hip_tensor_factory
+    if host_decoder is None:
+        from .bitexact_context_codec import decode as host_decoder
+
+    previous = torch.get_default_dtype()
+    torch.set_default_dtype(dtype)
+    try:
+        with torch.device("meta"):
+            model = model_factory()
+    finally:
+        torch.set_default_dtype(previous)
+
+    try:
+        params = dict(model.named_parameters(remove_duplicate=False))
+    except TypeError:
+        params = dict(model.named_parameters())
+    if not params:
+        raise ContextServingError("model has no named parameters")
+    missing = sorted(set(params) - set(entries))
+    if missing:
+        raise ContextServingError(f"package missing required model parameters: {missing[:12]}")
+    wrong = [(n, tuple(entries[n]["shape"]), tuple(p.shape)) for n, p in params.items()
+             if tuple(entries[n]["shape"]) != tuple(p.shape)]
+    if wrong:
+        raise ContextServingError(f"manifest/model shape mismatch: {wrong[:8]}")
+
+    def frame_of(name):
+        try:
+            return pkg.read_frame(package, entries[name])
+        except pkg.PackageError as exc:
+            raise ContextServingError(str(exc)) from exc
+
+    def host_value(name, parameter):
+        row = entries[name]
+        decoded = host_decoder(frame_of(name))
+        if isinstance(decoded, torch.Tensor):
+            if decoded.dtype != torch.bfloat16:
+                raise ContextServingError("host BCTX decoder did not return BF16")
+            decoded = decoded.detach().cpu().contiguous().view(torch.uint16).numpy()
+        if tuple(decoded.shape) != pkg.frame_shape(row["shape"]):
+            raise ContextServingError(f"BCTX decoded frame geometry mismatch: {name}")
+        if hashlib.sha256(decoded.astype("<u2", copy=False).tobytes()).hexdigest() != row["source_sha256"]:
+            raise ContextServingError(f"BCTX decoded-source identity mismatch: {name}")
+        runtime = _runtime_dtype(model, name, parameter, dtype)
+        value = torch.from_numpy(decoded.copy()).view(torch.bfloat16).reshape(tuple(parameter.shape))
+        return value.to(runtime).contiguous(), runtime
+
+    def create_context(name):
+        row = entries[name]
+        context = tensor_factory(frame_of(name), stride=stride, device=device)
+        if tuple(context.shape) != pkg.frame_shape(row["shape"]):
+            raise ContextServingError(f"indexed BCTX shape mismatch: {name}")
+        if context.source_sha256 != row["source_sha256"]:
+            raise ContextServingError(f"BCTX decoded-source identity mismatch: {name}")
+        if getattr(context, "frame_sha256", None) != row["frame_sha256"]:
+            raise ContextServingError(f"BCTX backend frame identity mismatch: {name}")
+        resident = getattr(context, "resident_bytes", None)
+        if type(resident) is not int or resident < 0:
+            raise ContextServingError(f"BCTX backend lacks valid resident_bytes: {name}")
+        return context, resident
+
+    def record(name, kind, resident=0, **extra):
+        row = entries[name]
+        return dict(kind=kind, shape=list(row["shape"]), source_sha256=row["source_sha256"],
+                    frame_sha256=row["frame_sha256"], frame_bytes=row["frame_bytes"],
+                    resident_context_bytes=resident, **extra)
+
+    coded = [(module_name, module, f"{module_name}.weight" if module_name else "weight")
+             for module_name, module in list(model.named_modules())
+             if isinstance(module, (nn.Linear, nn.Embedding))]
+    coded = [item for item in coded if item[2] in entries]
+    contexts, done = {}, 0
+
+    def accept(name, result):
+        nonlocal done
+        contexts[name] = result
+        done += 1
+        if done % 25 == 0 or done == len(coded):
+            log(f"[bctx] indexed {done}/{len(coded)} compressed tensors")
+            if progress_callback is not None:
+                progress_callback(done, len(coded), name)
+
+    if loader_workers == 1:
+        for _, _, weight_name in coded:
+            accept(weight_name, create_context(weight_name))
+    elif coded:
+        with ThreadPoolExecutor(max_workers=loader_workers, thread_name_prefix="bctx-index") as pool:
+            futures = {pool.submit(create_context, item[2]): item[2] for item in coded}
+            for future in as_completed(futures):
+                accept(futures[future], future.result())
+
+    consumed, replacements = {}, {}
+    for module_name, module, weight_name in coded:
+        context, resident = contexts[weight_name]
+        if isinstance(module, nn.Linear):
+            bias = None
+            if module.bias is not None:
+                bias_name = f"{module_name}.bias" if module_name else "bias"
+                if bias_name not in entries:
+                    raise ContextServingError(f"package missing required linear bias: {bias_name}")
+                value, runtime = host_value(bias_name, module.bias)
+                bias = nn.Parameter(value, requires_grad=False)
+                consumed[bias_name] = record(bias_name, "dense_bias", runtime_dtype=str(runtime))
+            replacements[module_name] = BctxLinear(context, bias, batch_invariant=batch_invariant)
+            consumed[weight_name] = record(weight_name, "compressed_linear", resident)
+        else:
+            replacements[module_name] = BctxEmbedding(context, padding_idx=module.padding_idx)
+            consumed[weight_name] = record(weight_name, "compressed_embedding", resident)
+    # parents before children, so that a replaced parent is not looked up through a stale child
+    for name, replacement in sorted(replacements.items(), key=lambda item: item[0].count(".")):
+        parent, attr = _parent_and_attr(model, name)
+        setattr(parent, attr, replacement)
+
+    for name, parameter in params.items():
+        if name in consumed:
+            continue
+        value, runtime = host_value(name, parameter)
+        parent, attr = _parent_and_attr(model, name)
+        parent._parameters[attr] = nn.Parameter(value, requires_grad=False)
+        consumed[name] = record(name, "dense_parameter", runtime_dtype=str(runtime))
+
+    left = [f"parameter:{n}" for n, p in model.named_parameters() if p.is_meta]
+    left += [f"buffer:{n}" for n, b in model.named_buffers() if b.is_meta]
+    if left:
+        raise ContextServingError(f"model contains unfilled meta tensors: {left[:12]}")
+    model.to(device)
+    compressed = [n for n, r in consumed.items() if r["kind"].startswith("compressed")]
+    receipt = {
+        "schema": "georefine.bctx_serving_load.v1", "status": "ok", "format": "BCTX v1",
+        "device": str(device), "dtype_default": str(dtype),
+        "package_manifest": str(package / "manifest.json"),
+        "tensor_count": len(entries), "consumed_count": len(consumed),
+        "unused_package_tensors": sorted(set(entries) - set(consumed)),
+        "compressed_tensor_count": len(compressed),
+        "resident_context_bytes": sum(consumed[n]["resident_context_bytes"] for n in compressed),
+        "dense_parameter_bytes": sum(p.numel() * p.element_size() for p in model.parameters()),
+        "buffer_bytes": sum(b.numel() * b.element_size() for b in model.buffers()),
+        "consumed_tensors": consumed, "restored_bf16_control": False, "transcoded": False,
+    }
+    return model, receipt

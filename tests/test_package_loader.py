@@ -1,0 +1,188 @@
+"""Package reader/writer and the model loader, on the CPU: a host-backed stand-in for the
+device tensor object exercises every check the loader makes (the reference's own loader
+tests use the same device, tests/test_bitexact_context_serving.py:14-47)."""
+import hashlib
+import json
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+from georefine_amd import bitexact_context_codec as codec
+from georefine_amd import bitexact_context_package as pkg
+from georefine_amd import serving
+
+
+class TinyModel(nn.Module):
+    def __init__(self, *, bad_buffer=False):
+        super().__init__()
+        self.emb = nn.Embedding(8, 4)
+        self.lin = nn.Linear(4, 3)
+        self.norm = nn.LayerNorm(4)
+        self.fp32_exception = nn.Parameter(torch.empty(2))
+        self._keep_in_fp32_modules_strict = {"fp32_exception"}
+        if bad_buffer:
+            self.register_buffer("stuck", torch.empty(1, device="meta"), persistent=False)
+
+    def forward(self, ids):
+        return self.lin(self.norm(self.emb(ids)))
+
+
+class HostContext:
+    """The tensor-object contract on the CPU: decode on the host, gather by indexing."""
+
+    def __init__(self, frame, *, stride, device, resident=37):
+        del stride
+        words = codec.decode(frame)
+        self.values = torch.from_numpy(words.copy()).view(torch.bfloat16)
+        self.shape = tuple(words.shape)
+        self.source_sha256 = hashlib.sha256(words.tobytes()).hexdigest()
+        self.frame_sha256 = hashlib.sha256(frame).hexdigest()
+        self.resident_bytes = resident
+        self.device = torch.device(device)
+
+    def decode(self, *, check=True):
+        return self.values.to(self.device).clone()
+
+    def gather_rows(self, ids, *, check=True):
+        return self.decode()[ids.to(self.device)]
+
+
+def _tensors():
+    return {
+        "emb.weight": torch.arange(32, dtype=torch.float32).reshape(8, 4).to(torch.bfloat16),
+        "lin.weight": torch.arange(12, dtype=torch.float32).reshape(3, 4).to(torch.bfloat16),
+        "lin.bias": torch.tensor([0.25, -0.5, 1.0], dtype=torch.bfloat16),
+        "norm.weight": torch.tensor([1.0, 0.75, 1.25, 0.5], dtype=torch.bfloat16),
+        "norm.bias": torch.zeros(4, dtype=torch.bfloat16),
+        "fp32_exception": torch.tensor([2.0, -3.0], dtype=torch.bfloat16),
+        "mtp.layers.0.weight": torch.ones(2, 2, 3, dtype=torch.bfloat16),
+    }
+
+
+def _package(tmp_path, drop=()):
+    tensors = {k: v for k, v in _tensors().items() if k not in drop}
+    path = tmp_path / "package"
+    pkg.write_package(path, tensors, sidecars={"config.json": b'{"hidden": 4}'})
+    return path, tensors
+
+
+def _load(path, **kw):
+    kw.setdefault("model_factory", TinyModel)
+    kw.setdefault("tensor_factory", HostContext)
+    kw.setdefault("log", lambda _: None)
+    return serving.load_bctx_model(path, device="cpu", **kw)
+
+
+def _edit_manifest(path, fn):
+    m = json.loads((path / "manifest.json").read_text())
+    fn(m)
+    (path / "manifest.json").write_text(json.dumps(m))
+
+
+def test_write_read_verify_round_trip(tmp_path):
+    path, tensors = _package(tmp_path)
+    manifest, entries = pkg.read_manifest(path)
+    assert manifest["schema"] == "bitexact-context-package-v1" and set(entries) == set(tensors)
+    for name, t in tensors.items():
+        row = entries[name]
+        assert row["shape"] == list(t.shape) and row["source_bytes"] == 2 * t.numel()
+        words = pkg.decode_tensor(path, row)
+        assert np.array_equal(words, t.view(torch.uint16).numpy())
+    assert pkg.frame_shape([2, 2, 3]) == (2, 6) and pkg.frame_shape([5]) == (1, 5)
+    totals = pkg.verify(path)
+    assert totals["tensors"] == len(tensors) and totals["source_bytes"] == sum(2 * t.numel() for t in tensors.values())
+
+
+def test_reader_rejects_tampering(tmp_path):
+    path, _ = _package(tmp_path)
+    frame = path / "frames" / "00001.bctx"
+    data = bytearray(frame.read_bytes())
+    data[-1] ^= 1
+    frame.write_bytes(bytes(data))
+    with pytest.raises(pkg.PackageError, match="identity mismatch"):
+        pkg.verify(path)
+    (path / "sidecars" / "config.json").write_bytes(b"{}")
+    frame.write_bytes(bytes(data[:-1]) + bytes([data[-1] ^ 1]))
+    with pytest.raises(pkg.PackageError, match="sidecar integrity"):
+        pkg.verify(path)
+
+
+@pytest.mark.parametrize("edit,message", [
+    (lambda m: m.update(schema="other"), "unsupported or incomplete"),
+    (lambda m: m.update(complete=False), "unsupported or incomplete"),
+    (lambda m: m["tensors"].append(dict(m["tensors"][0])), "duplicate tensor receipt"),
+    (lambda m: m["tensors"][0].update(frame="../outside.bctx"), "unsafe tensor frame path"),
+    (lambda m: m["tensors"][0].update(frame="/etc/passwd"), "unsafe tensor frame path"),
+    (lambda m: m["tensors"][0].update(source_bytes=7), "source byte count"),
+    (lambda m: m["tensors"][0].update(frame_sha256="xyz"), "invalid source/frame SHA"),
+    (lambda m: m["tensors"][0].update(shape=[8, -4]), "invalid tensor shape"),
+    (lambda m: m["tensors"][0].update(dtype="F16"), "incomplete or unsupported"),
+])
+def test_manifest_validation(tmp_path, edit, message):
+    path, _ = _package(tmp_path)
+    _edit_manifest(path, edit)
+    with pytest.raises(pkg.PackageError, match=message):
+        pkg.read_manifest(path)
+    with pytest.raises(serving.ContextServingError, match=message):
+        _load(path)
+
+
+@pytest.mark.parametrize("workers", [1, 3])
+def test_loader_fills_model_and_matches_dense(tmp_path, workers):
+    path, tensors = _package(tmp_path)
+    seen = []
+    model, receipt = _load(path, loader_workers=workers, progress_callback=lambda *a: seen.append(a))
+    assert isinstance(model.lin, serving.BctxLinear) and isinstance(model.emb, serving.BctxEmbedding)
+    assert model.fp32_exception.dtype == torch.float32 and model.norm.weight.dtype == torch.bfloat16
+    assert not any(p.is_meta for p in model.parameters())
+    dense = TinyModel().to(torch.bfloat16)
+    with torch.no_grad():
+        for name, t in tensors.items():
+            if name.startswith("mtp."):
+                continue
+            dict(dense.named_parameters())[name].copy_(t)
+    ids = torch.tensor([[0, 3, 7], [2, 2, 5]])
+    assert torch.equal(model(ids), dense(ids))
+    assert receipt["status"] == "ok" and receipt["compressed_tensor_count"] == 2
+    assert receipt["resident_context_bytes"] == 74 and receipt["unused_package_tensors"] == ["mtp.layers.0.weight"]
+    assert receipt["consumed_tensors"]["lin.bias"]["kind"] == "dense_bias"
+    assert receipt["consumed_tensors"]["fp32_exception"]["runtime_dtype"] == "torch.float32"
+    assert receipt["transcoded"] is False and seen and seen[-1][:2] == (2, 2)
+
+
+def test_loader_errors(tmp_path):
+    path, _ = _package(tmp_path, drop=("norm.bias",))
+    with pytest.raises(serving.ContextServingError, match="missing required model parameters"):
+        _load(path)
+    path2, _ = _package(tmp_path / "b")
+    with pytest.raises(serving.ContextServingError, match="unfilled meta tensors"):
+        _load(path2, model_factory=lambda: TinyModel(bad_buffer=True))
+    with pytest.raises(serving.ContextServingError, match="resident_bytes"):
+        _load(path2, tensor_factory=lambda f, **kw: HostContext(f, resident=-1, **kw))
+    with pytest.raises(ValueError):
+        _load(path2, loader_workers=0)
+    _edit_manifest(path2, lambda m: m["tensors"][1].update(shape=[4, 3]))
+    with pytest.raises(serving.ContextServingError, match="shape mismatch"):
+        _load(path2)
+
+
+def test_loader_checks_backend_identity(tmp_path):
+    path, _ = _package(tmp_path)
+
+    class WrongDigest(HostContext):
+        def __init__(self, *a, **kw):
+            super().__init__(*a, **kw)
+            self.source_sha256 = "0" * 64
+
+    with pytest.raises(serving.ContextServingError, match="decoded-source identity"):
+        _load(path, tensor_factory=WrongDigest)
+
+    class WrongShape(HostContext):
+        def __init__(self, *a, **kw):
+            super().__init__(*a, **kw)
+            self.shape = self.shape[::-1]
+
+    with pytest.raises(serving.ContextServingError, match="indexed BCTX shape mismatch"):
+        _load(path, tensor_factory=WrongShape)
