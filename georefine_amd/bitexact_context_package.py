@@ -12,12 +12,19 @@ The writer covers what tests and small deployments need (every tensor coded with
 (row classes, column classes) setting, optional sidecar files pinned by size and digest);
 the reference's package builder, with its per-tensor configuration search and archive of
 model assets, is outside this library.
+
+Predictive candidates.  A manifest may carry ``selected_candidates``: tensors whose frame is
+a PPCX frame coded against one other tensor of the package (``mode`` "single") or against
+the row-wise mix of two (``"mixbf16"``, with a ``[rows, 3]`` BF16 coefficient file), possibly
+stored transposed.  The fields and their checks follow the reference's predictive package
+(GCR/bitexact_predictive_package.py:433-537; coefficient files :59-86).
 """
 from __future__ import annotations
 
 import hashlib
 import json
 import math
+import zlib
 from pathlib import Path, PurePosixPath
 
 import numpy as np
@@ -182,3 +189,142 @@ def write_package(package, tensors, *, row_classes=16, col_classes=4, sidecars=N
                 "tensors": rows, "metadata_assets": assets}
     (package / "manifest.json").write_text(json.dumps(manifest, indent=1), encoding="utf-8")
     return manifest
+
+
+# ------------------------------------------------------------------ predictive candidates
+
+def _inside(package, value, what):
+    if not isinstance(value, str):
+        raise PackageError(f"{what} path must be a string")
+    rel = PurePosixPath(value)
+    if rel.is_absolute() or not rel.parts or ".." in rel.parts:
+        raise PackageError(f"unsafe {what} path")
+    return Path(package).joinpath(*rel.parts)
+
+
+def read_candidates(package, manifest, entries):
+    """Validated ``selected_candidates`` of a manifest ({} when it has none): every candidate
+    names a receipt, its references exist with the digests the receipts pin, the reference
+    graph has no cycle, and mixed candidates carry coefficients of the references' row count."""
+    selected = manifest.get("selected_candidates") or {}
+    if not isinstance(selected, dict):
+        raise PackageError("selected_candidates must be an object")
+    frames = set()
+    for name, c in selected.items():
+        row = entries.get(name)
+        if row is None or not isinstance(c, dict) or c.get("name") != name:
+            raise PackageError(f"candidate schema/name mismatch: {name}")
+        refs = c.get("references")
+        wanted = {"single": 1, "mixbf16": 2}.get(c.get("mode"))
+        if wanted is None:
+            raise PackageError(f"candidate mode unsupported: {name}")
+        if not isinstance(refs, list) or len(refs) != wanted:
+            raise PackageError(f"candidate reference list invalid: {name}")
+        for ref in refs:
+            other = entries.get(ref.get("name")) if isinstance(ref, dict) else None
+            if other is None or ref["name"] == name or ref.get("sha256") != other["source_sha256"]:
+                raise PackageError(f"reference identity SHA mismatch: {name}")
+        if (c.get("transform") not in ("identity", "target transpose") or c.get("shape") != row["shape"]
+                or c.get("source_sha256") != row["source_sha256"] or c.get("source_bytes") != row["source_bytes"]):
+            raise PackageError(f"candidate source identity/transform invalid: {name}")
+        if type(c.get("frame_bytes")) is not int or c["frame_bytes"] <= 0 or not _is_digest(c.get("frame_sha256")):
+            raise PackageError(f"candidate frame pin invalid: {name}")
+        rel = _inside(package, c.get("frame"), "candidate frame").relative_to(Path(package)).as_posix()
+        if rel in frames:
+            raise PackageError("candidate frame is shared by multiple tensors")
+        frames.add(rel)
+        if c["mode"] == "mixbf16":
+            coeff, shapes = c.get("coefficients"), [entries[r["name"]]["shape"] for r in refs]
+            if shapes[0] != shapes[1]:
+                raise PackageError(f"mixed reference geometry mismatch: {name}")
+            if (not isinstance(coeff, dict) or coeff.get("shape") != [frame_shape(shapes[0])[0], 3]
+                    or not _is_digest(c.get("derived_reference_sha256"))):
+                raise PackageError(f"mixed coefficient metadata invalid: {name}")
+    state = {}
+
+    def visit(name):
+        if state.get(name) == 1:
+            raise PackageError("candidate reference cycle")
+        if name in state:
+            return
+        state[name] = 1
+        for ref in selected.get(name, {}).get("references", ()):
+            visit(ref["name"])
+        state[name] = 2
+
+    for name in selected:
+        visit(name)
+    return selected
+
+
+def read_candidate_frame(package, candidate):
+    frame = _inside(package, candidate["frame"], "candidate frame").read_bytes()
+    if len(frame) != candidate["frame_bytes"] or hashlib.sha256(frame).hexdigest() != candidate["frame_sha256"]:
+        raise PackageError(f"candidate frame integrity mismatch: {candidate['name']}")
+    return frame
+
+
+def read_coefficients(package, candidate):
+    """The ``[rows, 3]`` BF16 coefficient words of a mixed candidate (stored raw or deflated)."""
+    c = candidate["coefficients"]
+    encoded = _inside(package, c.get("path"), "coefficient").read_bytes()
+    if len(encoded) != c.get("bytes") or hashlib.sha256(encoded).hexdigest() != c.get("sha256"):
+        raise PackageError("mixed coefficient checksum mismatch")
+    rows, three = c["shape"]
+    expected = rows * three * 2
+    encoding = c.get("encoding", "identity")
+    if encoding == "identity":
+        raw = encoded
+    elif encoding == "zlib":
+        d = zlib.decompressobj()
+        try:
+            raw = d.decompress(encoded, expected + 1)
+            if len(raw) > expected or d.unconsumed_tail:
+                raise PackageError("mixed coefficient decompression exceeds declared shape")
+            raw += d.flush()
+        except zlib.error as exc:
+            raise PackageError("mixed coefficient zlib data is corrupt") from exc
+        if not d.eof or d.unused_data:
+            raise PackageError("mixed coefficient compressed stream is incomplete or has trailing bytes")
+    else:
+        raise PackageError("unsupported coefficient encoding")
+    if len(raw) != expected:
+        raise PackageError("mixed coefficient byte count mismatch")
+    return np.frombuffer(raw, dtype="<u2").reshape(rows, three).copy()
+
+
+def add_candidate(package, name, *, references, transform="identity", coefficients=None):
+    """Code the tensor ``name`` of an existing package against its references and record
+    the candidate in the manifest (the writer-side counterpart of ``read_candidates``).
+    ``references``: one tensor name, or two with ``coefficients`` ([rows, 3] uint16 words)."""
+    from . import bitexact_predictive_codec as ppcx
+    from . import bitexact_predictive_mix as mix
+    package = Path(package)
+    manifest, entries = read_manifest(package)
+    row = entries[name]
+    words = [decode_tensor(package, entries[r]).reshape(frame_shape(entries[r]["shape"])) for r in references]
+    target = decode_tensor(package, row).reshape(frame_shape(row["shape"]))
+    if transform == "target transpose":
+        target = np.ascontiguousarray(target.T)
+    candidate = {"name": name, "mode": "single" if len(references) == 1 else "mixbf16", "transform": transform,
+                 "references": [{"name": r, "sha256": entries[r]["source_sha256"]} for r in references],
+                 "shape": row["shape"], "source_sha256": row["source_sha256"], "source_bytes": row["source_bytes"]}
+    reference = words[0]
+    if len(references) == 2:
+        coeff = np.ascontiguousarray(coefficients, dtype="<u2")
+        reference = np.ascontiguousarray(mix.predict(words[0], words[1], coeff))
+        (package / "predictive-coefficients").mkdir(exist_ok=True)
+        rel = f"predictive-coefficients/{len(manifest.get('selected_candidates') or {}):05d}.bf16"
+        (package / rel).write_bytes(coeff.tobytes())
+        candidate["coefficients"] = {"path": rel, "shape": list(coeff.shape), "bytes": coeff.nbytes,
+                                     "decoded_bytes": coeff.nbytes, "encoding": "identity",
+                                     "sha256": hashlib.sha256(coeff.tobytes()).hexdigest()}
+        candidate["derived_reference_sha256"] = hashlib.sha256(reference.tobytes()).hexdigest()
+    frame = ppcx.encode(target, reference)
+    (package / "predictive-frames").mkdir(exist_ok=True)
+    rel = f"predictive-frames/{len(manifest.get('selected_candidates') or {}):05d}.ppcx"
+    (package / rel).write_bytes(frame)
+    candidate.update(frame=rel, frame_bytes=len(frame), frame_sha256=hashlib.sha256(frame).hexdigest())
+    manifest.setdefault("selected_candidates", {})[name] = candidate
+    (package / "manifest.json").write_text(json.dumps(manifest, indent=1), encoding="utf-8")
+    return candidate

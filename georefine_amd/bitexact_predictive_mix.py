@@ -121,11 +121,15 @@ def _mix_device(up, gate, coeff):
 
 
 def predict(up, gate, coeff):
-    """uint16 word matrices on the host, or bfloat16 tensors on the GPU (same bits either way)."""
+    """uint16 word matrices or bfloat16 tensors on the host, or bfloat16 tensors on the GPU
+    (same bits either way)."""
     try:
         import torch
     except ImportError:
         torch = None
     if torch is not None and isinstance(up, torch.Tensor):
+        if up.device.type == "cpu":  # host tensors: the same arithmetic on their bit patterns
+            words = [t.detach().contiguous().view(torch.uint16).numpy() for t in (up, gate, coeff)]
+            return torch.from_numpy(np.ascontiguousarray(_mix_cpu(*words))).view(torch.bfloat16)
         return _mix_device(up, gate, coeff)
     return _mix_cpu(up, gate, coeff)

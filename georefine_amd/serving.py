@@ -156,8 +156,8 @@ def _runtime_dtype(model, name, parameter, requested):
 
 
 def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
-                    tensor_factory=None, host_decoder=None, loader_workers=1, batch_invariant=False,
-                    log=print, progress_callback=None):
+                    tensor_factory=None, predictive_factory=None, mix_predictor=None, host_decoder=None,
+                    loader_workers=1, batch_invariant=False, log=print, progress_callback=None):
     """Build ``model_factory()`` on the meta device and fill it from a BCTX package without
     ever holding a dense checkpoint: returns ``(model, receipt)``.
 
@@ -168,12 +168,22 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
     ``loader_workers`` threads); the object's geometry, decoded-source digest, frame digest
     and ``resident_bytes`` are checked against the receipt.  Every other parameter and every
     linear bias is decoded on the host, digest checked, and installed dense.  The model must
-    end with no meta tensor left.  What this loader leaves to the caller is the model
+    end with no meta tensor left.
+
+    Weights listed under the manifest's ``selected_candidates`` are PPCX frames coded against
+    other tensors of the package (GCR/bitexact_predictive_serving.py:880-935): their
+    references get tensor objects first, ``predictive_factory(frame, reference_words,
+    stride=, device=)`` indexes the frame against the reference words (for ``mixbf16`` the
+    row-wise mix of two references with the candidate's coefficients, whose digest is
+    checked), and the module receives a ``PredictiveContextTensor`` that resolves the
+    references when it decodes.  What this loader leaves to the caller is the model
     construction itself (the reference reads a Transformers config and generation config
     from the package's sidecars): ``model_factory`` returns the module to fill."""
     import hashlib
     from concurrent.futures import ThreadPoolExecutor, as_completed
     from pathlib import Path
+
+    import numpy as np
 
     from . import bitexact_context_package as pkg
     if isinstance(loader_workers, bool) or not isinstance(loader_workers, int) or loader_workers < 1:
@@ -187,8 +197,16 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         raise ContextServingError(str(exc)) from exc
     if tensor_factory is None:
         tensor_factory = hip_tensor_factory
+    if predictive_factory is None:
+        predictive_factory = hip_predictive_factory
+    if mix_predictor is None:
+        from .bitexact_predictive_mix import predict as mix_predictor
     if host_decoder is None:
         from .bitexact_context_codec import decode as host_decoder
+    try:
+        selected = pkg.read_candidates(package, manifest, entries)
+    except pkg.PackageError as exc:
+        raise ContextServingError(str(exc)) from exc
 
     previous = torch.get_default_dtype()
     torch.set_default_dtype(dtype)
@@ -248,7 +266,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         return context, resident
 
     def record(name, kind, resident=0, **extra):
-        row = entries[name]
+        row = selected.get(name) if kind.startswith("compressed") and name in selected else entries[name]
         return dict(kind=kind, shape=list(row["shape"]), source_sha256=row["source_sha256"],
                     frame_sha256=row["frame_sha256"], frame_bytes=row["frame_bytes"],
                     resident_context_bytes=resident, **extra)
@@ -257,25 +275,106 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
              for module_name, module in list(model.named_modules())
              if isinstance(module, (nn.Linear, nn.Embedding))]
     coded = [item for item in coded if item[2] in entries]
+
+    # tensors that need an object on the device: the coded weights and, transitively, the
+    # references of predictive candidates; plain frames first (in parallel), then the
+    # candidates in dependency order
+    needed, order = set(), []
+
+    def need(name):
+        if name in needed:
+            return
+        needed.add(name)
+        for ref in selected.get(name, {}).get("references", ()):
+            need(ref["name"])
+        order.append(name)
+
+    for _, _, weight_name in coded:
+        need(weight_name)
+    plain = [name for name in order if name not in selected]
     contexts, done = {}, 0
 
     def accept(name, result):
         nonlocal done
         contexts[name] = result
         done += 1
-        if done % 25 == 0 or done == len(coded):
-            log(f"[bctx] indexed {done}/{len(coded)} compressed tensors")
+        if done % 25 == 0 or done == len(order):
+            log(f"[bctx] indexed {done}/{len(order)} compressed tensors")
             if progress_callback is not None:
-                progress_callback(done, len(coded), name)
+                progress_callback(done, len(order), name)
 
     if loader_workers == 1:
-        for _, _, weight_name in coded:
-            accept(weight_name, create_context(weight_name))
-    elif coded:
+        for name in plain:
+            accept(name, create_context(name))
+    elif plain:
         with ThreadPoolExecutor(max_workers=loader_workers, thread_name_prefix="bctx-index") as pool:
-            futures = {pool.submit(create_context, item[2]): item[2] for item in coded}
+            futures = {pool.submit(create_context, name): name for name in plain}
             for future in as_completed(futures):
                 accept(futures[future], future.result())
+
+    host_words = {}  # frame-shaped uint16 words of references, dropped once the candidates are indexed
+
+    def words_of(name):
+        if name in host_words:
+            return host_words[name]
+        row = entries[name]
+        if name in selected:
+            from .bitexact_predictive_codec import decode as predictive_decode
+            value = predictive_decode(candidate_frame(name), reference_words(name))
+            if selected[name]["transform"] == "target transpose":
+                value = value.T
+        else:
+            value = host_decoder(frame_of(name))
+            if isinstance(value, torch.Tensor):
+                value = value.detach().cpu().contiguous().view(torch.uint16).numpy()
+        value = np.ascontiguousarray(value).reshape(pkg.frame_shape(row["shape"]))
+        if hashlib.sha256(value.astype("<u2", copy=False).tobytes()).hexdigest() != row["source_sha256"]:
+            raise ContextServingError(f"BCTX decoded-source identity mismatch: {name}")
+        host_words[name] = value
+        return value
+
+    def candidate_frame(name):
+        try:
+            return pkg.read_candidate_frame(package, selected[name])
+        except (pkg.PackageError, OSError) as exc:
+            raise ContextServingError(str(exc)) from exc
+
+    def reference_words(name):
+        c = selected[name]
+        refs = [words_of(ref["name"]) for ref in c["references"]]
+        if c["mode"] == "single":
+            return refs[0]
+        derived = np.ascontiguousarray(mix_predictor(refs[0], refs[1], pkg.read_coefficients(package, c)), dtype="<u2")
+        if hashlib.sha256(derived.tobytes()).hexdigest() != c["derived_reference_sha256"]:
+            raise ContextServingError(f"derived reference checksum mismatch: {name}")
+        return derived
+
+    for name in order:
+        if name not in selected:
+            continue
+        c, row = selected[name], entries[name]
+        native = predictive_factory(candidate_frame(name), reference_words(name), stride=stride, device=device)
+        geometry = pkg.frame_shape(row["shape"])
+        if c["transform"] == "target transpose":
+            geometry = geometry[::-1]
+        if tuple(native.shape) != geometry:
+            raise ContextServingError(f"PPCX frame geometry mismatch: {name}")
+        if getattr(native, "frame_sha256", None) != c["frame_sha256"]:
+            raise ContextServingError(f"PPCX frame identity mismatch: {name}")
+        own = getattr(native, "resident_bytes", None)
+        if type(own) is not int or own < 0:
+            raise ContextServingError(f"PPCX resident byte accounting missing: {name}")
+        coefficients = None
+        if c["mode"] == "mixbf16":
+            coefficients = torch.from_numpy(pkg.read_coefficients(package, c)).view(torch.bfloat16).to(device)
+            own += coefficients.numel() * coefficients.element_size()
+        wrapped = PredictiveContextTensor(
+            native, [contexts[ref["name"]][0] for ref in c["references"]],
+            predictor=mix_predictor if c["mode"] == "mixbf16" else None, coefficients=coefficients,
+            transform=c["transform"], shape=pkg.frame_shape(row["shape"]), source_sha256=row["source_sha256"],
+            frame_sha256=c["frame_sha256"], resident_bytes=own)
+        accept(name, (wrapped, own))
+    host_words.clear()
 
     consumed, replacements = {}, {}
     for module_name, module, weight_name in coded:

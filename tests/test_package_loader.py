@@ -186,3 +186,110 @@ def test_loader_checks_backend_identity(tmp_path):
 
     with pytest.raises(serving.ContextServingError, match="indexed BCTX shape mismatch"):
         _load(path, tensor_factory=WrongShape)
+
+
+# ------------------------------------------------------------------ predictive candidates
+
+class HostPredictive:
+    """The predictive tensor-object contract on the CPU."""
+
+    def __init__(self, frame, reference_words, stride=1024, device="cpu"):
+        from georefine_amd import bitexact_predictive_codec as ppcx
+        del stride
+        self.reference = np.ascontiguousarray(reference_words)
+        words = ppcx.decode(frame, self.reference)
+        self.values = torch.from_numpy(words.copy()).view(torch.bfloat16)
+        self.shape = tuple(words.shape)
+        self.source_sha256 = hashlib.sha256(words.tobytes()).hexdigest()
+        self.frame_sha256 = hashlib.sha256(frame).hexdigest()
+        self.resident_bytes = 11
+        self.device = torch.device(device)
+
+    def decode(self, reference, *, check=True):
+        assert np.array_equal(reference.contiguous().view(torch.uint16).numpy(), self.reference)
+        return self.values.to(self.device).clone()
+
+
+class GatedNet(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.up = nn.Linear(32, 16, bias=False)
+        self.gate = nn.Linear(32, 16, bias=False)
+        self.down = nn.Linear(16, 32, bias=False)
+        self.twin = nn.Linear(32, 16, bias=False)
+
+    def forward(self, x):
+        return self.down(self.up(x) * self.gate(x)) + self.twin(x).sum(-1, keepdim=True)
+
+
+def _gated_package(tmp_path):
+    from conftest import bf16_words, weight_like, words_to_float
+    from georefine_amd import bitexact_predictive_mix as mix
+    rng = np.random.default_rng(3)
+    up, gate = weight_like(rng, 16, 32), weight_like(rng, 16, 32)
+    down_t = bf16_words(0.7 * words_to_float(up) - 0.2 * words_to_float(gate) + rng.normal(0, 1e-4, (16, 32)))
+    twin = bf16_words(words_to_float(up) + rng.normal(0, 1e-4, (16, 32)))
+    tensors = {"up.weight": up, "gate.weight": gate, "down.weight": np.ascontiguousarray(down_t.T), "twin.weight": twin}
+    path = tmp_path / "package"
+    pkg.write_package(path, tensors)
+    coeff = mix.fit_mixed_coefficients(down_t, up, gate)
+    pkg.add_candidate(path, "down.weight", references=["up.weight", "gate.weight"], transform="target transpose",
+                      coefficients=coeff)
+    pkg.add_candidate(path, "twin.weight", references=["up.weight"])
+    return path, tensors
+
+
+def test_loader_resolves_predictive_candidates(tmp_path):
+    path, tensors = _gated_package(tmp_path)
+    manifest, entries = pkg.read_manifest(path)
+    selected = pkg.read_candidates(path, manifest, entries)
+    assert selected["down.weight"]["mode"] == "mixbf16" and selected["twin.weight"]["mode"] == "single"
+    assert pkg.read_coefficients(path, selected["down.weight"]).shape == (16, 3)
+    model, receipt = _load(path, model_factory=GatedNet, predictive_factory=HostPredictive)
+    assert isinstance(model.down.context_weight, serving.PredictiveContextTensor)
+    assert model.down.context_weight.transform == "target transpose" and model.down.context_weight.shape == (32, 16)
+    for name, words in tensors.items():
+        module = getattr(model, name.split(".")[0])
+        assert np.array_equal(module.weight.view(torch.uint16).numpy(), words), name
+    dense = GatedNet().to(torch.bfloat16)
+    with torch.no_grad():
+        for name, words in tensors.items():
+            dict(dense.named_parameters())[name].copy_(torch.from_numpy(words).view(torch.bfloat16))
+    x = torch.randn(5, 32, dtype=torch.bfloat16)
+    assert torch.equal(model(x), dense(x))
+    assert receipt["compressed_tensor_count"] == 4
+    assert receipt["consumed_tensors"]["down.weight"]["frame_sha256"] == selected["down.weight"]["frame_sha256"]
+    assert receipt["resident_context_bytes"] == 37 + 37 + (11 + 16 * 3 * 2) + 11
+
+
+@pytest.mark.parametrize("edit,message", [
+    (lambda c: c["twin.weight"]["references"][0].update(sha256="0" * 64), "reference identity SHA mismatch"),
+    (lambda c: c["twin.weight"].update(mode="triple"), "candidate mode unsupported"),
+    (lambda c: c["twin.weight"].update(transform="rotate"), "transform invalid"),
+    (lambda c: c["twin.weight"].update(frame="../x.ppcx"), "unsafe candidate frame path"),
+    (lambda c: c["down.weight"].update(derived_reference_sha256="f" * 64), "derived reference checksum"),
+    (lambda c: c["down.weight"]["coefficients"].update(shape=[15, 3]), "coefficient metadata invalid"),
+    (lambda c: c["twin.weight"].update(frame_sha256="a" * 64), "candidate frame integrity"),
+])
+def test_candidate_validation(tmp_path, edit, message):
+    path, _ = _gated_package(tmp_path)
+    _edit_manifest(path, lambda m: edit(m["selected_candidates"]))
+    with pytest.raises(serving.ContextServingError, match=message):
+        _load(path, model_factory=GatedNet, predictive_factory=HostPredictive)
+
+
+def test_candidate_cycle_is_rejected(tmp_path):
+    path, _ = _gated_package(tmp_path)
+
+    def make_cycle(m):
+        c = dict(m["selected_candidates"]["twin.weight"])
+        up = next(r for r in m["tensors"] if r["name"] == "up.weight")
+        twin = next(r for r in m["tensors"] if r["name"] == "twin.weight")
+        c.update(name="up.weight", shape=up["shape"], source_sha256=up["source_sha256"], source_bytes=up["source_bytes"],
+                 references=[{"name": "twin.weight", "sha256": twin["source_sha256"]}], frame="predictive-frames/9.ppcx")
+        m["selected_candidates"]["up.weight"] = c
+
+    _edit_manifest(path, make_cycle)
+    manifest, entries = pkg.read_manifest(path)
+    with pytest.raises(pkg.PackageError, match="cycle"):
+        pkg.read_candidates(path, manifest, entries)
