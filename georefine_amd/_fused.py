@@ -38,11 +38,12 @@ def choose_shift(nc, budget=LUT_BUDGET):
     return shift
 
 
-def sparse_tables(freq, nr, nc, shift):
+def sparse_tables(freq, nr, nc, shift, image=None):
     """Per row class: u8 lookup [nc << lognb] and u64 entries [nc][tabn+1].
 
     Entry(column class c, sparse i): low32 = start | (freq & 0xFFFF) << 16 with 0 standing for
-    65536, high32 = symbol << 5.  Unused entries are (start 0, freq 65536): a forward scan
+    65536, high32 = image(symbols), the symbol's bits in the BF16 word (default: symbol << 5,
+    the context codec's 10-bit main symbol).  Unused entries are (start 0, freq 65536): a forward scan
     always stops on them.  The lookup byte of a bucket is the sparse index of the symbol
     that owns most of the bucket's slots (the first of them on a tie), which minimises the
     slots whose lookup has to scan to a neighbouring entry."""
@@ -68,7 +69,7 @@ def sparse_tables(freq, nr, nc, shift):
             starts = np.concatenate(([0], np.cumsum(fs)[:-1]))
             ends = starts + fs
             lo = starts | ((fs & 0xFFFF) << 16)
-            hi = syms << 5
+            hi = syms << 5 if image is None else image(syms)
             tab[rho, c, :syms.size] = (lo.astype(np.uint64) | (hi.astype(np.uint64) << np.uint64(32)))
             first = np.searchsorted(starts, lo_slot, side="right") - 1
             last = np.searchsorted(starts, hi_slot - 1, side="right") - 1
@@ -196,7 +197,8 @@ def build_tiles(row_class, nr, r):
 class FramePlan:
     """Frame-level derived arrays (shared by every tiling) and a tiling factory."""
 
-    def __init__(self, shape, nr, nc, row_class, main_freq, seg_states, seg_offsets, main_bytes, seg_len):
+    def __init__(self, shape, nr, nc, row_class, main_freq, seg_states, seg_offsets, main_bytes, seg_len,
+                 image=None):
         rows, cols = shape
         if rows * cols > 0xFFFFFFFF:
             raise FusedUnsupported("matrix too large")
@@ -204,7 +206,7 @@ class FramePlan:
         self.spr = cols // seg_len
         self.shift = choose_shift(nc)
         self.lognb = 16 - self.shift
-        self.lut, self.tab, self.tabn = sparse_tables(main_freq, nr, nc, self.shift)
+        self.lut, self.tab, self.tabn = sparse_tables(main_freq, nr, nc, self.shift, image)
         self.seg_state = np.concatenate((seg_states, [1 << 23])).astype(np.uint32)
         self.seg_offset = np.concatenate((seg_offsets, [main_bytes])).astype(np.uint32)
         self.row_class = np.asarray(row_class)

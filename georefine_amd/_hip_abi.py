@@ -38,8 +38,16 @@ class GrfFusedTiling(ctypes.Structure):
             "threads", "lanes_per_row", "rows_per_tile", "n_slabs", "n_tiles", "piece_cap")]
 
 
+class GrfPpcxFused(ctypes.Structure):
+    _fields_ = [(name, ctypes.c_void_p) for name in (
+        "main_bytes", "raw5", "seg_state", "seg_offset", "lut", "tab")] + [
+        (name, ctypes.c_uint32) for name in (
+            "main_n_bytes", "rows", "cols", "n_labels", "seg_len", "segs_per_row", "shift", "lognb", "tabn")]
+
+
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
-                  "grf_bctx_fused_decode", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes", "grf_last_error", "grf_abi_version")
+                  "grf_bctx_fused_decode", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
+                  "grf_ppcx_bins", "grf_ppcx_fused_decode", "grf_last_error", "grf_abi_version")
 
 
 def declare(L):
@@ -61,5 +69,9 @@ def declare(L):
     L.grf_bctx_fused_decode.restype = i
     L.grf_bctx_fused_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, u32]
     L.grf_bctx_fused_lds_bytes.restype = u32
+    L.grf_ppcx_bins.argtypes = [vp, vp, vp, u32, u32, vp, vp]
+    L.grf_ppcx_bins.restype = i
+    L.grf_ppcx_fused_decode.argtypes = [ctypes.POINTER(GrfPpcxFused), tiling, vp, vp, vp, vp]
+    L.grf_ppcx_fused_decode.restype = i
     L.grf_last_error.restype = ctypes.c_char_p
     L.grf_abi_version.restype = i

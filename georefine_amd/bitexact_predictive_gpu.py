@@ -17,7 +17,7 @@ import os
 
 import numpy as np
 
-from . import _hip_abi, _native, _tables
+from . import _fused, _hip_abi, _native, _tables
 from . import bitexact_predictive_codec as codec
 
 
@@ -47,8 +47,29 @@ def _checkpoints(stream, ctx, freq, vocab, stride):
     return states, offsets, symbols
 
 
-def _read_frame(frame, reference, stride):
-    """Parse, validate and index a frame against its reference words."""
+def _word_image(main):
+    """Bits of a main symbol in the BF16 word: sign, exponent, mantissa bits 6..5
+    (GCR/bitexact_predictive_codec.py:248)."""
+    return ((main & 1024) << 5) | (((main >> 2) & 255) << 7) | ((main & 3) << 5)
+
+
+def _fused_plan(ix, stream, contexts, segment=None):
+    """Segment index, per-label tables and tilings for the tile walker, or FusedUnsupported."""
+    r, c = ix["shape"]
+    if c % 32:
+        raise _fused.FusedUnsupported("row length is not a multiple of 32")
+    seg_len = next((s for s in ([segment] if segment else []) + [64, 128, 32, 256] if s and s % 32 == 0 and c % s == 0), None)
+    if seg_len is None:
+        raise _fused.FusedUnsupported("no segment length divides the row length")
+    states, offsets, _ = _checkpoints(stream, contexts, ix["main_freq"], codec.MAIN_VOCAB, seg_len)
+    return _fused.FramePlan((r, c), 16, 16, ix["labels"], ix["main_freq"], states, offsets, len(stream), seg_len,
+                            image=_word_image)
+
+
+def _read_frame(frame, reference, stride, *, fused=False, fused_segment=None):
+    """Parse, validate and index a frame against its reference words.  With ``fused`` the
+    result also carries ``fused_plan`` (or ``fused_reason``) and keeps the residuals in the
+    packed 5-bit form whatever the frame's mode (``resident_mode`` 0)."""
     if not isinstance(frame, (bytes, bytearray, memoryview)):
         raise codec.CodecError("frame must be bytes")
     info = codec.parse(frame, reference)
@@ -70,14 +91,26 @@ def _read_frame(frame, reference, stride):
     result.update(labels=info["labels"], flips=info["flips"], thresholds=info["thresholds"], main_freq=freq,
                   main_stream=np.frombuffer(info["stream"], dtype=np.uint8).copy(), main_states=states,
                   main_offsets=offsets)
+    result["resident_mode"] = info["mode"]
+    if fused:
+        try:
+            result["fused_plan"] = _fused_plan(result, info["stream"], ctx, fused_segment)
+            result["resident_mode"] = 0
+        except _fused.FusedUnsupported as exc:
+            result["fused_reason"] = str(exc)
     if info["mode"] == 0:
         residual = codec._unpackbits(info["data"], 5, n, "raw5")
         result.update(raw5=np.frombuffer(info["data"], dtype=np.uint8).copy(), residual_symbols=residual)
     else:
         rf = info["residual_freq"].reshape(codec.RES_CONTEXTS, codec.RES_VOCAB)
         rs, ro, residual = _checkpoints(info["residual_stream"], main, rf, codec.RES_VOCAB, stride)
-        result.update(residual_freq=rf, residual_stream=np.frombuffer(info["residual_stream"], dtype=np.uint8).copy(),
-                      residual_states=rs, residual_offsets=ro)
+        if result["resident_mode"] == 0:
+            # the index builder has decoded and validated the residual stream; it stays on the
+            # device as the packed fields the same encoder emits for its mode-0 candidate
+            result.update(raw5=np.frombuffer(codec._packbits(residual, 5), dtype=np.uint8).copy())
+        else:
+            result.update(residual_freq=rf, residual_stream=np.frombuffer(info["residual_stream"], dtype=np.uint8).copy(),
+                          residual_states=rs, residual_offsets=ro)
     if hashlib.sha256(codec.join_symbols(main, residual).tobytes()).digest() != target_hash:
         raise codec.CodecError("target checksum mismatch")
     return result
@@ -86,10 +119,11 @@ def _read_frame(frame, reference, stride):
 class HipPredictiveTensor:
     """A PPCX-coded BF16 matrix resident on one MI355X; decoding needs the reference matrix."""
 
-    def __init__(self, frame, reference_uint16_numpy, stride=1024, device="cuda:0"):
+    def __init__(self, frame, reference_uint16_numpy, stride=1024, device="cuda:0", *, fused=True,
+                 fused_segment=None):
         if not isinstance(stride, int) or not 1 <= stride <= 65536:
             raise codec.CodecError("invalid checkpoint stride")
-        ix = _read_frame(frame, reference_uint16_numpy, stride)
+        ix = _read_frame(frame, reference_uint16_numpy, stride, fused=fused, fused_segment=fused_segment)
         import torch
         if not torch.cuda.is_available():
             raise RuntimeError("a ROCm GPU is required")
@@ -97,12 +131,17 @@ class HipPredictiveTensor:
         self.shape = ix["shape"]
         self.n = math.prod(self.shape)
         self.stride, self.mode = stride, ix["mode"]
+        self.resident_mode = ix.get("resident_mode", self.mode)
+        self._plan = ix.pop("fused_plan", None)
+        self.fused_reason = ix.pop("fused_reason", None)
         self.device = torch.device(device)
         for key in ("source_sha256", "target_sha256", "reference_sha256", "frame_sha256", "frame_bytes"):
             setattr(self, key, ix[key])
         self.buffers = {}
         for name, array in ix.items():
             if isinstance(array, np.ndarray) and name != "residual_symbols":
+                if name in ("raw5", "main_stream"):  # the kernels read whole dwords / 16-byte chunks at the end
+                    array = np.concatenate((array, np.zeros(16, dtype=np.uint8)))
                 self.buffers[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
         for name in ("main", "residual"):
             if name + "_freq" in ix:
@@ -115,12 +154,12 @@ class HipPredictiveTensor:
         if self.mode != 2:
             b = self.buffers
             f = _hip_abi.GrfPpcxFrame()
-            f.main.bytes, f.main.n_bytes = b["main_stream"].data_ptr(), b["main_stream"].numel()
+            f.main.bytes, f.main.n_bytes = b["main_stream"].data_ptr(), b["main_stream"].numel() - 16
             f.main.vocab, f.main.nctx = codec.MAIN_VOCAB, codec.MAIN_CONTEXTS
             f.main.cum, f.main.bucket = b["main_cum"].data_ptr(), b["main_bucket"].data_ptr()
             f.main.states, f.main.offsets = b["main_states"].data_ptr(), b["main_offsets"].data_ptr()
-            if self.mode == 0:
-                f.residual.bytes, f.residual.n_bytes = b["raw5"].data_ptr(), b["raw5"].numel()
+            if self.resident_mode == 0:
+                f.residual.bytes, f.residual.n_bytes = b["raw5"].data_ptr(), b["raw5"].numel() - 16
             else:
                 f.residual.bytes, f.residual.n_bytes = b["residual_stream"].data_ptr(), b["residual_stream"].numel()
                 f.residual.vocab, f.residual.nctx = codec.RES_VOCAB, codec.RES_CONTEXTS
@@ -129,16 +168,74 @@ class HipPredictiveTensor:
                 f.residual.offsets = b["residual_offsets"].data_ptr()
             f.labels, f.flips, f.thresholds = b["labels"].data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr()
             f.rows, f.cols = self.shape
-            f.mode, f.stride = self.mode, stride
+            f.mode, f.stride = self.resident_mode, stride
             self._frame = f
+        self.fused = None
+        if self._plan is not None:
+            try:
+                self._prepare_fused()
+            except _fused.FusedUnsupported as exc:
+                self.fused, self.fused_reason = None, str(exc)
+        self.resident_bytes = int(sum(t.numel() * t.element_size() for t in self.buffers.values()) + 4)
 
-    def decode(self, reference_bf16_device, check=True):
+    def _prepare_fused(self):
+        """Upload the walker's derived arrays: segment index, per-label tables, store tiling."""
+        import torch
+        plan, b = self._plan, self.buffers
+        host = plan.tiling(0)
+        for name, array in (("fused_seg_state", plan.seg_state), ("fused_seg_offset", plan.seg_offset),
+                            ("fused_lut", plan.lut), ("fused_tab", plan.tab.view(np.int64)),
+                            ("fused_tile_rows", host["tile_rows"].view(np.int32)),
+                            ("fused_tile_class", host["tile_class"])):
+            b[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
+        f = _hip_abi.GrfPpcxFused()
+        f.main_bytes, f.raw5 = b["main_stream"].data_ptr(), b["raw5"].data_ptr()
+        f.seg_state, f.seg_offset = b["fused_seg_state"].data_ptr(), b["fused_seg_offset"].data_ptr()
+        f.lut, f.tab = b["fused_lut"].data_ptr(), b["fused_tab"].data_ptr()
+        f.main_n_bytes = b["main_stream"].numel() - 16
+        f.rows, f.cols = self.shape
+        f.n_labels = 16
+        sc = plan.scalars()
+        f.seg_len, f.segs_per_row, f.shift, f.lognb, f.tabn = (sc["seg_len"], sc["segs_per_row"], sc["shift"],
+                                                                sc["lognb"], sc["tabn"])
+        g = _hip_abi.GrfFusedTiling()
+        g.tile_rows, g.tile_class = b["fused_tile_rows"].data_ptr(), b["fused_tile_class"].data_ptr()
+        for key, value in host["scalars"].items():
+            setattr(g, key, value)
+        self.fused, self._tiling = f, g
+        self.fused_plan = dict(sc, **host["scalars"], lds=host["lds"])
+
+    def _status(self, status, check):
+        if status:
+            raise codec.CodecError(f"device decode launch failed ({status}): "
+                                   + self._lib.grf_last_error().decode(errors="replace"))
+        if check and self.error.item():
+            raise codec.CodecError("HIP PPCX checkpoint/context mismatch")
+
+    def decode(self, reference_bf16_device, check=True, *, general=False):
+        """BF16 [rows, cols].  Frames the tile walker supports take two launches (bins of the
+        reference, then the walk); ``general`` forces the one-lane-per-checkpoint kernel."""
         import torch
         if self.mode == 2:
             return self.buffers["raw"].view(torch.bfloat16).reshape(self.shape)
         ref = reference_bf16_device.to(device=self.device).contiguous()
         if tuple(ref.shape) != tuple(self.shape) or ref.dtype != torch.bfloat16:
             raise ValueError("reference device tensor shape/dtype mismatch")
+        if self.fused is not None and not general:
+            bins = torch.empty(self.n // 8, device=self.device, dtype=torch.int32)
+            out = torch.empty(self.shape, device=self.device, dtype=torch.uint16)
+            self.error.zero_()
+            b = self.buffers
+            with torch.cuda.device(self.device):
+                stream = torch.cuda.current_stream(self.device).cuda_stream
+                status = self._lib.grf_ppcx_bins(ref.data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr(),
+                                                 self.shape[0], self.shape[1], bins.data_ptr(), stream)
+                if not status:
+                    status = self._lib.grf_ppcx_fused_decode(ctypes.byref(self.fused), ctypes.byref(self._tiling),
+                                                             bins.data_ptr(), out.data_ptr(), self.error.data_ptr(),
+                                                             stream)
+            self._status(status, check)
+            return out.view(torch.bfloat16)
         count = (self.n + self.stride - 1) // self.stride
         out = torch.empty(count * self.stride, device=self.device, dtype=torch.uint16)
         self.error.zero_()
@@ -146,11 +243,7 @@ class HipPredictiveTensor:
             status = self._lib.grf_ppcx_decode(ctypes.byref(self._frame), ref.data_ptr(), out.data_ptr(),
                                                self.error.data_ptr(),
                                                torch.cuda.current_stream(self.device).cuda_stream)
-        if status:
-            raise codec.CodecError(f"device decode launch failed ({status}): "
-                                   + self._lib.grf_last_error().decode(errors="replace"))
-        if check and self.error.item():
-            raise codec.CodecError("HIP PPCX checkpoint/context mismatch")
+        self._status(status, check)
         return out[:self.n].view(torch.bfloat16).reshape(self.shape)
 
 

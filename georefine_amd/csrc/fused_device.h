@@ -214,8 +214,16 @@ __device__ __forceinline__ void fused_advance(Cursor &c, const StepFetch &s, uin
 // One step (number K of its group of 16) of one segment, for the column class held in byte
 // BYTE of `ccw`.  Returns the image of the symbol's bits in the BF16 word (symbol << 5).
 template <int K>
+__device__ __forceinline__ uint32_t fused_symbol_in(Cursor &c, uint32_t block, const FusedParams &q);
+
+template <int K>
 __device__ __forceinline__ uint32_t fused_symbol(Cursor &c, uint32_t ccw, const FusedParams &q) {
-  const uint32_t block = fused_block_offset<K % 4>(ccw, q.block_pitch);
+  return fused_symbol_in<K>(c, fused_block_offset<K % 4>(ccw, q.block_pitch), q);
+}
+
+// The step given the LDS offset `block` of its context's table block.
+template <int K>
+__device__ __forceinline__ uint32_t fused_symbol_in(Cursor &c, uint32_t block, const FusedParams &q) {
   StepFetch s;
   const uint32_t idx = fused_fetch_index(c.state, block, q);
   fused_fetch_bytes<K>(s, c);

@@ -1,0 +1,259 @@
+// Fused decode of PPCX frames: the tile walker of the context codec with the predictive
+// symbol model.
+//
+// A PPCX main symbol is coded in the context (row label, bin of the reference word at the
+// same position) -- GCR/bitexact_predictive_codec.py:179-186, device form
+// GCR/bitexact_predictive_gpu_kernels.py:24-58.  The row label takes the part of the row
+// class (a tile holds rows of one label, so 16 bin contexts are live and their tables fit in
+// LDS); the bin takes the part of the column class, but differs per element.  It is computed
+// from the dense reference words by a separate elementwise kernel into a transient plane of
+// 4-bit bins, which the walker then reads like column classes: 8 bytes per 16 symbols.
+// Doing the threshold search inside the walk would add ~12 instructions to a 25-instruction
+// step; the plane costs one pass over the reference at memory speed.
+//
+// Residuals are the packed 5-bit fields of the frame (GCR/bitexact_predictive_codec.py:145-166,
+// MSB first): 10 bytes per 16 symbols, so every second group starts half a dword in.
+#include <hip/hip_runtime.h>
+
+#include <string>
+
+#include "fused_device.h"
+
+namespace grf {
+int set_error(int code, const std::string &what);                                                  // decode_general.hip
+int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who);  // fused_gemv.hip
+}
+
+namespace {
+
+using grf::FusedLdsLayout;
+
+// ---- bins plane ----
+
+// A workgroup first tabulates the bin of all 65 536 sign-aligned words in LDS (64 KiB, one
+// byte each; 64 entries per thread), then streams its share of the matrix through the
+// table: per element one xor with the row's flip, one LDS byte read and one shift-or.
+// 16 elements per thread and pass: 32 bytes of reference words in, two dwords of eight
+// 4-bit bins out (element i of the matrix in bits 4*(i%8) of dword i/8).
+constexpr uint32_t kBinsThreads = 1024;
+
+__global__ __launch_bounds__(kBinsThreads) void ppcx_bins_kernel(const uint16_t *reference, const uint8_t *flips,
+                                                                  const uint16_t *thresholds, uint32_t cols,
+                                                                  uint64_t n, uint32_t *bins) {
+  extern __shared__ __align__(16) uint8_t table[];  // bin of the sign-aligned word
+  __shared__ uint16_t th[16];
+  if (threadIdx.x < 15) th[threadIdx.x] = thresholds[threadIdx.x];
+  __syncthreads();
+  for (uint32_t a = threadIdx.x * 4; a < 65536; a += kBinsThreads * 4) {
+    uint32_t four = 0;
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) four |= grf::threshold_bin(th, grf::ordinal_key(a + i, 0)) << (8 * i);
+    *reinterpret_cast<uint32_t *>(table + a) = four;
+  }
+  __syncthreads();
+  const uint64_t stride = (uint64_t)gridDim.x * kBinsThreads * 16;
+  for (uint64_t first = ((uint64_t)blockIdx.x * kBinsThreads + threadIdx.x) * 16; first < n; first += stride) {
+    const uint4 *src = reinterpret_cast<const uint4 *>(reference + first);  // cols % 16 == 0: one row
+    const uint4 ra = src[0], rb = src[1];
+    const uint32_t flip = flips[first / cols] ? 0x80008000u : 0u;
+    const uint32_t w[8] = {ra.x ^ flip, ra.y ^ flip, ra.z ^ flip, ra.w ^ flip,
+                           rb.x ^ flip, rb.y ^ flip, rb.z ^ flip, rb.w ^ flip};
+    uint32_t packed[2] = {0, 0};
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const uint32_t a = (i % 2) ? (w[i / 2] >> 16) : (w[i / 2] & 0xFFFFu);
+      packed[i / 8] |= (uint32_t)table[a] << (4 * (i % 8));
+    }
+    *reinterpret_cast<uint2 *>(bins + first / 8) = make_uint2(packed[0], packed[1]);
+  }
+}
+
+// ---- walker ----
+
+// Sixteen packed 5-bit residuals: 80 bits that start `lead` bits (0 or 16) into three
+// big-endian dwords.
+struct Raw5x16 {
+  uint32_t w0, w1, w2;  // the 80 bits left-aligned in w0:w1:w2
+  __device__ __forceinline__ void set(uint32_t a, uint32_t b, uint32_t c, uint32_t lead) {
+    a = __builtin_bswap32(a);
+    b = __builtin_bswap32(b);
+    c = __builtin_bswap32(c);
+    // shift the 96-bit string left by lead (alignbit shifts a 64-bit pair right by 32 - lead)
+    w0 = lead ? __builtin_amdgcn_alignbit(a, b, 32 - lead) : a;
+    w1 = lead ? __builtin_amdgcn_alignbit(b, c, 32 - lead) : b;
+    w2 = lead ? c << lead : c;
+  }
+  template <int K>
+  __device__ __forceinline__ uint32_t field() const {
+    constexpr int bit = K * 5, word = bit / 32, off = bit % 32;
+    const uint32_t a = word == 0 ? w0 : (word == 1 ? w1 : w2);
+    if constexpr (off + 5 <= 32) {
+      return __builtin_amdgcn_ubfe(a, 32 - 5 - off, 5);
+    } else {
+      const uint32_t b = word == 0 ? w1 : w2;
+      return __builtin_amdgcn_ubfe(__builtin_amdgcn_alignbit(a, b, 64 - 5 - off), 0, 5);
+    }
+  }
+};
+
+struct PpcxWalk {
+  grf::Cursor c;
+  uint32_t ip0, gofs, seg;
+  const uint8_t *rawp;    // the segment's first residual byte (5 * S / 8 bytes per segment)
+  const uint2 *binp;      // the segment's bins, 8 bytes per 16 symbols
+  uint32_t n0, n1, n2;
+  uint2 nb;
+
+  __device__ __forceinline__ static const uint32_t *group_dwords(const uint8_t *rawp, uint32_t g) {
+    return reinterpret_cast<const uint32_t *>(rawp + ((10 * g) & ~3u));
+  }
+  __device__ __forceinline__ void open(const grf_bctx_fused &f, uint32_t seg_, uint32_t piece_off, uint32_t a0,
+                                       uint64_t elem0) {
+    seg = seg_;
+    gofs = f.seg_offset[seg];
+    ip0 = piece_off + (gofs - a0);
+    c.open(f.seg_state[seg], ip0);
+    rawp = f.raw6 + elem0 / 8 * 5;
+    binp = reinterpret_cast<const uint2 *>(f.col_class) + elem0 / 16;
+    const uint32_t *d = group_dwords(rawp, 0);
+    n0 = d[0];
+    n1 = d[1];
+    n2 = d[2];
+    nb = binp[0];
+  }
+
+  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const grf::FusedParams &q, uint32_t (&pair)[8]) {
+    Raw5x16 rr;
+    rr.set(n0, n1, n2, (t & 16u) ? 16u : 0u);
+    const uint32_t bw[2] = {nb.x, nb.y};
+    {  // the last group loads itself again rather than branch around the loads
+      const uint32_t next = min(t / 16 + 1, S / 16 - 1);
+      const uint32_t *d = group_dwords(rawp, next);
+      n0 = d[0];
+      n1 = d[1];
+      n2 = d[2];
+      nb = binp[next];
+    }
+    uint32_t bits[16];
+#define GRF_STEP(k)                                                                                   \
+  {                                                                                                   \
+    const uint32_t bin = __builtin_amdgcn_ubfe(bw[(k) / 8], 4 * ((k) % 8), 4);                        \
+    const uint32_t hi = grf::fused_symbol_in<k>(c, __umul24(bin, q.block_pitch), q);                  \
+    bits[k] = hi | rr.field<k>();                                                                     \
+  }
+    GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
+    GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
+#undef GRF_STEP
+    c.end_group();
+#pragma unroll
+    for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
+  }
+
+  __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
+    return c.state == f.seg_state[seg + 1] && gofs + (c.j - ip0) == f.seg_offset[seg + 1];
+  }
+};
+
+// `f` carries the PPCX frame in the walker's frame structure: raw6 = packed 5-bit
+// residuals, col_class = the bins plane, nr = labels, nc = 16 bins.
+__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_ppcx_kernel(grf_bctx_fused f, grf_fused_tiling g,
+                                                                            uint16_t *out, int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const FusedLdsLayout L(f, g, 0);
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
+  const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
+  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, g.tile_class[tile], tid, nthreads);
+  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
+  const uint32_t r = tid / P, p = tid % P;
+  const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
+  uint32_t bad = 0;
+  for (uint32_t b = 0; b < g.n_slabs; ++b) {
+    if (b) __syncthreads();  // everyone is done with the previous slab's stream bytes
+    const uint32_t first_seg = b * P;
+    const uint32_t nseg = min(P, f.segs_per_row - first_seg);
+    uint32_t a0 = 0, seg_base = 0;
+    const uint32_t piece_off = L.stream + r * g.piece_cap;
+    if (row != grf::kNoRow) {
+      seg_base = row * f.segs_per_row + first_seg;
+      a0 = grf::fused_stage_piece(lds, piece_off, f, seg_base, nseg, p, P);
+    }
+    __syncthreads();
+    if (row != grf::kNoRow && p < nseg) {
+      const uint64_t elem0 = (uint64_t)row * K + (uint64_t)(first_seg + p) * S;
+      PpcxWalk w;
+      w.open(f, seg_base + p, piece_off, a0, elem0);
+      for (uint32_t t = 0; t < S; t += 16) {
+        uint32_t pair[8];
+        w.decode16(t, S, q, pair);
+        uint4 *dst = reinterpret_cast<uint4 *>(out + elem0 + t);
+        dst[0] = make_uint4(pair[0], pair[1], pair[2], pair[3]);
+        dst[1] = make_uint4(pair[4], pair[5], pair[6], pair[7]);
+      }
+      if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
+    }
+  }
+  if (bad) atomicOr(error, (int)bad);
+}
+
+}  // namespace
+
+extern "C" {
+
+int grf_ppcx_bins(const uint16_t *reference, const uint8_t *flips, const uint16_t *thresholds, uint32_t rows,
+                  uint32_t cols, uint32_t *bins, void *hip_stream) {
+  if (!reference || !flips || !thresholds || !bins)
+    return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_bins: null argument");
+  if (!rows || !cols || cols % 16 || ((uintptr_t)reference & 15) || ((uintptr_t)bins & 7))
+    return grf::set_error(GRF_BAD_ARGUMENT,
+                          "grf_ppcx_bins: row length must be a multiple of 16, reference 16-byte and bins 8-byte aligned");
+  const uint64_t n = (uint64_t)rows * cols;
+  if (n > 0xFFFFFFFFull) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_bins: matrix too large");
+  const uint64_t chunks = (n / 16 + kBinsThreads - 1) / kBinsThreads;
+  const uint32_t blocks = (uint32_t)(chunks < 512 ? chunks : 512);  // two workgroups per CU amortise the table
+  hipLaunchKernelGGL(ppcx_bins_kernel, dim3(blocks), dim3(kBinsThreads), 65536, (hipStream_t)hip_stream, reference,
+                     flips, thresholds, cols, n, bins);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("bins kernel: ") + hipGetErrorString(e));
+  return GRF_OK;
+}
+
+int grf_ppcx_fused_decode(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins,
+                          uint16_t *out, int32_t *error, void *hip_stream) {
+  if (!frame || !tiling || !bins || !out || !error)
+    return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_fused_decode: null argument");
+  grf_bctx_fused f{};
+  f.main_bytes = frame->main_bytes;
+  f.raw6 = frame->raw5;
+  f.seg_state = frame->seg_state;
+  f.seg_offset = frame->seg_offset;
+  f.lut = frame->lut;
+  f.tab = frame->tab;
+  f.col_class = reinterpret_cast<const uint8_t *>(bins);
+  f.main_n_bytes = frame->main_n_bytes;
+  f.rows = frame->rows;
+  f.cols = frame->cols;
+  f.nr = frame->n_labels;
+  f.nc = 16;
+  f.seg_len = frame->seg_len;
+  f.segs_per_row = frame->segs_per_row;
+  f.shift = frame->shift;
+  f.lognb = frame->lognb;
+  f.tabn = frame->tabn;
+  if (int rc = grf::check_fused_frame(f, *tiling, "grf_ppcx_fused_decode")) return rc;
+  if (f.seg_len % 32)  // a segment's residual bytes must start on a dword
+    return grf::set_error(GRF_UNSUPPORTED, "grf_ppcx_fused_decode: segment length must be a multiple of 32");
+  const FusedLdsLayout L(f, *tiling, 0);
+  if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
+  if (L.total > 64 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(fused_ppcx_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
+    if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("LDS attribute: ") + hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(fused_ppcx_kernel, dim3(tiling->n_tiles), dim3(tiling->threads), L.total,
+                     (hipStream_t)hip_stream, f, *tiling, out, error);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
+  return GRF_OK;
+}
+
+}  // extern "C"

@@ -223,6 +223,44 @@ uint32_t grf_bctx_gemm_lds_bytes(const grf_bctx_fused *frame, const grf_fused_ti
 /* LDS bytes a launch needs for the given m_rows (0 for the store sink). */
 uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint32_t m_rows);
 
+/* PPCX frame prepared for the tile walker (modes 0 and 1 with the residuals resident as the
+ * frame's packed 5-bit form; GCR/bitexact_predictive_codec.py:145-166, 179-186).  The row
+ * label plays the part of the row class, the reference-word bin that of the column class:
+ *   main_bytes  the frame's main rANS stream, readable for 16 bytes past main_n_bytes
+ *   raw5        packed 5-bit residuals, MSB first, readable for 16 bytes past the end
+ *   seg_state / seg_offset  as in grf_bctx_fused, contexts label[row]*16 + bin
+ *   lut  u8 [n_labels][16 << lognb], tab u64 [n_labels][16][tabn+1]   as in grf_bctx_fused,
+ *        entry high32 = the symbol's bits in the BF16 word (sign, exponent, mantissa 6..5)
+ * seg_len must be a multiple of 32.  Tilings are built over row labels. */
+typedef struct grf_ppcx_fused {
+  const uint8_t *main_bytes;
+  const uint8_t *raw5;
+  const uint32_t *seg_state;
+  const uint32_t *seg_offset;
+  const uint8_t *lut;
+  const uint64_t *tab;
+  uint32_t main_n_bytes;
+  uint32_t rows, cols;
+  uint32_t n_labels;
+  uint32_t seg_len, segs_per_row;
+  uint32_t shift, lognb, tabn;
+} grf_ppcx_fused;
+
+/* The bin of every reference word (GCR/bitexact_predictive_codec.py:106-110, device form
+ * GCR/bitexact_predictive_gpu_kernels.py:36-42: sign alignment by the row's flip, ordinal
+ * key, number of thresholds <= key), packed 4 bits per element: element i in bits
+ * 4*(i%8) of bins[i/8].  reference: BF16 [rows][cols] dense, 16-byte aligned, cols % 16 == 0;
+ * flips u8 [rows]; thresholds u16 [15]; bins u32 [rows*cols/8]. */
+int grf_ppcx_bins(const uint16_t *reference, const uint8_t *flips, const uint16_t *thresholds, uint32_t rows,
+                  uint32_t cols, uint32_t *bins, void *hip_stream);
+
+/* Decode a prepared PPCX frame to dense BF16 words given the bins of its reference (replaces
+ * the Triton launch of CudaPredictiveTensor.decode, GCR/bitexact_predictive_gpu.py:160-174,
+ * for frames that meet the walker's limits).  A reference that is not the one the frame was
+ * coded against makes segments miss their checkpoints: GRF_ERR_CHECKPOINT in *error. */
+int grf_ppcx_fused_decode(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins,
+                          uint16_t *out, int32_t *error, void *hip_stream);
+
 const char *grf_last_error(void);
 int grf_abi_version(void);
 

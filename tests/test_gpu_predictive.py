@@ -58,9 +58,36 @@ def test_ppcx_decode_matches_oracle(oracle, name, target, ref, mode, stride):
     ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
     got = t.decode(ref_dev).view(torch.uint16).cpu().numpy()
     assert np.array_equal(got, expect)
+    if mode != 2 and target.shape[1] % 32 == 0:
+        assert t.fused is not None, t.fused_reason   # decode() above ran the tile walker
+        assert t.resident_mode == 0
+        assert np.array_equal(t.decode(ref_dev, general=True).view(torch.uint16).cpu().numpy(), expect)
+    else:
+        assert t.fused is None
     assert t.frame_sha256 == hashlib.sha256(frame).hexdigest()
     assert t.source_sha256 == hashlib.sha256(target.tobytes()).hexdigest()
     assert isinstance(t.resident_bytes, int) and t.resident_bytes > 0
+
+
+@pytest.mark.parametrize("segment", [32, 64, 128, 256])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_ppcx_tile_walker_every_segment_length(oracle, segment, mode):
+    import torch
+    from georefine_amd import bitexact_predictive_codec as codec
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
+    rng = np.random.default_rng(segment + mode)
+    target = weight_like(rng, 150, 768)
+    tf = (target.astype(np.uint32) << 16).view(np.float32)
+    ref = bf16_words(tf * rng.choice([-1.0, 1.0], size=(150, 1)).astype(np.float32)
+                     + rng.normal(0, 0.003, target.shape).astype(np.float32))  # some rows sign-flipped
+    frame = _frame_for_mode(codec, target, ref, mode)
+    t = HipPredictiveTensor(frame, ref, stride=1024, device="cuda:0", fused_segment=segment)
+    assert t.fused is not None and t.fused_plan["seg_len"] == segment
+    ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
+    assert np.array_equal(t.decode(ref_dev).view(torch.uint16).cpu().numpy(), target)
+    unfused = HipPredictiveTensor(frame, ref, stride=1024, device="cuda:0", fused=False)
+    assert unfused.fused is None and unfused.resident_mode == mode
+    assert np.array_equal(unfused.decode(ref_dev).view(torch.uint16).cpu().numpy(), target)
 
 
 def test_ppcx_wrong_reference_on_device_sets_error(oracle):
@@ -70,8 +97,11 @@ def test_ppcx_wrong_reference_on_device_sets_error(oracle):
     _, target, ref = next(_pairs())
     t = HipPredictiveTensor(_frame_for_mode(codec, target, ref, 0), ref, stride=64)
     other = torch.from_numpy(np.roll(ref, 3, axis=1).copy()).view(torch.bfloat16).cuda()
+    assert t.fused is not None
     with pytest.raises(codec.CodecError):  # contexts differ: segments miss their checkpoints
         t.decode(other)
+    with pytest.raises(codec.CodecError):
+        t.decode(other, general=True)
     with pytest.raises(ValueError):
         t.decode(other[:, :8])
 
