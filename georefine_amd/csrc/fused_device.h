@@ -148,6 +148,13 @@ __device__ __forceinline__ void fused_fetch_bytes(StepFetch &s, const Cursor &c)
   // byte of either register is looked at)
   s.bytes = __builtin_amdgcn_perm(lds_load_u8(c.j + 2 * K), lds_load_u8(c.j + 2 * K + 1), 0x0c0c0400u);
 }
+// Keeps the combination of the two bytes in the block that loaded them: left alone, the
+// compiler sinks it past the scan branch and then re-masks both bytes there.
+__device__ __forceinline__ void fused_pin_bytes(StepFetch &s) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(s.bytes));
+#endif
+}
 __device__ __forceinline__ void fused_fetch_entry(StepFetch &s, uint32_t idx, uint32_t block) {
   s.ta = fused_lshl3_add(idx, block);
   s.e0 = *reinterpret_cast<lds_v2u32 *>(s.ta);
@@ -228,6 +235,7 @@ __device__ __forceinline__ uint32_t fused_symbol_in(Cursor &c, uint32_t block, c
   const uint32_t idx = fused_fetch_index(c.state, block, q);
   fused_fetch_bytes<K>(s, c);
   fused_fetch_entry(s, idx, block);
+  fused_pin_bytes(s);
   uint64_t miss;
   uint32_t rel = fused_locate(c.state, s.e0.x, miss);
   if (__builtin_expect(fused_lane_in(miss), 0)) fused_scan(c.state, s, rel);
@@ -235,7 +243,8 @@ __device__ __forceinline__ uint32_t fused_symbol_in(Cursor &c, uint32_t block, c
   return s.e0.y;
 }
 
-// Sixteen packed 6-bit residuals (12 bytes, MSB first) -> field k, k compile-time.
+// Sixteen packed 6-bit residuals (12 bytes, MSB first) -> field k, k compile-time, sign
+// extended: bits 0..4 are the mantissa's low bits, every bit from 5 up copies the sign.
 struct Raw6x16 {
   uint32_t w0, w1, w2;  // big-endian dwords
   __device__ __forceinline__ void set(uint32_t a, uint32_t b, uint32_t c) {
@@ -249,10 +258,10 @@ struct Raw6x16 {
     constexpr int word = bit / 32, off = bit % 32;
     const uint32_t a = word == 0 ? w0 : (word == 1 ? w1 : w2);
     if constexpr (off + 6 <= 32) {
-      return __builtin_amdgcn_ubfe(a, 32 - 6 - off, 6);
+      return (uint32_t)__builtin_amdgcn_sbfe((int32_t)a, 32 - 6 - off, 6);
     } else {
       const uint32_t b = word == 0 ? w1 : w2;
-      return __builtin_amdgcn_ubfe(__builtin_amdgcn_alignbit(a, b, 64 - 6 - off), 0, 6);
+      return (uint32_t)__builtin_amdgcn_sbfe((int32_t)__builtin_amdgcn_alignbit(a, b, 64 - 6 - off), 0, 6);
     }
   }
 };
@@ -274,23 +283,33 @@ __device__ __forceinline__ void fused_load_tables(uint8_t *lds, uint32_t blocks,
   }
 }
 
-// Copy the main-stream bytes of one row piece (segments [seg_base, seg_base+nseg)) to LDS
-// at piece_off, keeping the 16-byte phase of the global address.  The P lanes of the row
-// share the copy.  Returns the aligned global start so lanes can place their cursors.
+// Byte range of one row piece (segments [seg_base, seg_base+nseg)) in the main stream.  The
+// kernels fetch it one slab ahead: it is the first of two dependent global reads before a
+// slab's bytes can be copied.
+struct PieceSpan {
+  uint32_t g0, g1;
+  __device__ __forceinline__ void fetch(const grf_bctx_fused &f, uint32_t seg_base, uint32_t nseg) {
+    g0 = f.seg_offset[seg_base];
+    g1 = f.seg_offset[seg_base + nseg];
+  }
+};
+
+// Copy the main-stream bytes of one row piece to LDS at piece_off, keeping the 16-byte
+// phase of the global address.  The P lanes of the row share the copy.  Returns the
+// aligned global start so lanes can place their cursors.
 __device__ __forceinline__ uint32_t fused_stage_piece(uint8_t *lds, uint32_t piece_off, const grf_bctx_fused &f,
-                                                      uint32_t seg_base, uint32_t nseg, uint32_t p, uint32_t P) {
-  const uint32_t g0 = f.seg_offset[seg_base], g1 = f.seg_offset[seg_base + nseg];
-  const uint32_t a0 = g0 & ~15u;
-  for (uint32_t o = a0 + p * 16; o < g1; o += P * 16)
+                                                      const PieceSpan &span, uint32_t p, uint32_t P) {
+  const uint32_t a0 = span.g0 & ~15u;
+  for (uint32_t o = a0 + p * 16; o < span.g1; o += P * 16)
     *reinterpret_cast<uint4 *>(lds + piece_off + (o - a0)) = *reinterpret_cast<const uint4 *>(f.main_bytes + o);
   return a0;
 }
 
 // BF16 word in bits 0..15 (bits above are unspecified): symbol bits | mantissa low 5 bits
-// | sign << 15.  r6 * (1 + 2^10) puts the five mantissa bits at 0..4 and the sign at 15
-// (a 24-bit multiply); the mask drops the copies that land elsewhere.
-__device__ __forceinline__ uint32_t fused_word_bits(uint32_t hi, uint32_t r6) {
-  return ((r6 * 0x401u) & 0x801Fu) | hi;
+// | sign << 15, from the sign-extended residual field: its copy of the sign at bit 15 and
+// its low five bits are kept, one and-or.
+__device__ __forceinline__ uint32_t fused_word_bits(uint32_t hi, uint32_t r6_sign_extended) {
+  return (r6_sign_extended & 0x801Fu) | hi;
 }
 
 // A lane's walk over one segment: rANS cursor, plus the registers that hold the packed
@@ -303,20 +322,23 @@ struct SegmentWalk {
   uint32_t n0, n1, n2;
   uint4 nc4;
 
-  // walks segment `seg_`, whose row piece was staged at piece_off from global offset a0;
-  // elem0 / col0: the segment's first element / column
-  __device__ __forceinline__ void open(const grf_bctx_fused &f, uint32_t seg_, uint32_t piece_off, uint32_t a0,
-                                       uint64_t elem0, uint32_t col0) {
+  // Global reads for segment `seg_` (elem0 / col0: its first element / column), issued
+  // before the workgroup waits for the slab's stream bytes so that their latency overlaps it.
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t col0) {
     seg = seg_;
     gofs = f.seg_offset[seg];
-    ip0 = piece_off + (gofs - a0);
-    c.open(f.seg_state[seg], ip0);
+    c.state = f.seg_state[seg];
     rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
     ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
     n0 = rawp[0];
     n1 = rawp[1];
     n2 = rawp[2];
     nc4 = ccp[0];
+  }
+  // the row piece was staged at piece_off from global offset a0
+  __device__ __forceinline__ void start(uint32_t piece_off, uint32_t a0) {
+    ip0 = piece_off + (gofs - a0);
+    c.j = ip0;
   }
 
   // Decode symbols [t, t+16) of the segment into eight BF16 pairs (word k in the low half,

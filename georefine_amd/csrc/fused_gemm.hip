@@ -86,23 +86,26 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
   for (uint32_t j = 0; j < kMaxAcc; ++j) acc[j] = (float4v){0.f, 0.f, 0.f, 0.f};
   uint32_t bad = 0;
 
+  grf::PieceSpan span{0, 0};
+  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
     __syncthreads();  // previous slab's stream bytes and tiles are no longer read
     const uint32_t first_seg = b * P;
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
-    uint32_t a0 = 0, seg_base = 0;
     const uint32_t piece_off = L.stream + r * g.piece_cap;
+    const bool active = row != grf::kNoRow && p < nseg;
+    const uint32_t seg_base = row != grf::kNoRow ? row * f.segs_per_row + first_seg : 0;
+    const uint32_t col0 = (first_seg + p) * S;
+    grf::SegmentWalk w;
+    uint32_t a0 = 0;
+    if (active) w.prefetch(f, seg_base + p, (uint64_t)row * K + col0, col0);
     if (row != grf::kNoRow) {
-      seg_base = row * f.segs_per_row + first_seg;
-      a0 = grf::fused_stage_piece(lds, piece_off, f, seg_base, nseg, p, P);
+      a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
+      if (b + 1 < g.n_slabs)  // the next slab's byte range, while this one is walked
+        span.fetch(f, seg_base + P, min(P, f.segs_per_row - first_seg - P));
     }
     __syncthreads();
-    const bool active = row != grf::kNoRow && p < nseg;
-    grf::SegmentWalk w;
-    if (active) {
-      const uint32_t col0 = (first_seg + p) * S;
-      w.open(f, seg_base + p, piece_off, a0, (uint64_t)row * K + col0, col0);
-    }
+    if (active) w.start(piece_off, a0);
     for (uint32_t t = 0; t < S; t += kGroup) {
       if (active) {  // 16 words of this lane's segment -> word tile
         uint32_t pair[8];

@@ -62,6 +62,8 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   float *rowsum = reinterpret_cast<float *>(lds + L.rowsum);  // [R][M] running sums
   uint32_t bad = 0;
 
+  grf::PieceSpan span{0, 0};
+  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
     if (b) __syncthreads();  // everyone is done with the previous slab's LDS data
     const uint32_t col_base = b * width;
@@ -76,18 +78,22 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
     }
     const uint32_t first_seg = b * P;
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
-    uint32_t a0 = 0, seg_base = 0;
     const uint32_t piece_off = L.stream + r * g.piece_cap;
+    const bool walks = row != grf::kNoRow && p < nseg;
+    const uint32_t seg_base = row != grf::kNoRow ? row * f.segs_per_row + first_seg : 0;
+    const uint32_t col0 = (first_seg + p) * S;
+    const uint64_t elem0 = (uint64_t)row * K + col0;
+    grf::SegmentWalk w;
+    uint32_t a0 = 0;
+    if (walks) w.prefetch(f, seg_base + p, elem0, col0);
     if (row != grf::kNoRow) {
-      seg_base = row * f.segs_per_row + first_seg;
-      a0 = grf::fused_stage_piece(lds, piece_off, f, seg_base, nseg, p, P);
+      a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
+      if (b + 1 < g.n_slabs)  // the next slab's byte range, while this one is walked
+        span.fetch(f, seg_base + P, min(P, f.segs_per_row - first_seg - P));
     }
     __syncthreads();
-    if (row != grf::kNoRow && p < nseg) {
-      const uint32_t col0 = (first_seg + p) * S;
-      const uint64_t elem0 = (uint64_t)row * K + col0;
-      grf::SegmentWalk w;
-      w.open(f, seg_base + p, piece_off, a0, elem0, col0);
+    if (walks) {
+      w.start(piece_off, a0);
       const uint16_t *xr = xs + p * xpitch;
       float acc[M];
 #pragma unroll

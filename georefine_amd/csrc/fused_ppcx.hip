@@ -107,12 +107,11 @@ struct PpcxWalk {
   __device__ __forceinline__ static const uint32_t *group_dwords(const uint8_t *rawp, uint32_t g) {
     return reinterpret_cast<const uint32_t *>(rawp + ((10 * g) & ~3u));
   }
-  __device__ __forceinline__ void open(const grf_bctx_fused &f, uint32_t seg_, uint32_t piece_off, uint32_t a0,
-                                       uint64_t elem0) {
+  // global reads of the segment, issued before the wait for the slab's stream bytes
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0) {
     seg = seg_;
     gofs = f.seg_offset[seg];
-    ip0 = piece_off + (gofs - a0);
-    c.open(f.seg_state[seg], ip0);
+    c.state = f.seg_state[seg];
     rawp = f.raw6 + elem0 / 8 * 5;
     binp = reinterpret_cast<const uint2 *>(f.col_class) + elem0 / 16;
     const uint32_t *d = group_dwords(rawp, 0);
@@ -120,6 +119,10 @@ struct PpcxWalk {
     n1 = d[1];
     n2 = d[2];
     nb = binp[0];
+  }
+  __device__ __forceinline__ void start(uint32_t piece_off, uint32_t a0) {
+    ip0 = piece_off + (gofs - a0);
+    c.j = ip0;
   }
 
   __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const grf::FusedParams &q, uint32_t (&pair)[8]) {
@@ -167,21 +170,26 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_ppcx_kernel(grf_b
   const uint32_t r = tid / P, p = tid % P;
   const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
   uint32_t bad = 0;
+  grf::PieceSpan span{0, 0};
+  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
     if (b) __syncthreads();  // everyone is done with the previous slab's stream bytes
     const uint32_t first_seg = b * P;
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
-    uint32_t a0 = 0, seg_base = 0;
     const uint32_t piece_off = L.stream + r * g.piece_cap;
+    const bool walks = row != grf::kNoRow && p < nseg;
+    const uint32_t seg_base = row != grf::kNoRow ? row * f.segs_per_row + first_seg : 0;
+    const uint64_t elem0 = (uint64_t)row * K + (uint64_t)(first_seg + p) * S;
+    PpcxWalk w;
+    uint32_t a0 = 0;
+    if (walks) w.prefetch(f, seg_base + p, elem0);
     if (row != grf::kNoRow) {
-      seg_base = row * f.segs_per_row + first_seg;
-      a0 = grf::fused_stage_piece(lds, piece_off, f, seg_base, nseg, p, P);
+      a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
+      if (b + 1 < g.n_slabs) span.fetch(f, seg_base + P, min(P, f.segs_per_row - first_seg - P));
     }
     __syncthreads();
-    if (row != grf::kNoRow && p < nseg) {
-      const uint64_t elem0 = (uint64_t)row * K + (uint64_t)(first_seg + p) * S;
-      PpcxWalk w;
-      w.open(f, seg_base + p, piece_off, a0, elem0);
+    if (walks) {
+      w.start(piece_off, a0);
       for (uint32_t t = 0; t < S; t += 16) {
         uint32_t pair[8];
         w.decode16(t, S, q, pair);
