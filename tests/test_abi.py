@@ -38,7 +38,8 @@ def test_device_library_reports_its_abi_version_without_a_gpu():
 def test_struct_mirrors_match_the_header_field_order():
     text = (ROOT / "include/georefine_amd.h").read_text()
     for struct_name, mirror in (("grf_bctx_fused", _hip_abi.GrfBctxFused), ("grf_fused_tiling", _hip_abi.GrfFusedTiling),
-                                ("grf_stream", _hip_abi.GrfStream)):
+                                ("grf_stream", _hip_abi.GrfStream), ("grf_ppcx_fused", _hip_abi.GrfPpcxFused),
+                                ("grf_bctx_frame", _hip_abi.GrfBctxFrame), ("grf_ppcx_frame", _hip_abi.GrfPpcxFrame)):
         body = re.search(r"typedef struct " + struct_name + r" \{(.*?)\} " + struct_name + ";", text, flags=re.S).group(1)
         body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
         fields = []
