@@ -300,8 +300,12 @@ struct PieceSpan {
 __device__ __forceinline__ uint32_t fused_stage_piece(uint8_t *lds, uint32_t piece_off, const grf_bctx_fused &f,
                                                       const PieceSpan &span, uint32_t p, uint32_t P) {
   const uint32_t a0 = span.g0 & ~15u;
+  // read once: a streaming load, so that these bytes do not push the residual lines, which
+  // a lane touches four times over a segment, out of the L2
+  typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
   for (uint32_t o = a0 + p * 16; o < span.g1; o += P * 16)
-    *reinterpret_cast<uint4 *>(lds + piece_off + (o - a0)) = *reinterpret_cast<const uint4 *>(f.main_bytes + o);
+    *reinterpret_cast<u32x4 *>(lds + piece_off + (o - a0)) =
+        __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(f.main_bytes + o));
   return a0;
 }
 
