@@ -95,3 +95,56 @@ def test_unsupported_frames_are_reported():
         with pytest.raises(_fused.FusedUnsupported):
             _fused.FramePlan(ix["shape"], ix["nr"], ix["nc"], ix["rows"], ix["main_freq"], ix["fused_states"],
                              ix["fused_offsets"], len(ix["main_stream"]), 64)
+
+
+def test_predictive_plan_walks_to_the_target_words():
+    """The tile walker's host data for a PPCX frame, replayed on the CPU: from every segment's
+    checkpoint, bucket lookup -> entry scan -> state update -> byte refill must reproduce the
+    target's main symbols (as their image in the BF16 word) and land on the next checkpoint."""
+    from georefine_amd import bitexact_predictive_codec as ppcx
+    from georefine_amd.bitexact_predictive_gpu import _read_frame, _word_image
+    rng = np.random.default_rng(9)
+    target = weight_like(rng, 64, 256)
+    tf = (target.astype(np.uint32) << 16).view(np.float32)
+    ref = bf16_words(tf * rng.choice([-1.0, 1.0], size=(64, 1)).astype(np.float32)
+                     + rng.normal(0, 0.003, target.shape).astype(np.float32))
+    frame = ppcx.encode(target, ref)
+    ix = _read_frame(frame, ref, 1024, fused=True, fused_segment=32)
+    assert ix["mode"] in (0, 1), "the sample must be large enough for an entropy-coded frame"
+    plan = ix["fused_plan"]
+    assert ix["resident_mode"] == 0 and plan.seg_len == 32 and plan.nc == 16 and plan.nr == 16
+    # packed residual fields are the frame's own form
+    main, residual = ppcx.split_symbols(target)
+    assert np.array_equal(np.frombuffer(ppcx._packbits(residual.ravel(), 5), dtype=np.uint8), ix["raw5"])
+    ctx = ppcx.contexts(ref, ix["labels"], ix["flips"], ix["thresholds"]).reshape(target.shape)
+    stream = ix["main_stream"]
+    spr = plan.spr
+    for row in range(target.shape[0]):
+        label = int(ix["labels"][row])
+        for seg in range(spr):
+            k = row * spr + seg
+            state, ip = int(plan.seg_state[k]), int(plan.seg_offset[k])
+            for t in range(plan.seg_len):
+                col = seg * plan.seg_len + t
+                c = int(ctx[row, col])
+                assert c // 16 == label
+                sym_image, start, freq = emulate_lookup(plan, label, c % 16, np.array([state & 0xFFFF]))
+                assert (sym_image[0] << 5) == _word_image(int(main[row, col]))
+                state = int(freq[0]) * (state >> 16) + (state & 0xFFFF) - int(start[0])
+                while state < (1 << 23):
+                    state = (state << 8) | int(stream[ip])
+                    ip += 1
+            assert state == int(plan.seg_state[k + 1]) and ip == int(plan.seg_offset[k + 1])
+    tiling = plan.tiling(0)
+    assert tiling["lds"] <= _fused.MAX_LDS
+    assert ix.get("fused_reason") is None
+
+
+def test_predictive_plan_refuses_rows_that_are_not_a_multiple_of_32():
+    from georefine_amd import bitexact_predictive_codec as ppcx
+    from georefine_amd.bitexact_predictive_gpu import _read_frame
+    rng = np.random.default_rng(10)
+    target = weight_like(rng, 96, 176)
+    ref = target ^ np.uint16(1)
+    ix = _read_frame(ppcx.encode(target, ref), ref, 64, fused=True)
+    assert ix["mode"] in (0, 1) and "fused_plan" not in ix and "multiple of 32" in ix["fused_reason"]
