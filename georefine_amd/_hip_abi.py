@@ -47,7 +47,8 @@ class GrfPpcxFused(ctypes.Structure):
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
                   "grf_bctx_fused_decode", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
-                  "grf_ppcx_bins", "grf_ppcx_fused_decode", "grf_last_error", "grf_abi_version")
+                  "grf_ppcx_bins", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_last_error",
+                  "grf_abi_version")
 
 
 def declare(L):
@@ -73,5 +74,9 @@ def declare(L):
     L.grf_ppcx_bins.restype = i
     L.grf_ppcx_fused_decode.argtypes = [ctypes.POINTER(GrfPpcxFused), tiling, vp, vp, vp, vp]
     L.grf_ppcx_fused_decode.restype = i
+    L.grf_ppcx_gemv.argtypes = [ctypes.POINTER(GrfPpcxFused), tiling, vp, vp, u32, u32, vp, u32, vp, vp, vp]
+    L.grf_ppcx_gemv.restype = i
+    L.grf_ppcx_gemm.argtypes = L.grf_ppcx_gemv.argtypes
+    L.grf_ppcx_gemm.restype = i
     L.grf_last_error.restype = ctypes.c_char_p
     L.grf_abi_version.restype = i

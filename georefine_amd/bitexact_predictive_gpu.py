@@ -149,7 +149,7 @@ class HipPredictiveTensor:
                 self.buffers[name + "_cum"] = torch.from_numpy(cum).to(self.device)
                 self.buffers[name + "_bucket"] = torch.from_numpy(_tables.coarse_buckets(cum)).to(self.device)
         self.error = torch.zeros((), device=self.device, dtype=torch.int32)
-        self.resident_bytes = int(sum(t.numel() * t.element_size() for t in self.buffers.values()) + 4)
+        self._tilings = {}
         self._frame = None
         if self.mode != 2:
             b = self.buffers
@@ -176,17 +176,20 @@ class HipPredictiveTensor:
                 self._prepare_fused()
             except _fused.FusedUnsupported as exc:
                 self.fused, self.fused_reason = None, str(exc)
-        self.resident_bytes = int(sum(t.numel() * t.element_size() for t in self.buffers.values()) + 4)
+
+    @property
+    def resident_bytes(self):
+        """Every device allocation this tensor holds: buffers, tilings made so far, the error word."""
+        total = sum(t.numel() * t.element_size() for t in self.buffers.values()) + 4
+        total += sum(rows.numel() * 4 + classes.numel() for _, rows, classes, _ in self._tilings.values())
+        return int(total)
 
     def _prepare_fused(self):
         """Upload the walker's derived arrays: segment index, per-label tables, store tiling."""
         import torch
         plan, b = self._plan, self.buffers
-        host = plan.tiling(0)
         for name, array in (("fused_seg_state", plan.seg_state), ("fused_seg_offset", plan.seg_offset),
-                            ("fused_lut", plan.lut), ("fused_tab", plan.tab.view(np.int64)),
-                            ("fused_tile_rows", host["tile_rows"].view(np.int32)),
-                            ("fused_tile_class", host["tile_class"])):
+                            ("fused_lut", plan.lut), ("fused_tab", plan.tab.view(np.int64))):
             b[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
         f = _hip_abi.GrfPpcxFused()
         f.main_bytes, f.raw5 = b["main_stream"].data_ptr(), b["raw5"].data_ptr()
@@ -198,12 +201,76 @@ class HipPredictiveTensor:
         sc = plan.scalars()
         f.seg_len, f.segs_per_row, f.shift, f.lognb, f.tabn = (sc["seg_len"], sc["segs_per_row"], sc["shift"],
                                                                 sc["lognb"], sc["tabn"])
-        g = _hip_abi.GrfFusedTiling()
-        g.tile_rows, g.tile_class = b["fused_tile_rows"].data_ptr(), b["fused_tile_class"].data_ptr()
-        for key, value in host["scalars"].items():
-            setattr(g, key, value)
-        self.fused, self._tiling = f, g
-        self.fused_plan = dict(sc, **host["scalars"], lds=host["lds"])
+        self.fused = f
+        store = self._tiling_for(0)
+        self.fused_plan = dict(sc, **store[3])
+
+    def _tiling_for(self, key):
+        """Device copy of a tiling: key 0 = store sink, 1/2/4/8 = GEMV row buckets, "gemm"."""
+        import torch
+        if key not in self._tilings:
+            host = self._plan.gemm_tiling() if key == "gemm" else self._plan.tiling(key)
+            rows = torch.from_numpy(host["tile_rows"].view(np.int32)).to(self.device)
+            classes = torch.from_numpy(host["tile_class"]).to(self.device)
+            g = _hip_abi.GrfFusedTiling()
+            g.tile_rows, g.tile_class = rows.data_ptr(), classes.data_ptr()
+            for name, value in host["scalars"].items():
+                setattr(g, name, value)
+            self._tilings[key] = (g, rows, classes, dict(host["scalars"], lds=host["lds"]))
+        return self._tilings[key]
+
+    def _bins(self, ref):
+        """Transient plane of 4-bit bins of the reference words (one launch)."""
+        import torch
+        bins = torch.empty(self.n // 8, device=self.device, dtype=torch.int32)
+        b = self.buffers
+        status = self._lib.grf_ppcx_bins(ref.data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr(),
+                                         self.shape[0], self.shape[1], bins.data_ptr(),
+                                         torch.cuda.current_stream(self.device).cuda_stream)
+        return bins, status
+
+    def _reference(self, reference_bf16_device):
+        import torch
+        ref = reference_bf16_device.to(device=self.device).contiguous()
+        if tuple(ref.shape) != tuple(self.shape) or ref.dtype != torch.bfloat16:
+            raise ValueError("reference device tensor shape/dtype mismatch")
+        return ref
+
+    def linear(self, reference_bf16_device, x, bias=None, *, check=False, batch_invariant=False):
+        """y = x W^T + bias with W decoded on the fly against the reference: the fused GEMV for
+        up to 8 activation rows, the batch-invariant fused GEMM above (or always, on request).
+        Frames the tile walker cannot take are decoded and multiplied densely."""
+        import torch
+        if self.fused is None or x.dtype != torch.bfloat16:
+            return torch.nn.functional.linear(x, self.decode(reference_bf16_device, check=check), bias)
+        ref = self._reference(reference_bf16_device)
+        x2 = x.reshape(-1, x.shape[-1]).to(self.device)
+        if x2.shape[-1] != self.shape[1]:
+            raise ValueError("activation width does not match the weight")
+        m = x2.shape[0]
+        use_gemm = batch_invariant or m > 8
+        align = 4 if use_gemm else 2  # elements: the GEMM reads 8 bytes at a time, the GEMV 4
+        if x2.stride(-1) != 1 or x2.stride(0) % align or x2.data_ptr() % (2 * align):
+            x2 = x2.contiguous()
+        if bias is not None:
+            bias = bias.to(device=self.device, dtype=torch.bfloat16).contiguous()
+        y = torch.empty((m, self.shape[0]), device=self.device, dtype=torch.bfloat16)
+        if m:
+            self.error.zero_()
+            with torch.cuda.device(self.device):
+                bins, status = self._bins(ref)
+                if not status:
+                    if use_gemm:
+                        fn, tiling = self._lib.grf_ppcx_gemm, self._tiling_for("gemm")[0]
+                    else:
+                        fn = self._lib.grf_ppcx_gemv
+                        tiling = self._tiling_for(next(v for v in (1, 2, 4, 8) if v >= m))[0]
+                    status = fn(ctypes.byref(self.fused), ctypes.byref(tiling), bins.data_ptr(), x2.data_ptr(),
+                                x2.stride(0), m, y.data_ptr(), y.stride(0),
+                                bias.data_ptr() if bias is not None else None, self.error.data_ptr(),
+                                torch.cuda.current_stream(self.device).cuda_stream)
+            self._status(status, check)
+        return y.reshape(*x.shape[:-1], self.shape[0])
 
     def _status(self, status, check):
         if status:
@@ -218,22 +285,17 @@ class HipPredictiveTensor:
         import torch
         if self.mode == 2:
             return self.buffers["raw"].view(torch.bfloat16).reshape(self.shape)
-        ref = reference_bf16_device.to(device=self.device).contiguous()
-        if tuple(ref.shape) != tuple(self.shape) or ref.dtype != torch.bfloat16:
-            raise ValueError("reference device tensor shape/dtype mismatch")
+        ref = self._reference(reference_bf16_device)
         if self.fused is not None and not general:
-            bins = torch.empty(self.n // 8, device=self.device, dtype=torch.int32)
             out = torch.empty(self.shape, device=self.device, dtype=torch.uint16)
             self.error.zero_()
-            b = self.buffers
             with torch.cuda.device(self.device):
-                stream = torch.cuda.current_stream(self.device).cuda_stream
-                status = self._lib.grf_ppcx_bins(ref.data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr(),
-                                                 self.shape[0], self.shape[1], bins.data_ptr(), stream)
+                bins, status = self._bins(ref)
                 if not status:
-                    status = self._lib.grf_ppcx_fused_decode(ctypes.byref(self.fused), ctypes.byref(self._tiling),
-                                                             bins.data_ptr(), out.data_ptr(), self.error.data_ptr(),
-                                                             stream)
+                    status = self._lib.grf_ppcx_fused_decode(ctypes.byref(self.fused),
+                                                             ctypes.byref(self._tiling_for(0)[0]), bins.data_ptr(),
+                                                             out.data_ptr(), self.error.data_ptr(),
+                                                             torch.cuda.current_stream(self.device).cuda_stream)
             self._status(status, check)
             return out.view(torch.bfloat16)
         count = (self.n + self.stride - 1) // self.stride

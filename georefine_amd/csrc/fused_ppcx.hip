@@ -13,20 +13,11 @@
 //
 // Residuals are the packed 5-bit fields of the frame (GCR/bitexact_predictive_codec.py:145-166,
 // MSB first): 10 bytes per 16 symbols, so every second group starts half a dword in.
-#include <hip/hip_runtime.h>
-
-#include <string>
-
-#include "fused_device.h"
-
-namespace grf {
-int set_error(int code, const std::string &what);                                                  // decode_general.hip
-int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who);  // fused_gemv.hip
-}
+//
+// The walker plugs into the generic sinks of fused_kernels.h: store (decode), GEMV, GEMM.
+#include "fused_kernels.h"
 
 namespace {
-
-using grf::FusedLdsLayout;
 
 // ---- bins plane ----
 
@@ -108,7 +99,7 @@ struct PpcxWalk {
     return reinterpret_cast<const uint32_t *>(rawp + ((10 * g) & ~3u));
   }
   // global reads of the segment, issued before the wait for the slab's stream bytes
-  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0) {
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t) {
     seg = seg_;
     gofs = f.seg_offset[seg];
     c.state = f.seg_state[seg];
@@ -157,50 +148,33 @@ struct PpcxWalk {
   }
 };
 
-// `f` carries the PPCX frame in the walker's frame structure: raw6 = packed 5-bit
-// residuals, col_class = the bins plane, nr = labels, nc = 16 bins.
-__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_ppcx_kernel(grf_bctx_fused f, grf_fused_tiling g,
-                                                                            uint16_t *out, int32_t *error) {
-  extern __shared__ __align__(16) uint8_t lds[];
-  const FusedLdsLayout L(f, g, 0);
-  const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
-  const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
-  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, g.tile_class[tile], tid, nthreads);
-  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
-  const uint32_t r = tid / P, p = tid % P;
-  const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
-  uint32_t bad = 0;
-  grf::PieceSpan span{0, 0};
-  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
-  for (uint32_t b = 0; b < g.n_slabs; ++b) {
-    if (b) __syncthreads();  // everyone is done with the previous slab's stream bytes
-    const uint32_t first_seg = b * P;
-    const uint32_t nseg = min(P, f.segs_per_row - first_seg);
-    const uint32_t piece_off = L.stream + r * g.piece_cap;
-    const bool walks = row != grf::kNoRow && p < nseg;
-    const uint32_t seg_base = row != grf::kNoRow ? row * f.segs_per_row + first_seg : 0;
-    const uint64_t elem0 = (uint64_t)row * K + (uint64_t)(first_seg + p) * S;
-    PpcxWalk w;
-    uint32_t a0 = 0;
-    if (walks) w.prefetch(f, seg_base + p, elem0);
-    if (row != grf::kNoRow) {
-      a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
-      if (b + 1 < g.n_slabs) span.fetch(f, seg_base + P, min(P, f.segs_per_row - first_seg - P));
-    }
-    __syncthreads();
-    if (walks) {
-      w.start(piece_off, a0);
-      for (uint32_t t = 0; t < S; t += 16) {
-        uint32_t pair[8];
-        w.decode16(t, S, q, pair);
-        uint4 *dst = reinterpret_cast<uint4 *>(out + elem0 + t);
-        dst[0] = make_uint4(pair[0], pair[1], pair[2], pair[3]);
-        dst[1] = make_uint4(pair[4], pair[5], pair[6], pair[7]);
-      }
-      if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
-    }
-  }
-  if (bad) atomicOr(error, (int)bad);
+// The PPCX frame in the walker's frame structure: raw6 = packed 5-bit residuals,
+// col_class = the bins plane, nr = labels, nc = 16 bins.
+int walker_frame(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const char *who,
+                 grf_bctx_fused &f) {
+  if (!frame || !tiling || !bins) return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": null argument");
+  f = grf_bctx_fused{};
+  f.main_bytes = frame->main_bytes;
+  f.raw6 = frame->raw5;
+  f.seg_state = frame->seg_state;
+  f.seg_offset = frame->seg_offset;
+  f.lut = frame->lut;
+  f.tab = frame->tab;
+  f.col_class = reinterpret_cast<const uint8_t *>(bins);
+  f.main_n_bytes = frame->main_n_bytes;
+  f.rows = frame->rows;
+  f.cols = frame->cols;
+  f.nr = frame->n_labels;
+  f.nc = 16;
+  f.seg_len = frame->seg_len;
+  f.segs_per_row = frame->segs_per_row;
+  f.shift = frame->shift;
+  f.lognb = frame->lognb;
+  f.tabn = frame->tabn;
+  if (int rc = grf::check_fused_frame(f, *tiling, who)) return rc;
+  if (f.seg_len % 32)  // a segment's residual bytes must start on a dword
+    return grf::set_error(GRF_UNSUPPORTED, std::string(who) + ": segment length must be a multiple of 32");
+  return GRF_OK;
 }
 
 }  // namespace
@@ -227,41 +201,31 @@ int grf_ppcx_bins(const uint16_t *reference, const uint8_t *flips, const uint16_
 
 int grf_ppcx_fused_decode(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins,
                           uint16_t *out, int32_t *error, void *hip_stream) {
-  if (!frame || !tiling || !bins || !out || !error)
-    return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_fused_decode: null argument");
-  grf_bctx_fused f{};
-  f.main_bytes = frame->main_bytes;
-  f.raw6 = frame->raw5;
-  f.seg_state = frame->seg_state;
-  f.seg_offset = frame->seg_offset;
-  f.lut = frame->lut;
-  f.tab = frame->tab;
-  f.col_class = reinterpret_cast<const uint8_t *>(bins);
-  f.main_n_bytes = frame->main_n_bytes;
-  f.rows = frame->rows;
-  f.cols = frame->cols;
-  f.nr = frame->n_labels;
-  f.nc = 16;
-  f.seg_len = frame->seg_len;
-  f.segs_per_row = frame->segs_per_row;
-  f.shift = frame->shift;
-  f.lognb = frame->lognb;
-  f.tabn = frame->tabn;
-  if (int rc = grf::check_fused_frame(f, *tiling, "grf_ppcx_fused_decode")) return rc;
-  if (f.seg_len % 32)  // a segment's residual bytes must start on a dword
-    return grf::set_error(GRF_UNSUPPORTED, "grf_ppcx_fused_decode: segment length must be a multiple of 32");
-  const FusedLdsLayout L(f, *tiling, 0);
-  if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
-  if (L.total > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(fused_ppcx_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
-    if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("LDS attribute: ") + hipGetErrorString(e));
-  }
-  hipLaunchKernelGGL(fused_ppcx_kernel, dim3(tiling->n_tiles), dim3(tiling->threads), L.total,
-                     (hipStream_t)hip_stream, f, *tiling, out, error);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
-  return GRF_OK;
+  if (!out || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_fused_decode: null argument");
+  grf_bctx_fused f;
+  if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_fused_decode", f)) return rc;
+  return grf::launch_walk<PpcxWalk, 1, true>(f, *tiling, nullptr, 0, nullptr, 0, nullptr, out, error,
+                                             (hipStream_t)hip_stream);
+}
+
+int grf_ppcx_gemv(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const uint16_t *x,
+                  uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
+                  void *hip_stream) {
+  if (!x || !y || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemv: null argument");
+  grf_bctx_fused f;
+  if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_gemv", f)) return rc;
+  return grf::launch_gemv<PpcxWalk>("grf_ppcx_gemv", f, *tiling, x, ldx, m_rows, y, ldy, bias, error,
+                                    (hipStream_t)hip_stream);
+}
+
+int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const uint16_t *x,
+                  uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
+                  void *hip_stream) {
+  if (!x || !y || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemm: null argument");
+  grf_bctx_fused f;
+  if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_gemm", f)) return rc;
+  return grf::launch_gemm<PpcxWalk>("grf_ppcx_gemm", f, *tiling, x, ldx, m_rows, y, ldy, bias, error,
+                                    (hipStream_t)hip_stream);
 }
 
 }  // extern "C"

@@ -113,15 +113,7 @@ class PredictiveContextTensor:
 
     def decode(self, *, check=True):
         with self._decode_lock:
-            refs = [ctx.decode(check=check) for ctx in self.references]
-            if len(refs) == 1:
-                reference = refs[0]
-            else:
-                if self.predictor is None:
-                    from .bitexact_predictive_mix import predict as default_predictor
-                    self.predictor = default_predictor
-                reference = self.predictor(refs[0], refs[1], self.coefficients)
-            value = self.native.decode(reference, check=check)
+            value = self.native.decode(self._reference(check), check=check)
             if self.transform == "target transpose":
                 value = value.transpose(-2, -1).contiguous()
             return value
@@ -129,9 +121,24 @@ class PredictiveContextTensor:
     def gather_rows(self, ids, *, check=True):
         return self.decode(check=check)[ids]
 
+    def _reference(self, check):
+        refs = [ctx.decode(check=check) for ctx in self.references]
+        if len(refs) == 1:
+            return refs[0]
+        if self.predictor is None:
+            from .bitexact_predictive_mix import predict as default_predictor
+            self.predictor = default_predictor
+        return self.predictor(refs[0], refs[1], self.coefficients)
+
     def linear(self, x, bias=None, *, check=False, batch_invariant=False):
-        """Decode against the references, then the dense matmul (no fused PPCX kernel yet)."""
-        return torch.nn.functional.linear(x, self.decode(check=check), bias)
+        """x W^T + bias.  A frame stored untransposed goes through the native tensor's fused
+        product (reference decoded, then decode and dot in one kernel); a transposed frame holds
+        W^T row by row, so it is decoded and multiplied densely."""
+        fused = getattr(self.native, "linear", None)
+        if fused is None or self.transform == "target transpose":
+            return torch.nn.functional.linear(x, self.decode(check=check), bias)
+        with self._decode_lock:
+            return fused(self._reference(check), x, bias, check=check, batch_invariant=batch_invariant)
 
 
 # ----------------------------------------------------------------------------- loader

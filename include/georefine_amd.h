@@ -261,6 +261,18 @@ int grf_ppcx_bins(const uint16_t *reference, const uint8_t *flips, const uint16_
 int grf_ppcx_fused_decode(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins,
                           uint16_t *out, int32_t *error, void *hip_stream);
 
+/* Fused products on a prepared PPCX frame given the bins of its reference: the sinks and the
+ * reduction orders of grf_bctx_gemv (1 <= m_rows <= 8, tilings as for that function) and
+ * grf_bctx_gemm (any m_rows, one tiling for every row count).  They replace decode() +
+ * F.linear of PredictiveContextTensor weights (GCR/bitexact_predictive_serving.py:490-523)
+ * for frames stored untransposed. */
+int grf_ppcx_gemv(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const uint16_t *x,
+                  uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
+                  void *hip_stream);
+int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const uint16_t *x,
+                  uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
+                  void *hip_stream);
+
 const char *grf_last_error(void);
 int grf_abi_version(void);
 

@@ -152,3 +152,41 @@ def test_serving_modules_with_fused_and_predictive_weights(oracle):
     assert np.array_equal(wrapped.decode().view(torch.uint16).cpu().numpy(), target.T)
     out = serving.BctxLinear(wrapped)(torch.ones(2, 128, dtype=torch.bfloat16, device="cuda"))
     assert out.shape == (2, 256)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle, mode):
+    """The predictive walker behind the GEMV and GEMM sinks: within 1e-2 of the dense product
+    of the decoded target (the tolerance of the fused products), GEMV rows bit-equal for
+    M = 1..8, GEMM rows bit-equal for every batch."""
+    import torch
+    from georefine_amd import bitexact_predictive_codec as codec
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
+    rng = np.random.default_rng(40 + mode)
+    target = weight_like(rng, 200, 1280)
+    tf = (target.astype(np.uint32) << 16).view(np.float32)
+    ref = bf16_words(tf + rng.normal(0, 0.003, target.shape).astype(np.float32))
+    t = HipPredictiveTensor(_frame_for_mode(codec, target, ref, mode), ref, stride=1024, device="cuda:0")
+    assert t.fused is not None, t.fused_reason
+    ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
+    dense_w = torch.from_numpy(target).view(torch.bfloat16).cuda().float()
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(40, 1280)))).view(torch.bfloat16).cuda()
+    bias = torch.from_numpy(bf16_words(rng.normal(0, 1, size=200))).view(torch.bfloat16).cuda()
+    want = torch.nn.functional.linear(x.float(), dense_w, bias.float())
+    scale = torch.nn.functional.linear(x.float().abs(), dense_w.abs(), bias.float().abs())
+
+    def close(y, rows):
+        return bool((y.float() - want[:rows]).abs().le(1e-2 * want[:rows].abs().clamp_min(1e-3 * scale[:rows])).all())
+
+    y8 = t.linear(ref_dev, x[:8], bias, check=True)
+    assert y8.shape == (8, 200) and close(y8, 8)
+    for m in (1, 2, 3, 5):
+        assert torch.equal(t.linear(ref_dev, x[:m], bias).view(torch.uint16), y8[:m].view(torch.uint16))
+    y40 = t.linear(ref_dev, x, bias, check=True)            # more than 8 rows: the matrix-core kernel
+    assert close(y40, 40)
+    for m in (1, 8, 17, 32):
+        ym = t.linear(ref_dev, x[:m], bias, batch_invariant=True)
+        assert torch.equal(ym.view(torch.uint16), y40[:m].view(torch.uint16)), m
+    wrong = torch.from_numpy(np.roll(ref, 5, axis=1).copy()).view(torch.bfloat16).cuda()
+    with pytest.raises(codec.CodecError):
+        t.linear(wrong, x[:2], check=True)
