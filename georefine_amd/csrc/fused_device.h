@@ -1,8 +1,8 @@
 // The fused decoder: one walker over a checkpointed segment whose decoded BF16
 // words go to a sink (dot-product chain for the GEMV, LDS tile for the GEMM,
-// global store for decode()).  Because every sink is fed by the same walker,
-// words proven bit-exact through the store sink are the words the fused sinks
-// consume.
+// global store for decode(); fused_kernels.h).  Because every sink is fed by the
+// same walker, words proven bit-exact through the store sink are the words the
+// fused sinks consume.
 //
 // Work decomposition (packed-residual frames, segment length S divides the row
 // length K):
@@ -21,10 +21,10 @@
 //
 // Symbol lookup: slot>>shift indexes a u8 table giving the sparse index of the
 // symbol that owns most of the bucket's slots; that symbol's 8-byte entry is read and
-// assumed to own the slot.  Entry: low32 = start | (freq & 0xFFFF)<<16 (0 stands for 65536), high32 = symbol<<5
-// (the symbol's bits in the BF16 word).  When a symbol boundary inside the bucket
-// separates the slot from that symbol, a scan over the neighbouring entries finishes
-// the search.
+// assumed to own the slot.  Entry: low32 = start | (freq & 0xFFFF)<<16 (0 stands for
+// 65536), high32 = the symbol's bits in the BF16 word (symbol<<5 for this codec).  When a
+// symbol boundary inside the bucket separates the slot from that symbol, a scan over the
+// neighbouring entries finishes the search.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -67,7 +67,6 @@ struct FusedLdsLayout {
 };
 
 typedef __attribute__((address_space(3))) uint8_t lds_u8;
-typedef __attribute__((address_space(3))) uint32_t lds_u32;
 typedef uint32_t v2u32 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) v2u32 lds_v2u32;
 
@@ -126,10 +125,6 @@ struct StepFetch {
 // 2 - n and the byte reads carry 2k in their offset field.
 struct Cursor {
   uint32_t state, j;
-  __device__ __forceinline__ void open(uint32_t state_, uint32_t ip_) {
-    state = state_;
-    j = ip_;
-  }
   __device__ __forceinline__ void end_group() { j += 32; }  // after 16 steps: j is ip again
 };
 
