@@ -60,8 +60,6 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
-
-  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
 
   const uint32_t r = tid / P, p = tid % P;
@@ -73,8 +71,11 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   float *rowsum = reinterpret_cast<float *>(lds + L.rowsum);  // [R][M] running sums
   uint32_t bad = 0;
 
+  // the first slab's byte range is two dependent global reads away (row, then offsets):
+  // start them before the tables are copied so that the latencies overlap
   grf::PieceSpan span{0, 0};
   if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
+  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
     if (b) __syncthreads();  // everyone is done with the previous slab's LDS data
     const uint32_t col_base = b * width;
@@ -240,11 +241,13 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
-  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
 
   const uint32_t r = tid / P, p = tid % P;
   const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
+  grf::PieceSpan span{0, 0};  // started before the table copy so that the latencies overlap
+  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
+  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
 
   // contraction roles: wave -> one 16-column block of the tile (nt) and every MW-th row tile
   const uint32_t wave = tid / 64, lane = tid % 64, nwaves = nthreads / 64;
@@ -258,8 +261,6 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
   for (uint32_t j = 0; j < kMaxAcc; ++j) acc[j] = (float4v){0.f, 0.f, 0.f, 0.f};
   uint32_t bad = 0;
 
-  grf::PieceSpan span{0, 0};
-  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
     __syncthreads();  // previous slab's stream bytes and tiles are no longer read
     const uint32_t first_seg = b * P;
