@@ -20,10 +20,17 @@ class FusedUnsupported(ValueError):
     """The frame cannot use the fused kernels (the caller falls back to decode + dense)."""
 
 
-def choose_segment(cols, preferred=None):
-    """Largest supported segment length that divides the row length."""
+SMALL_MATRIX = 8 << 20  # elements below which the walk, not the machine, bounds a launch
+
+
+def choose_segment(cols, preferred=None, rows=None):
+    """Segment length that divides the row length: 64 by default (index 1 bit per weight).
+    A launch takes at least one segment's worth of dependent steps, so matrices too small to
+    fill the GPU several times over get 32 (2 bits per weight of index, three quarters of
+    the time)."""
     order = [preferred] if preferred else []
-    order += [64, 128, 32, 256, 16]
+    small = rows is not None and rows * cols < SMALL_MATRIX
+    order += [32, 64, 16, 128, 256] if small else [64, 128, 32, 256, 16]
     for s in order:
         if s and s % 16 == 0 and cols % s == 0:
             return s

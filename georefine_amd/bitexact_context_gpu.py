@@ -124,7 +124,8 @@ class HipContextTensor:
         segment = None
         if fused:
             try:
-                segment = _fused.choose_segment(base.HEADER.unpack_from(frame)[6], fused_segment)
+                header = base.HEADER.unpack_from(frame)
+                segment = _fused.choose_segment(header[6], fused_segment, rows=header[5])
             except _fused.FusedUnsupported:
                 segment = None
         indexed = index_frame(frame, stride, fused_segment=segment, raw6_residual=segment is not None)

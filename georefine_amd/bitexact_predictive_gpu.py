@@ -58,7 +58,8 @@ def _fused_plan(ix, stream, contexts, segment=None):
     r, c = ix["shape"]
     if c % 32:
         raise _fused.FusedUnsupported("row length is not a multiple of 32")
-    seg_len = next((s for s in ([segment] if segment else []) + [64, 128, 32, 256] if s and s % 32 == 0 and c % s == 0), None)
+    order = [32, 64, 128, 256] if r * c < _fused.SMALL_MATRIX else [64, 128, 32, 256]
+    seg_len = next((s for s in ([segment] if segment else []) + order if s and s % 32 == 0 and c % s == 0), None)
     if seg_len is None:
         raise _fused.FusedUnsupported("no segment length divides the row length")
     states, offsets, _ = _checkpoints(stream, contexts, ix["main_freq"], codec.MAIN_VOCAB, seg_len)

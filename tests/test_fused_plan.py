@@ -88,6 +88,7 @@ def test_unsupported_frames_are_reported():
         _fused.choose_segment(67)
     assert _fused.choose_segment(5120) == 64 and _fused.choose_segment(48) == 16
     assert _fused.choose_segment(5120, 128) == 128
+    assert _fused.choose_segment(5120, rows=1024) == 32 and _fused.choose_segment(5120, rows=17408) == 64
     words = np.arange(65536, dtype=np.uint16).reshape(256, 256)  # 1024 distinct symbols in one context
     frame = codec.encode(words, row_classes=1, col_classes=1)
     if frame[5] != 1:
