@@ -246,7 +246,7 @@ class FramePlan:
         which an output element accumulates follows the tiling, so it must not change with M."""
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
             self.spr, self.class_rows, self._cap,
-            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, 128, p_, r_, cap_), gemm=True)
+            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, 64, p_, r_, cap_), gemm=True)
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,

@@ -206,6 +206,7 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 constexpr uint32_t kGroup = 16;      // columns decoded between two contractions
 constexpr uint32_t kMaxAcc = 4;      // 16x16 output blocks a wave may own
 constexpr uint32_t kMaxRowsPerLaunch = 128;
+constexpr uint32_t kChunkTiles = 4;  // 16-row activation tiles staged in LDS at a time (64 rows)
 
 // LDS regions of the GEMM kernel.  Word and activation tiles hold, per (row, p), one
 // 32-byte run of 16 BF16 values; a row's runs are padded by 8 bytes so that the 16 rows
@@ -237,7 +238,8 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
                                                                             uint32_t ldy, const uint16_t *bias,
                                                                             int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  const GemmLdsLayout L(f, g, MT * 16);
+  constexpr uint32_t CT = MT < kChunkTiles ? MT : kChunkTiles;  // activation tiles per chunk
+  const GemmLdsLayout L(f, g, CT * 16);
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
@@ -289,31 +291,36 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
         dst[2] = make_uint2(pair[4], pair[5]);
         dst[3] = make_uint2(pair[6], pair[7]);
       }
-      // the same 16 columns of every lane-segment of the activations -> activation tile
-      for (uint32_t c = tid; c < MT * 16 * P * 4; c += nthreads) {
-        const uint32_t part = c % 4, pp = (c / 4) % P, m = c / (4 * P);
-        const uint32_t col = (first_seg + pp) * S + t + part * 4;
-        uint2 v = make_uint2(0u, 0u);
-        if (m < m_rows && pp < nseg) v = *reinterpret_cast<const uint2 *>(x + (size_t)m * ldx + col);
-        *reinterpret_cast<uint2 *>(lds + L.xt + m * L.xt_pitch + pp * 32 + part * 8) = v;
-      }
-      __syncthreads();
-      if (contracts) {
-        const uint8_t *brow = lds + L.wt + (nt * 16 + li) * L.wt_pitch + kq * 8;
+      // The same 16 columns of every lane-segment of the activations -> activation tile, 64
+      // rows at a time: the tile's size bounds the lanes per row a tiling can have, and an
+      // output element's sequence of operations does not depend on the chunking.
+      for (uint32_t mc = 0; mc < MT; mc += CT) {
+        if (mc) __syncthreads();  // the previous chunk has been consumed
+        for (uint32_t c = tid; c < CT * 16 * P * 4; c += nthreads) {
+          const uint32_t part = c % 4, pp = (c / 4) % P, ml = c / (4 * P), m = mc * 16 + ml;
+          const uint32_t col = (first_seg + pp) * S + t + part * 4;
+          uint2 v = make_uint2(0u, 0u);
+          if (m < m_rows && pp < nseg) v = *reinterpret_cast<const uint2 *>(x + (size_t)m * ldx + col);
+          *reinterpret_cast<uint2 *>(lds + L.xt + ml * L.xt_pitch + pp * 32 + part * 8) = v;
+        }
+        __syncthreads();
+        if (contracts) {
+          const uint8_t *brow = lds + L.wt + (nt * 16 + li) * L.wt_pitch + kq * 8;
 #pragma unroll
-        for (uint32_t j = 0; j < kMaxAcc; ++j) {
-          const uint32_t mt = mslot + j * MW;
-          if (mt < MT) {
-            const uint8_t *arow = lds + L.xt + (mt * 16 + li) * L.xt_pitch + kq * 8;
-            for (uint32_t pp = 0; pp < nseg; ++pp) {
-              const short4v a = *reinterpret_cast<const short4v *>(arow + pp * 32);
-              const short4v bb = *reinterpret_cast<const short4v *>(brow + pp * 32);
+          for (uint32_t j = 0; j < kMaxAcc; ++j) {
+            const uint32_t mt = mslot + j * MW;
+            if (mt >= mc && mt < mc + CT && mt < MT) {
+              const uint8_t *arow = lds + L.xt + ((mt - mc) * 16 + li) * L.xt_pitch + kq * 8;
+              for (uint32_t pp = 0; pp < nseg; ++pp) {
+                const short4v a = *reinterpret_cast<const short4v *>(arow + pp * 32);
+                const short4v bb = *reinterpret_cast<const short4v *>(brow + pp * 32);
 #if defined(__HIP_DEVICE_COMPILE__)
-              acc[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, bb, acc[j], 0, 0, 0);
+                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, bb, acc[j], 0, 0, 0);
 #else
-              (void)a;
-              (void)bb;
+                (void)a;
+                (void)bb;
 #endif
+              }
             }
           }
         }
@@ -347,7 +354,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
 template <class Walk, int MT>
 int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
            uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error, hipStream_t s) {
-  const GemmLdsLayout L(f, g, MT * 16);
+  const GemmLdsLayout L(f, g, (MT < kChunkTiles ? MT : kChunkTiles) * 16);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused GEMM: LDS demand exceeds 160 KiB");
   const uint32_t nwaves = g.threads / 64, NT = (g.rows_per_tile + 15) / 16;
   if (NT > nwaves) return grf::set_error(GRF_BAD_ARGUMENT, "fused GEMM: more column blocks than waves");
@@ -390,7 +397,7 @@ int launch_gemm(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
 
 inline uint32_t gemm_lds_bytes(const grf_bctx_fused &f, const grf_fused_tiling &g, uint32_t m_rows) {
   const uint32_t m = m_rows > kMaxRowsPerLaunch ? kMaxRowsPerLaunch : m_rows;
-  const uint32_t mt = m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8;
+  const uint32_t mt = m <= 16 ? 1 : m <= 32 ? 2 : 4;  // activations are staged 64 rows at a time
   return GemmLdsLayout(f, g, mt * 16).total;
 }
 
