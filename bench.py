@@ -240,7 +240,8 @@ def main():
                             "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in names},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "kernel": (f"fused_walk_kernel<{m},false>" if m <= 8 else "fused_gemm_kernel") + f" on {dom}"},
+                     "kernel": (f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, false>" if m <= 8
+                                else "grf::fused_gemm_kernel<grf::SegmentWalk, MT>") + f" on {dom}"},
     }
     if not args.no_cpu_baseline:
         log("timing the CPU oracle on whole frames ...")
