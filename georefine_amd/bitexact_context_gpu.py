@@ -116,6 +116,8 @@ def _device_stream(buffers, name, vocab, nctx):
 class HipContextTensor:
     """A BCTX-coded BF16 matrix resident on one MI355X."""
 
+    DENSE_ABOVE = 64  # activation rows above which linear() decodes to a dense transient
+
     def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None):
         import torch
         if not torch.cuda.is_available():
@@ -323,15 +325,16 @@ class HipContextTensor:
     def linear(self, x, bias=None, *, check=False, batch_invariant=False):
         """y = x @ W.T (+ bias) with W decoded inside the kernel; x is BF16 [..., K].
 
-        Up to 8 activation rows run the fused decode-GEMV, more run the fused decode-GEMM;
-        ``batch_invariant=True`` sends every row count through the GEMM so that a row's
-        output never depends on the batch it arrives in.  Frames the fused kernels cannot
-        take are decoded on the device and multiplied densely.  ``check=True`` reads the
-        error word back (a host sync)."""
+        Up to 8 activation rows run the fused decode-GEMV, up to 64 the fused decode-GEMM;
+        above that a fused decode to a dense transient followed by the library matmul is
+        faster (measured crossover between 64 and 96 rows).  ``batch_invariant=True`` sends
+        every row count through the GEMM so that a row's output never depends on the batch
+        it arrives in.  Frames the fused kernels cannot take are decoded on the device and
+        multiplied densely.  ``check=True`` reads the error word back (a host sync)."""
         import torch.nn.functional as F
-        if self.fused is None:
-            return F.linear(x.to(self.device), self.decode(check=check), bias)
         m = math.prod(x.shape[:-1])
+        if self.fused is None or (m > self.DENSE_ABOVE and not batch_invariant):
+            return F.linear(x.to(self.device), self.decode(check=check), bias)
         if batch_invariant or m > 8 or m == 0:
             return self.gemm(x, bias, check=check)
         return self.gemv(x, bias, check=check)

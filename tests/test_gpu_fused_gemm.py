@@ -58,6 +58,12 @@ def test_gemm_bias_strided_input_and_dense_agreement(oracle):
     dense = torch.nn.functional.linear(x.float(), t.decode().float(), bias.float())
     assert torch.allclose(y.float(), dense, rtol=1e-2, atol=2e-2)
     assert t.gemm(x[:0]).shape == (0, 192)
+    # above DENSE_ABOVE rows linear() decodes to a dense transient unless batch invariance is asked for
+    big = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(t.DENSE_ABOVE + 6, 768)))).view(torch.bfloat16).cuda()
+    assert torch.equal(t.linear(big, bias), torch.nn.functional.linear(big, t.decode(), bias))
+    invariant = t.linear(big, bias, batch_invariant=True)
+    assert torch.equal(invariant[:40].view(torch.uint16), t.gemm(big[:40], bias).view(torch.uint16))
+    assert torch.allclose(invariant.float(), t.linear(big, bias).float(), rtol=1e-2, atol=2e-2)
 
 
 def test_gemm_checkpoint_mismatch_sets_error(oracle):
