@@ -53,18 +53,16 @@ def _word_image(main):
     return ((main & 1024) << 5) | (((main >> 2) & 255) << 7) | ((main & 3) << 5)
 
 
-def _fused_plan(ix, stream, contexts, segment=None):
-    """Segment index, per-label tables and tilings for the tile walker, or FusedUnsupported."""
-    r, c = ix["shape"]
+def _fused_segment(shape, segment=None):
+    """Segment length for the tile walker (a multiple of 32 that divides the row length)."""
+    r, c = shape
     if c % 32:
         raise _fused.FusedUnsupported("row length is not a multiple of 32")
     order = [32, 64, 128, 256] if r * c < _fused.SMALL_MATRIX else [64, 128, 32, 256]
     seg_len = next((s for s in ([segment] if segment else []) + order if s and s % 32 == 0 and c % s == 0), None)
     if seg_len is None:
         raise _fused.FusedUnsupported("no segment length divides the row length")
-    states, offsets, _ = _checkpoints(stream, contexts, ix["main_freq"], codec.MAIN_VOCAB, seg_len)
-    return _fused.FramePlan((r, c), 16, 16, ix["labels"], ix["main_freq"], states, offsets, len(stream), seg_len,
-                            image=_word_image)
+    return seg_len
 
 
 def _read_frame(frame, reference, stride, *, fused=False, fused_segment=None):
@@ -88,14 +86,28 @@ def _read_frame(frame, reference, stride, *, fused=False, fused_segment=None):
         return result
     freq = info["main_freq"].reshape(codec.MAIN_CONTEXTS, codec.MAIN_VOCAB)
     ctx = codec.contexts(info["reference"], info["labels"], info["flips"], info["thresholds"])
-    states, offsets, main = _checkpoints(info["stream"], ctx, freq, codec.MAIN_VOCAB, stride)
+    seg_len = None
+    if fused:
+        try:
+            seg_len = _fused_segment((r, c), fused_segment)
+        except _fused.FusedUnsupported as exc:
+            result["fused_reason"] = str(exc)
+    # one validated walk serves both indexes when the stride is a multiple of the segment length
+    if seg_len and stride % seg_len == 0:
+        fs, fo, main = _checkpoints(info["stream"], ctx, freq, codec.MAIN_VOCAB, seg_len)
+        states, offsets = fs[::stride // seg_len].copy(), fo[::stride // seg_len].copy()
+    else:
+        states, offsets, main = _checkpoints(info["stream"], ctx, freq, codec.MAIN_VOCAB, stride)
+        if seg_len:
+            fs, fo, _ = _checkpoints(info["stream"], ctx, freq, codec.MAIN_VOCAB, seg_len)
     result.update(labels=info["labels"], flips=info["flips"], thresholds=info["thresholds"], main_freq=freq,
                   main_stream=np.frombuffer(info["stream"], dtype=np.uint8).copy(), main_states=states,
                   main_offsets=offsets)
     result["resident_mode"] = info["mode"]
-    if fused:
+    if seg_len:
         try:
-            result["fused_plan"] = _fused_plan(result, info["stream"], ctx, fused_segment)
+            result["fused_plan"] = _fused.FramePlan((r, c), 16, 16, info["labels"], freq, fs, fo, len(info["stream"]),
+                                                    seg_len, image=_word_image)
             result["resident_mode"] = 0
         except _fused.FusedUnsupported as exc:
             result["fused_reason"] = str(exc)
