@@ -132,6 +132,8 @@ def _read_frame(frame, reference, stride, *, fused=False, fused_segment=None):
 class HipPredictiveTensor:
     """A PPCX-coded BF16 matrix resident on one MI355X; decoding needs the reference matrix."""
 
+    DENSE_ABOVE = 8  # activation rows above which linear() decodes to a dense transient
+
     def __init__(self, frame, reference_uint16_numpy, stride=1024, device="cuda:0", *, fused=True,
                  fused_segment=None):
         if not isinstance(stride, int) or not 1 <= stride <= 65536:
@@ -251,16 +253,18 @@ class HipPredictiveTensor:
 
     def linear(self, reference_bf16_device, x, bias=None, *, check=False, batch_invariant=False):
         """y = x W^T + bias with W decoded on the fly against the reference: the fused GEMV for
-        up to 8 activation rows, the batch-invariant fused GEMM above (or always, on request).
+        up to 8 activation rows; above that the fused decode to a dense transient plus the
+        library matmul is faster (the 16 bin contexts leave the GEMM little LDS), unless
+        ``batch_invariant`` asks for the fused GEMM, whose rows do not depend on the batch.
         Frames the tile walker cannot take are decoded and multiplied densely."""
         import torch
-        if self.fused is None or x.dtype != torch.bfloat16:
+        m = math.prod(x.shape[:-1])
+        if self.fused is None or x.dtype != torch.bfloat16 or (m > self.DENSE_ABOVE and not batch_invariant):
             return torch.nn.functional.linear(x, self.decode(reference_bf16_device, check=check), bias)
         ref = self._reference(reference_bf16_device)
         x2 = x.reshape(-1, x.shape[-1]).to(self.device)
         if x2.shape[-1] != self.shape[1]:
             raise ValueError("activation width does not match the weight")
-        m = x2.shape[0]
         use_gemm = batch_invariant or m > 8
         align = 4 if use_gemm else 2  # elements: the GEMM reads 8 bytes at a time, the GEMV 4
         if x2.stride(-1) != 1 or x2.stride(0) % align or x2.data_ptr() % (2 * align):

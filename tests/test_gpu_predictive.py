@@ -182,7 +182,8 @@ def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle,
     assert y8.shape == (8, 200) and close(y8, 8)
     for m in (1, 2, 3, 5):
         assert torch.equal(t.linear(ref_dev, x[:m], bias).view(torch.uint16), y8[:m].view(torch.uint16))
-    y40 = t.linear(ref_dev, x, bias, check=True)            # more than 8 rows: the matrix-core kernel
+    y40 = t.linear(ref_dev, x, bias, check=True, batch_invariant=True)  # the matrix-core kernel
+    assert close(t.linear(ref_dev, x, bias, check=True), 40)             # default above 8 rows: decode + dense
     assert close(y40, 40)
     for m in (1, 8, 17, 32):
         ym = t.linear(ref_dev, x[:m], bias, batch_invariant=True)
