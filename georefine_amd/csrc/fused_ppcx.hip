@@ -42,20 +42,33 @@ __global__ __launch_bounds__(kBinsThreads) void ppcx_bins_kernel(const uint16_t 
     *reinterpret_cast<uint32_t *>(table + a) = four;
   }
   __syncthreads();
+  // two chunks of 16 elements per thread and pass, their loads issued together
   const uint64_t stride = (uint64_t)gridDim.x * kBinsThreads * 16;
-  for (uint64_t first = ((uint64_t)blockIdx.x * kBinsThreads + threadIdx.x) * 16; first < n; first += stride) {
-    const uint4 *src = reinterpret_cast<const uint4 *>(reference + first);  // cols % 16 == 0: one row
-    const uint4 ra = src[0], rb = src[1];
-    const uint32_t flip = flips[first / cols] ? 0x80008000u : 0u;
-    const uint32_t w[8] = {ra.x ^ flip, ra.y ^ flip, ra.z ^ flip, ra.w ^ flip,
-                           rb.x ^ flip, rb.y ^ flip, rb.z ^ flip, rb.w ^ flip};
-    uint32_t packed[2] = {0, 0};
+  for (uint64_t first = ((uint64_t)blockIdx.x * kBinsThreads + threadIdx.x) * 16; first < n; first += 2 * stride) {
+    const uint64_t at[2] = {first, first + stride};
+    uint4 raw[2][2];
+    uint32_t flip[2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const uint32_t a = (i % 2) ? (w[i / 2] >> 16) : (w[i / 2] & 0xFFFFu);
-      packed[i / 8] |= (uint32_t)table[a] << (4 * (i % 8));
+    for (int c = 0; c < 2; ++c) {
+      if (at[c] >= n) continue;
+      const uint4 *src = reinterpret_cast<const uint4 *>(reference + at[c]);  // cols % 16 == 0: one row
+      raw[c][0] = src[0];
+      raw[c][1] = src[1];
+      flip[c] = flips[at[c] / cols] ? 0x80008000u : 0u;
     }
-    *reinterpret_cast<uint2 *>(bins + first / 8) = make_uint2(packed[0], packed[1]);
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      if (at[c] >= n) continue;
+      const uint32_t w[8] = {raw[c][0].x ^ flip[c], raw[c][0].y ^ flip[c], raw[c][0].z ^ flip[c], raw[c][0].w ^ flip[c],
+                             raw[c][1].x ^ flip[c], raw[c][1].y ^ flip[c], raw[c][1].z ^ flip[c], raw[c][1].w ^ flip[c]};
+      uint32_t packed[2] = {0, 0};
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const uint32_t a = (i % 2) ? (w[i / 2] >> 16) : (w[i / 2] & 0xFFFFu);
+        packed[i / 8] |= (uint32_t)table[a] << (4 * (i % 8));
+      }
+      *reinterpret_cast<uint2 *>(bins + at[c] / 8) = make_uint2(packed[0], packed[1]);
+    }
   }
 }
 
