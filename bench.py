@@ -29,6 +29,9 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBPS = 8000.0
 MODEL_BF16_BYTES = 55_586_113_293  # dense BF16 bytes of the 27B model one token has to read at batch 1
 SHAPES = {"gate": (17408, 5120), "up": (17408, 5120), "down": (5120, 17408)}
+# one layer of the whole-stack workload: attention projections, then the MLP
+LAYER = {"q": (6144, 5120), "k": (1024, 5120), "v": (1024, 5120), "o": (5120, 6144),
+         "gate": (17408, 5120), "up": (17408, 5120), "down": (5120, 17408)}
 
 
 def log(*a):
@@ -110,6 +113,117 @@ def cpu_baseline(frames, words_of, x_words, min_seconds=10.0, max_frames=12):
     return result
 
 
+def run_stack(args):
+    """Every coded linear of a 64-layer stack resident at once, one pass at batch 64.
+
+    Each layer holds q, k, v, o, gate, up and down as BCTX frames.  `--distinct-layers`
+    layers are generated and encoded from their own seeds; the others are device copies of
+    those in rotation (their own buffers, so a pass streams every layer's bytes from HBM,
+    but no further host encoding)."""
+    import torch
+    from concurrent.futures import ThreadPoolExecutor
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd.bitexact_context_gpu import HipContextTensor
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs a ROCm GPU")
+    m = args.batch if args.batch != 1 else 64
+    t0 = time.perf_counter()
+
+    def coded(job):
+        layer, j, name = job
+        rows, cols = LAYER[name]
+        return job, codec.encode(synth_weights(100 * layer + j, rows, cols))
+
+    jobs = [(d, j, name) for d in range(args.distinct_layers) for j, name in enumerate(LAYER)]
+    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
+        frames = dict(pool.map(coded, jobs))
+    log(f"encoded {len(jobs)} matrices in {time.perf_counter() - t0:.1f}s")
+    t0 = time.perf_counter()
+    base = {}
+    for job in jobs:
+        t = HipContextTensor(frames[job], stride=1024, device="cuda:0")
+        if t.fused is None:
+            sys.exit(f"bench.py: {job} is not eligible for the fused kernels: {t.fused_reason}")
+        t._gemm_tiling()
+        base[job] = t
+    log(f"indexed and uploaded in {time.perf_counter() - t0:.1f}s")
+    layers = []
+    for i in range(args.layers):
+        d = i % args.distinct_layers
+        src = {name: base[(d, j, name)] for j, name in enumerate(LAYER)}
+        layers.append(src if i < args.distinct_layers else {k: v.clone() for k, v in src.items()})
+    for layer in layers:
+        for t in layer.values():
+            t._gemm_tiling() if m > 8 else t._tiling(m)
+    torch.cuda.synchronize()
+    frame_bytes = sum(t.frame_bytes for layer in layers for t in layer.values())
+    resident = sum(t.resident_bytes for layer in layers for t in layer.values())
+    dense = sum(2 * r * c for r, c in LAYER.values()) * args.layers
+    log(f"{args.layers} layers resident: {dense} BF16 bytes as {frame_bytes} frame bytes, {resident} device bytes; "
+        f"torch reports {torch.cuda.memory_allocated()} allocated")
+
+    rng = np.random.default_rng(7)
+    x = {k: torch.from_numpy(bf16_words(rng.normal(0, 1, size=(m, k)))).view(torch.bfloat16).cuda()
+         for k in {c for _, c in LAYER.values()}}
+
+    def step():
+        for layer in layers:
+            for name, t in layer.items():
+                t.linear(x[LAYER[name][1]], batch_invariant=m > 8)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    # per-launch durations of the first layer's kernels, on the stream they run on
+    probes = {name: [] for name in LAYER}
+    wall0 = time.perf_counter()
+    for _ in range(args.steps):
+        for i, layer in enumerate(layers):
+            for name, t in layer.items():
+                if i == 0:
+                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    a.record()
+                t.linear(x[LAYER[name][1]], batch_invariant=m > 8)
+                if i == 0:
+                    b.record()
+                    probes[name].append((a, b))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    for layer in layers:
+        for name, t in layer.items():
+            if t.error.item():
+                sys.exit(f"bench.py: decoder error word set for {name}")
+    ms = {name: float(np.mean([a.elapsed_time(b) for a, b in ev])) for name, ev in probes.items()}
+    alg = {name: algorithmic_bytes(layers[0][name], m) for name in LAYER}
+    step_bytes = sum(algorithmic_bytes(t, m)["total"] for layer in layers[:args.distinct_layers] for t in layer.values())
+    step_bytes = step_bytes * args.layers // args.distinct_layers
+    ms_per_step = wall / args.steps * 1e3
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+    dom = max(LAYER, key=lambda n_: ms[n_])
+    achieved = alg[dom]["total"] / (ms[dom] * 1e-3) / 1e9
+    kernel = "grf::fused_gemm_kernel<grf::SegmentWalk, MT>" if m > 8 else f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, false>"
+    print(json.dumps({
+        "metric": "compressed-weight decode-GEMV GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": f"whole stack resident: {args.layers} layers x (q 5120->6144, k/v 5120->1024, o 6144->5120, "
+                               f"gate/up 5120->17408, down 17408->5120), one pass through every coded linear at batch {m}",
+                   "batch": m, "layers": args.layers, "distinct_layers": args.distinct_layers,
+                   "linears": args.layers * len(LAYER)},
+        "dense_bf16_bytes": dense, "frame_bytes": frame_bytes, "resident_device_bytes": resident,
+        "algorithmic_bytes_per_step": step_bytes,
+        "effective_bf16_GBps": round(dense / (ms_per_step * 1e-3) / 1e9, 2),
+        "tok_s_equiv": round(m / (ms_per_step * 1e-3), 1),
+        "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
+        "per_kernel": {n_: {"ms": round(ms[n_], 4), "alg_bytes": alg[n_]["total"],
+                            "GBps": round(alg[n_]["total"] / (ms[n_] * 1e-3) / 1e9, 2)} for n_ in LAYER},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": f"{kernel} on {dom}"},
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -122,9 +236,19 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB read + 128 MiB write elementwise kernel three times, so that a "
                          "counter profile of this command holds a kernel of known traffic to scale by")
+    ap.add_argument("--workload", choices=("mlp", "stack"), default="mlp",
+                    help="mlp: the three MLP matrices of one layer (the headline); stack: every coded linear of "
+                         "--layers layers resident at once, one pass at batch 64 (or --batch)")
+    ap.add_argument("--layers", type=int, default=64)
+    ap.add_argument("--distinct-layers", type=int, default=1,
+                    help="stack: layers encoded from their own seeds; the rest are device copies of these")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this decode path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists)")
+    if args.workload == "stack":
+        if not 1 <= args.distinct_layers <= args.layers:
+            sys.exit("bench.py: --distinct-layers must be between 1 and --layers")
+        return run_stack(args)
 
     import torch
     from georefine_amd import bitexact_context_codec as codec

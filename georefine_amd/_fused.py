@@ -104,14 +104,21 @@ def lds_bytes(nc, lognb, tabn, m, p, s, r, piece_cap):
     return total
 
 
-def lds_bytes_gemm(nc, lognb, tabn, m16, p, r, piece_cap):
+GEMM_MAX_TILES = 4  # 16-row activation tiles of one GEMM launch
+
+
+def gemm_shape(p, r):
+    """(row blocks, quads, threads) of the GEMM workgroup for p lanes per row and r rows: a
+    wave walks four lane-segments of sixteen rows."""
+    row_blocks, quads = -(-r // 16), -(-p // 4)
+    return row_blocks, quads, row_blocks * quads * 64
+
+
+def lds_bytes_gemm(nc, lognb, tabn, p, r, piece_cap):
     a16 = lambda v: (v + 15) // 16 * 16
-    pitch = p * 32 + 8
     total = a16(nc * (a16((tabn + 1) * 8) + (1 << lognb)))
     total = a16(total + r * piece_cap)
-    total = a16(total + a16(r) * pitch)
-    total = a16(total + m16 * pitch)
-    return total
+    return max(total, gemm_shape(p, r)[2] // 64 * GEMM_MAX_TILES * 1024)  # later: every wave's partial sums
 
 
 def piece_capacity(offsets, rows, spr, p):
@@ -127,7 +134,20 @@ def piece_capacity(offsets, rows, spr, p):
     return (longest + 2 + 15) // 16 * 16
 
 
-def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
+def _tiles(class_rows, r):
+    return sum(-(-int(cnt) // r) for cnt in class_rows if cnt)
+
+
+def _spread_rows(class_rows, r, capacity, floor=1):
+    """Fewer rows per tile while the tiles still fit the workgroup slots of the rounds
+    already paid for: idle lanes do not slow a workgroup down, idle CUs do (measured +4 % on
+    17408 x 5120 going from 464 tiles of 38 rows to 512 of 34)."""
+    while r > floor and _tiles(class_rows, r - 1) <= capacity:
+        r -= 1
+    return r
+
+
+def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
     """(threads T, lanes_per_row P, rows_per_tile R, ...): best modelled throughput.
 
     The walk is a chain of dependent steps per lane, so time ~ steps per lane x rounds
@@ -150,21 +170,14 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
             r = threads // p
             if forced_rows:
                 r = min(r, forced_rows)
-            if gemm:  # see below: at most waves/2 column blocks of 16 rows
-                r = min(r, (threads // 128) * 16)
             if r == 0:
                 continue
             n_slabs = -(-spr // p)
             if not forced and p > 1 and -(-spr // (p - 1)) == n_slabs:
                 continue  # a narrower slab of the same count wastes fewer lanes; it was scored already
-            if gemm:
-                # every 16-row column block needs a wave, and a wave owns at most 4 of the 8 row tiles
-                waves_wg, col_blocks = threads // 64, -(-r // 16)
-                if col_blocks > waves_wg or -(-8 // (waves_wg // col_blocks)) > 4:
-                    continue
             lanes = p * r
             lane_eff = spr / (n_slabs * p) * (lanes / threads)
-            tiles = sum(-(-int(cnt) // r) for cnt in class_rows if cnt)
+            tiles = _tiles(class_rows, r)
             fill = total_rows / (tiles * r)
             cap = piece_cap_fn(p)
             lds = lds_fn(p, r, cap)
@@ -184,17 +197,56 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, gemm=False):
     if best is None:
         raise FusedUnsupported("no tiling fits in LDS")
     _, threads, p, r, n_slabs, tiles, cap, lds, capacity = best
-    # Spread the rows over every workgroup slot of the rounds already paid for: fewer rows
-    # per tile cost nothing (idle lanes do not slow a workgroup down), idle CUs do
-    # (measured +4 % on 17408 x 5120 going from 464 tiles of 38 rows to 512 of 34).
-    if not gemm and not forced_rows:
-        while r > 1:
-            fewer = sum(-(-int(cnt) // (r - 1)) for cnt in class_rows if cnt)
-            if fewer > capacity:
-                break
-            r, tiles = r - 1, fewer
-        lds = lds_fn(p, r, cap)
+    if not forced_rows:
+        r = _spread_rows(class_rows, r, capacity)
+        tiles, lds = _tiles(class_rows, r), lds_fn(p, r, cap)
     return threads, p, r, n_slabs, tiles, cap, lds
+
+
+GEMM_WAVES_PER_SIMD = int(os.environ.get("GEOREFINE_GEMM_WAVES", "6"))
+
+
+def choose_gemm_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
+    """Tiling of the GEMM kernel: workgroups of (row blocks of 16) x (quads of 4
+    lane-segments) waves.  Same model as choose_tiling, counted in waves: a wave is busy
+    for as long as its busiest lane, so idle lanes inside a wave are free, idle waves and
+    idle CUs are not."""
+    best = None
+    total_rows = sum(int(c) for c in class_rows)
+    forced = os.environ.get("GEOREFINE_FUSED_GEMM_TILING")  # "lanes_per_row,rows": experiments only
+    choices = None
+    if forced:
+        p_, r_ = (int(v) for v in forced.split(","))
+        choices = [(min(p_, spr), r_)]
+    else:
+        choices = [(min(4 * quads, spr), 16 * blocks) for quads in range(1, -(-spr // 4) + 1)
+                   for blocks in range(1, 17) if quads * blocks <= 16]
+    for p, r in dict.fromkeys(choices):
+        row_blocks, quads, threads = gemm_shape(p, r)
+        if threads > 1024:
+            continue
+        n_slabs = -(-spr // p)
+        tiles = _tiles(class_rows, r)
+        cap = piece_cap_fn(p)
+        lds = lds_fn(p, r, cap)
+        if lds > MAX_LDS:
+            continue
+        per_simd = -(-(threads // 64) // 4)
+        per_cu = max(1, min(GEMM_WAVES_PER_SIMD // per_simd, MAX_LDS // lds))
+        slots = cus * per_cu
+        rounds = -(-tiles // slots)
+        r_used = r if forced else _spread_rows(class_rows, r, rounds * slots, floor=16 * (row_blocks - 1) + 1)
+        tiles_used = _tiles(class_rows, r_used)
+        # work = lane-steps; capacity = every wave slot of every round for the whole walk
+        work = total_rows * spr
+        paid = rounds * slots * (threads // 64) * 16 * 4 * n_slabs
+        waves = per_cu * (threads // 64)
+        score = work / paid * min(1.0, waves / 24)
+        if best is None or score > best[0] + 1e-9:
+            best = (score, threads, p, r_used, n_slabs, tiles_used, cap, lds_fn(p, r_used, cap))
+    if best is None:
+        raise FusedUnsupported("no GEMM tiling fits in LDS")
+    return best[1:]
 
 
 def build_tiles(row_class, nr, r):
@@ -259,9 +311,9 @@ class FramePlan:
     def gemm_tiling(self):
         """The one tiling every fused GEMM launch uses, whatever its row count: the order in
         which an output element accumulates follows the tiling, so it must not change with M."""
-        threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
+        threads, p, r, n_slabs, n_tiles, cap, lds = choose_gemm_tiling(
             self.spr, self.class_rows, self._cap,
-            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, 64, p_, r_, cap_), gemm=True)
+            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, p_, r_, cap_))
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,

@@ -47,6 +47,7 @@ class GrfPpcxFused(ctypes.Structure):
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
                   "grf_bctx_fused_decode", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
+                  "grf_gemm_workspace_bytes",
                   "grf_ppcx_bins", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_last_error",
                   "grf_abi_version")
 
@@ -62,10 +63,13 @@ def declare(L):
     tiling = ctypes.POINTER(GrfFusedTiling)
     L.grf_bctx_gemv.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, u32, u32, vp, u32, vp, vp, vp]
     L.grf_bctx_gemv.restype = i
-    L.grf_bctx_gemm.argtypes = L.grf_bctx_gemv.argtypes
+    L.grf_bctx_gemm.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, u32, u32, vp, u32, vp, vp, ctypes.c_size_t,
+                                vp, vp]
     L.grf_bctx_gemm.restype = i
-    L.grf_bctx_gemm_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, u32]
+    L.grf_bctx_gemm_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), tiling]
     L.grf_bctx_gemm_lds_bytes.restype = u32
+    L.grf_gemm_workspace_bytes.argtypes = [u32, u32]
+    L.grf_gemm_workspace_bytes.restype = ctypes.c_size_t
     L.grf_bctx_fused_decode.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, vp, vp]
     L.grf_bctx_fused_decode.restype = i
     L.grf_bctx_fused_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, u32]
@@ -76,7 +80,8 @@ def declare(L):
     L.grf_ppcx_fused_decode.restype = i
     L.grf_ppcx_gemv.argtypes = [ctypes.POINTER(GrfPpcxFused), tiling, vp, vp, u32, u32, vp, u32, vp, vp, vp]
     L.grf_ppcx_gemv.restype = i
-    L.grf_ppcx_gemm.argtypes = L.grf_ppcx_gemv.argtypes
+    L.grf_ppcx_gemm.argtypes = [ctypes.POINTER(GrfPpcxFused), tiling, vp, vp, u32, u32, vp, u32, vp, vp,
+                                ctypes.c_size_t, vp, vp]
     L.grf_ppcx_gemm.restype = i
     L.grf_last_error.restype = ctypes.c_char_p
     L.grf_abi_version.restype = i

@@ -116,6 +116,7 @@ def _device_stream(buffers, name, vocab, nctx):
 class HipContextTensor:
     """A BCTX-coded BF16 matrix resident on one MI355X."""
 
+    GEMV_UP_TO = 2    # activation rows linear() gives to the vector-ALU kernel
     DENSE_ABOVE = 64  # activation rows above which linear() decodes to a dense transient
 
     def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None):
@@ -170,6 +171,13 @@ class HipContextTensor:
         self.error = torch.zeros((), device=self.device, dtype=torch.int32)
         self.resident_bytes = int(sum(t.numel() * t.element_size() for t in self.buffers.values())
                                   + self.error.numel() * self.error.element_size())
+        self._plan = plan
+        self._bind()
+
+    def _bind(self):
+        """Descriptors over this object's device buffers (their addresses go into the structures
+        the kernels take), and the first tilings."""
+        plan = self._plan
         self._frame = None
         if self.mode != 1:
             f = _hip_abi.GrfBctxFrame()
@@ -178,10 +186,9 @@ class HipContextTensor:
             f.row_class = self.buffers["rows"].data_ptr()
             f.col_class = self.buffers["columns"].data_ptr()
             f.rows, f.cols = self.shape
-            f.nc, f.mode, f.stride = self.nc, self.resident_mode, stride
+            f.nc, f.mode, f.stride = self.nc, self.resident_mode, self.stride
             f.main.n_bytes = self._main_bytes
             self._frame = f
-        self._plan = plan
         self._tilings = {}
         if plan is not None:
             d = _hip_abi.GrfBctxFused()
@@ -200,6 +207,20 @@ class HipContextTensor:
                 self._tiling(0)
             except _fused.FusedUnsupported as exc:
                 self.fused, self.fused_reason = None, str(exc)
+
+    def clone(self):
+        """A second resident copy of the same coded matrix: every device buffer is duplicated
+        (nothing is decoded or indexed again), so a stack of layers with equal weights can be
+        laid out in device memory at the cost of one device-to-device copy each."""
+        import copy
+        import torch
+        other = copy.copy(self)
+        other.buffers = {k: v.clone() for k, v in self.buffers.items()}
+        other.error = torch.zeros_like(self.error)
+        other.resident_bytes = int(sum(t.numel() * t.element_size() for t in other.buffers.values())
+                                   + other.error.numel() * other.error.element_size())
+        other._bind()
+        return other
 
     def _tiling(self, m):
         """Device copy of the tiling used for m activation rows (0 = store sink); tilings
@@ -294,14 +315,20 @@ class HipContextTensor:
         y = torch.empty((x2.shape[0], self.shape[0]), device=self.device, dtype=torch.bfloat16)
         return x2, bias, y
 
-    def _fused_call(self, fn, tiling, x, bias, check):
+    def _fused_call(self, fn, tiling, x, bias, check, *, workspace=False):
+        import torch
         lead = x.shape[:-1]
         x2, bias, y = self._prepare_activations(x, bias, 4)
         if x2.shape[0]:
             self.error.zero_()
+            extra = ()
+            if workspace:  # transient: the activations in the matrix cores' operand order
+                size = self._lib.grf_gemm_workspace_bytes(self.shape[1], x2.shape[0])
+                packed = torch.empty(size, device=self.device, dtype=torch.uint8)
+                extra = (packed.data_ptr(), size)
             self._launch(fn, ctypes.byref(self.fused), ctypes.byref(tiling), x2.data_ptr(), x2.stride(0),
                          x2.shape[0], y.data_ptr(), y.stride(0), bias.data_ptr() if bias is not None else None,
-                         self.error.data_ptr())
+                         *extra, self.error.data_ptr())
             self._check(check)
         return y.reshape(*lead, self.shape[0])
 
@@ -320,13 +347,14 @@ class HipContextTensor:
         a row's output bits are the same whatever else is in the batch."""
         if self.fused is None:
             raise base.CodecError("frame is not eligible for the fused kernels: " + self.fused_reason)
-        return self._fused_call(self._lib.grf_bctx_gemm, self._gemm_tiling()[0], x, bias, check)
+        return self._fused_call(self._lib.grf_bctx_gemm, self._gemm_tiling()[0], x, bias, check, workspace=True)
 
     def linear(self, x, bias=None, *, check=False, batch_invariant=False):
         """y = x @ W.T (+ bias) with W decoded inside the kernel; x is BF16 [..., K].
 
-        Up to 8 activation rows run the fused decode-GEMV, up to 64 the fused decode-GEMM;
-        above that a fused decode to a dense transient followed by the library matmul is
+        One or two activation rows run the fused decode-GEMV, up to 64 the fused decode-GEMM
+        (one launch; from three rows on it is faster than the GEMV, whose cost grows with every
+        row); above that a fused decode to a dense transient followed by the library matmul is
         faster (measured crossover between 64 and 96 rows).  ``batch_invariant=True`` sends
         every row count through the GEMM so that a row's output never depends on the batch
         it arrives in.  Frames the fused kernels cannot take are decoded on the device and
@@ -335,7 +363,7 @@ class HipContextTensor:
         m = math.prod(x.shape[:-1])
         if self.fused is None or (m > self.DENSE_ABOVE and not batch_invariant):
             return F.linear(x.to(self.device), self.decode(check=check), bias)
-        if batch_invariant or m > 8 or m == 0:
+        if batch_invariant or m > self.GEMV_UP_TO or m == 0:
             return self.gemm(x, bias, check=check)
         return self.gemv(x, bias, check=check)
 

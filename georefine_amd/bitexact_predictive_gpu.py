@@ -132,7 +132,8 @@ def _read_frame(frame, reference, stride, *, fused=False, fused_segment=None):
 class HipPredictiveTensor:
     """A PPCX-coded BF16 matrix resident on one MI355X; decoding needs the reference matrix."""
 
-    DENSE_ABOVE = 8  # activation rows above which linear() decodes to a dense transient
+    GEMV_UP_TO = 1    # activation rows linear() gives to the vector-ALU kernel
+    DENSE_ABOVE = 64  # activation rows above which linear() decodes to a dense transient
 
     def __init__(self, frame, reference_uint16_numpy, stride=1024, device="cuda:0", *, fused=True,
                  fused_segment=None):
@@ -253,19 +254,38 @@ class HipPredictiveTensor:
 
     def linear(self, reference_bf16_device, x, bias=None, *, check=False, batch_invariant=False):
         """y = x W^T + bias with W decoded on the fly against the reference: the fused GEMV for
-        up to 8 activation rows; above that the fused decode to a dense transient plus the
-        library matmul is faster (the 16 bin contexts leave the GEMM little LDS), unless
-        ``batch_invariant`` asks for the fused GEMM, whose rows do not depend on the batch.
-        Frames the tile walker cannot take are decoded and multiplied densely."""
+        one activation row, the fused GEMM (matrix cores, one launch) for up to 64; above that
+        the fused decode to a dense transient plus the library matmul is faster, unless
+        ``batch_invariant`` asks for the fused GEMM throughout, whose rows do not depend on
+        the batch.  Frames the tile walker cannot take are decoded and multiplied densely."""
         import torch
         m = math.prod(x.shape[:-1])
         if self.fused is None or x.dtype != torch.bfloat16 or (m > self.DENSE_ABOVE and not batch_invariant):
             return torch.nn.functional.linear(x, self.decode(reference_bf16_device, check=check), bias)
+        return self._product(reference_bf16_device, x, bias, check, batch_invariant or m > self.GEMV_UP_TO)
+
+    def gemv(self, reference_bf16_device, x, bias=None, *, check=False):
+        """Fused decode-GEMV (vector ALUs) for 1..8 activation rows; a row's result does not
+        depend on how many rows the call carries."""
+        if not 1 <= math.prod(x.shape[:-1]) <= 8:
+            raise ValueError("gemv takes 1..8 activation rows")
+        return self._product(reference_bf16_device, x, bias, check, False)
+
+    def gemm(self, reference_bf16_device, x, bias=None, *, check=False):
+        """Fused decode-GEMM (matrix cores) for any number of activation rows, batch-invariant."""
+        return self._product(reference_bf16_device, x, bias, check, True)
+
+    def _product(self, reference_bf16_device, x, bias, check, use_gemm):
+        import torch
+        if self.fused is None:
+            raise codec.CodecError("frame is not eligible for the fused kernels: " + str(self.fused_reason))
+        if x.dtype != torch.bfloat16:
+            raise ValueError("activation must be bfloat16")
+        m = math.prod(x.shape[:-1])
         ref = self._reference(reference_bf16_device)
         x2 = x.reshape(-1, x.shape[-1]).to(self.device)
         if x2.shape[-1] != self.shape[1]:
             raise ValueError("activation width does not match the weight")
-        use_gemm = batch_invariant or m > 8
         align = 4 if use_gemm else 2  # elements: the GEMM reads 8 bytes at a time, the GEMV 4
         if x2.stride(-1) != 1 or x2.stride(0) % align or x2.data_ptr() % (2 * align):
             x2 = x2.contiguous()
@@ -277,14 +297,19 @@ class HipPredictiveTensor:
             with torch.cuda.device(self.device):
                 bins, status = self._bins(ref)
                 if not status:
+                    extra = ()
                     if use_gemm:
                         fn, tiling = self._lib.grf_ppcx_gemm, self._tiling_for("gemm")[0]
+                        # transient: the activations in the matrix cores' operand order
+                        size = self._lib.grf_gemm_workspace_bytes(self.shape[1], m)
+                        packed = torch.empty(size, device=self.device, dtype=torch.uint8)
+                        extra = (packed.data_ptr(), size)
                     else:
                         fn = self._lib.grf_ppcx_gemv
                         tiling = self._tiling_for(next(v for v in (1, 2, 4, 8) if v >= m))[0]
                     status = fn(ctypes.byref(self.fused), ctypes.byref(tiling), bins.data_ptr(), x2.data_ptr(),
                                 x2.stride(0), m, y.data_ptr(), y.stride(0),
-                                bias.data_ptr() if bias is not None else None, self.error.data_ptr(),
+                                bias.data_ptr() if bias is not None else None, *extra, self.error.data_ptr(),
                                 torch.cuda.current_stream(self.device).cuda_stream)
             self._status(status, check)
         return y.reshape(*x.shape[:-1], self.shape[0])

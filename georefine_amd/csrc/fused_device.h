@@ -320,6 +320,8 @@ struct SegmentWalk {
   const uint4 *ccp;
   uint32_t n0, n1, n2;
   uint4 nc4;
+  Raw6x16 rr;      // the group being decoded
+  uint32_t cw[4];
 
   // Global reads for segment `seg_` (elem0 / col0: its first element / column), issued
   // before the workgroup waits for the slab's stream bytes so that their latency overlaps it.
@@ -340,28 +342,39 @@ struct SegmentWalk {
     c.j = ip0;
   }
 
-  // Decode symbols [t, t+16) of the segment into eight BF16 pairs (word k in the low half,
-  // k+1 in the high half); loads the registers for the following group meanwhile.
-  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const FusedParams &q, uint32_t (&pair)[8]) {
-    Raw6x16 rr;
+  // Start the group of symbols [t, t+16): unpack its residuals and column classes, and load
+  // the registers of the following group meanwhile.
+  __device__ __forceinline__ void begin16(uint32_t t, uint32_t S) {
     rr.set(n0, n1, n2);
-    const uint32_t cw[4] = {nc4.x, nc4.y, nc4.z, nc4.w};
-    {  // the last group loads itself again rather than branch around the loads
-      const uint32_t next = min(t / 16 + 1, S / 16 - 1);
-      const uint32_t *nx = rawp + next * 3;
-      n0 = nx[0];
-      n1 = nx[1];
-      n2 = nx[2];
-      nc4 = ccp[next];
-    }
-    uint32_t bits[16];
-#define GRF_STEP(k) bits[k] = fused_word_bits(fused_symbol<k>(c, cw[(k) / 4], q), rr.field<k>());
+    cw[0] = nc4.x;
+    cw[1] = nc4.y;
+    cw[2] = nc4.z;
+    cw[3] = nc4.w;
+    // the last group loads itself again rather than branch around the loads
+    const uint32_t next = min(t / 16 + 1, S / 16 - 1);
+    const uint32_t *nx = rawp + next * 3;
+    n0 = nx[0];
+    n1 = nx[1];
+    n2 = nx[2];
+    nc4 = ccp[next];
+  }
+  // Half H (0 or 1) of the group: eight symbols into four BF16 pairs (word k in the low
+  // half, k+1 in the high half).
+  template <int H>
+  __device__ __forceinline__ void half(const FusedParams &q, uint32_t (&pair)[4]) {
+    uint32_t bits[8];
+#define GRF_STEP(i) bits[i] = fused_word_bits(fused_symbol<8 * H + (i)>(c, cw[(8 * H + (i)) / 4], q), rr.field<8 * H + (i)>());
     GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
-    GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
 #undef GRF_STEP
-    c.end_group();
+    if (H == 1) c.end_group();
 #pragma unroll
-    for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
+    for (int k = 0; k < 4; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
+  }
+  // Symbols [t, t+16) of the segment into eight BF16 pairs.
+  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const FusedParams &q, uint32_t (&pair)[8]) {
+    begin16(t, S);
+    half<0>(q, reinterpret_cast<uint32_t (&)[4]>(pair[0]));
+    half<1>(q, reinterpret_cast<uint32_t (&)[4]>(pair[4]));
   }
 
   // the segment must end exactly on the next checkpoint

@@ -199,72 +199,119 @@ int launch_gemv(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
 }
 
 // ---------------------------------------------------------------- GEMM sink
+//
+// Nothing decoded ever leaves the registers.  A wave covers 16 rows of the tile and four
+// lane-segments: lane l walks segment 4*quad + l/16 of row 16*block + l%16, and the eight
+// words a lane decodes in half a group are, as they stand, its share of the B operand of
+// v_mfma_f32_16x16x32_bf16 (column l%16, k-slots 8*(l/16)..+7).  The k-slots of one MFMA
+// are therefore 8 consecutive columns out of each of four different segments; the A
+// operand pairs them with the same columns of 16 activation rows, read with one 16-byte
+// load per lane from a copy of the activations laid out for exactly that (column chunk
+// major, see pack_activations_kernel).  No workgroup barrier inside a slab, no tile in LDS.
+//
+// At the end the waves of a row block (one per quad) hold partial sums over their
+// segments; they are added through LDS in quad order.
 
-typedef short short4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t kGroup = 16;      // columns decoded between two contractions
-constexpr uint32_t kMaxAcc = 4;      // 16x16 output blocks a wave may own
-constexpr uint32_t kMaxRowsPerLaunch = 128;
-constexpr uint32_t kChunkTiles = 4;  // 16-row activation tiles staged in LDS at a time (64 rows)
+constexpr uint32_t kMaxRowsPerLaunch = 64;  // four 16-row activation tiles per launch
+constexpr uint32_t kMaxTiles = kMaxRowsPerLaunch / 16;
 
-// LDS regions of the GEMM kernel.  Word and activation tiles hold, per (row, p), one
-// 32-byte run of 16 BF16 values; a row's runs are padded by 8 bytes so that the 16 rows
-// an MFMA operand touches fall into different banks.
-struct GemmLdsLayout {
-  uint32_t blocks, block_pitch, stream, wt, wt_pitch, xt, xt_pitch, total;
-  __host__ __device__ GemmLdsLayout(const grf_bctx_fused &f, const grf_fused_tiling &g, uint32_t m16) {
-    uint32_t at = 0;
-    blocks = at;
-    block_pitch = grf::fused_table_bytes(f) + (1u << f.lognb);
-    at = grf::align_up(at + f.nc * block_pitch, 16);
-    stream = at;
-    at = grf::align_up(at + g.rows_per_tile * g.piece_cap, 16);
-    wt_pitch = g.lanes_per_row * 32 + 8;
-    xt_pitch = wt_pitch;
-    wt = at;
-    at = grf::align_up(at + grf::align_up(g.rows_per_tile, 16) * wt_pitch, 16);
-    xt = at;
-    at = grf::align_up(at + m16 * xt_pitch, 16);
-    total = at;
+// Workgroup shape of the GEMM kernel for a tiling: row blocks x quads of lane-segments.
+struct GemmShape {
+  uint32_t row_blocks, quads, threads;
+  __host__ __device__ explicit GemmShape(const grf_fused_tiling &g) {
+    row_blocks = (g.rows_per_tile + 15) / 16;
+    quads = (g.lanes_per_row + 3) / 4;
+    threads = row_blocks * quads * 64;
   }
 };
 
-// MT: 16-row activation tiles per launch (m_rows <= 16*MT)
+// Tables and stream pieces as in the GEMV kernel; the same memory later holds the partial
+// sums of every wave (1 KiB per wave and activation tile).
+struct GemmLdsLayout {
+  uint32_t blocks, block_pitch, stream, total;
+  __host__ __device__ GemmLdsLayout(const grf_bctx_fused &f, const grf_fused_tiling &g) {
+    blocks = 0;
+    block_pitch = grf::fused_table_bytes(f) + (1u << f.lognb);
+    stream = grf::align_up(f.nc * block_pitch, 16);
+    total = grf::align_up(stream + g.rows_per_tile * g.piece_cap, 16);
+    const uint32_t sums = GemmShape(g).threads / 64 * kMaxTiles * 1024;
+    if (total < sums) total = sums;
+  }
+};
+
+// Activations in operand order: the 8 columns [8c, 8c+8) of row m at xp[c * m_pad + m]
+// (16 bytes); rows m_rows..m_pad-1 are zero.  A group of 64 threads moves 8 chunks of 8
+// rows, reading 128-byte runs of x and writing 128-byte runs of xp.
+static __global__ __launch_bounds__(256) void pack_activations_kernel(const uint16_t *x, uint32_t ldx, uint32_t m_rows,
+                                                                uint32_t m_pad, uint32_t chunks, uint4 *xp) {
+  const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
+  const uint32_t cc = idx % 8, ml = (idx / 8) % 8, blk = idx / 64;
+  const uint32_t m_blocks = m_pad / 8;
+  const uint32_t m = (blk % m_blocks) * 8 + ml, c = (blk / m_blocks) * 8 + cc;
+  if (c >= chunks) return;
+  uint4 v = make_uint4(0u, 0u, 0u, 0u);
+  if (m < m_rows) {
+    const uint2 *src = reinterpret_cast<const uint2 *>(x + (size_t)m * ldx + c * 8);
+    const uint2 a = src[0], b = src[1];
+    v = make_uint4(a.x, a.y, b.x, b.y);
+  }
+  xp[(size_t)c * m_pad + m] = v;
+}
+
+template <int MT>
+__device__ __forceinline__ void gemm_load_x(uint4 (&xa)[MT], const uint4 *xl, bool feeds) {
+#pragma unroll
+  for (int j = 0; j < MT; ++j) xa[j] = feeds ? xl[j * 16] : make_uint4(0u, 0u, 0u, 0u);
+}
+
+template <int MT>
+__device__ __forceinline__ void gemm_contract(float4v (&acc)[MT], const uint4 (&xa)[MT], const uint32_t (&w)[4]) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint4 wv = make_uint4(w[0], w[1], w[2], w[3]);
+  const bf16x8_t b = __builtin_bit_cast(bf16x8_t, wv);
+#pragma unroll
+  for (int j = 0; j < MT; ++j)
+    acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, xa[j]), b, acc[j], 0, 0, 0);
+#else
+  (void)acc;
+  (void)xa;
+  (void)w;
+#endif
+}
+
+// MT: 16-row activation tiles of this launch (m_rows <= 16 * MT, xp packed with m_pad = 16 * MT)
 template <class Walk, int MT>
-__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_bctx_fused f, grf_fused_tiling g,
-                                                                            const uint16_t *x, uint32_t ldx,
-                                                                            uint32_t m_rows, uint16_t *y,
-                                                                            uint32_t ldy, const uint16_t *bias,
-                                                                            int32_t *error) {
+__global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_gemm_kernel(grf_bctx_fused f, grf_fused_tiling g,
+                                                                            const uint4 *xp, uint32_t m_rows,
+                                                                            uint16_t *y, uint32_t ldy,
+                                                                            const uint16_t *bias, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  constexpr uint32_t CT = MT < kChunkTiles ? MT : kChunkTiles;  // activation tiles per chunk
-  const GemmLdsLayout L(f, g, CT * 16);
+  const GemmLdsLayout L(f, g);
+  const GemmShape shape(g);
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
+  constexpr uint32_t m_pad = MT * 16;
 
-  const uint32_t r = tid / P, p = tid % P;
-  const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
+  const uint32_t wave = tid / 64, lane = tid % 64;
+  const uint32_t rb = wave % shape.row_blocks, quad = wave / shape.row_blocks;
+  const uint32_t r = rb * 16 + lane % 16, p = quad * 4 + lane / 16;
+  const uint32_t row = (r < R && p < P) ? g.tile_rows[tile * R + r] : grf::kNoRow;
   grf::PieceSpan span{0, 0};  // started before the table copy so that the latencies overlap
   if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
 
-  // contraction roles: wave -> one 16-column block of the tile (nt) and every MW-th row tile
-  const uint32_t wave = tid / 64, lane = tid % 64, nwaves = nthreads / 64;
-  const uint32_t NT = (R + 15) / 16;
-  const uint32_t MW = nwaves / NT;  // waves per column block (host guarantees >= 1)
-  const uint32_t nt = wave % NT, mslot = wave / NT;
-  const bool contracts = mslot < MW;
-  const uint32_t li = lane % 16, kq = lane / 16;
-  float4v acc[kMaxAcc];
+  float4v acc[MT];
 #pragma unroll
-  for (uint32_t j = 0; j < kMaxAcc; ++j) acc[j] = (float4v){0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < MT; ++j) acc[j] = (float4v){0.f, 0.f, 0.f, 0.f};
   uint32_t bad = 0;
 
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
-    __syncthreads();  // previous slab's stream bytes and tiles are no longer read
+    if (b) __syncthreads();  // everyone is done with the previous slab's stream bytes
     const uint32_t first_seg = b * P;
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
     const uint32_t piece_off = L.stream + r * g.piece_cap;
@@ -280,125 +327,112 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_kernel(grf_b
         span.fetch(f, seg_base + P, min(P, f.segs_per_row - first_seg - P));
     }
     __syncthreads();
+    if (__ballot(active) == 0) continue;  // nothing to walk in this wave (the branch is per wave)
     if (active) w.start(piece_off, a0);
-    for (uint32_t t = 0; t < S; t += kGroup) {
-      if (active) {  // 16 words of this lane's segment -> word tile
-        uint32_t pair[8];
-        w.decode16(t, S, q, pair);
-        uint2 *dst = reinterpret_cast<uint2 *>(lds + L.wt + r * L.wt_pitch + p * 32);
-        dst[0] = make_uint2(pair[0], pair[1]);
-        dst[1] = make_uint2(pair[2], pair[3]);
-        dst[2] = make_uint2(pair[4], pair[5]);
-        dst[3] = make_uint2(pair[6], pair[7]);
+    // A lane's k-slots are real columns when its segment exists, whether or not its own
+    // row does; other lanes feed zeros (their weights are zero too, but 0 * NaN is not).
+    const bool feeds = p < nseg;
+    const uint4 *xl = xp + (size_t)(feeds ? col0 / 8 : 0) * m_pad + lane % 16;
+    uint4 xa[MT];
+    gemm_load_x<MT>(xa, xl, feeds);
+    for (uint32_t t = 0; t < S; t += 16) {
+      uint32_t lo[4] = {0u, 0u, 0u, 0u}, hi[4] = {0u, 0u, 0u, 0u};
+      if (active) {
+        w.begin16(t, S);
+        w.template half<0>(q, lo);
       }
-      // The same 16 columns of every lane-segment of the activations -> activation tile, 64
-      // rows at a time: the tile's size bounds the lanes per row a tiling can have, and an
-      // output element's sequence of operations does not depend on the chunking.
-      for (uint32_t mc = 0; mc < MT; mc += CT) {
-        if (mc) __syncthreads();  // the previous chunk has been consumed
-        for (uint32_t c = tid; c < CT * 16 * P * 4; c += nthreads) {
-          const uint32_t part = c % 4, pp = (c / 4) % P, ml = c / (4 * P), m = mc * 16 + ml;
-          const uint32_t col = (first_seg + pp) * S + t + part * 4;
-          uint2 v = make_uint2(0u, 0u);
-          if (m < m_rows && pp < nseg) v = *reinterpret_cast<const uint2 *>(x + (size_t)m * ldx + col);
-          *reinterpret_cast<uint2 *>(lds + L.xt + ml * L.xt_pitch + pp * 32 + part * 8) = v;
-        }
-        __syncthreads();
-        if (contracts) {
-          const uint8_t *brow = lds + L.wt + (nt * 16 + li) * L.wt_pitch + kq * 8;
-#pragma unroll
-          for (uint32_t j = 0; j < kMaxAcc; ++j) {
-            const uint32_t mt = mslot + j * MW;
-            if (mt >= mc && mt < mc + CT && mt < MT) {
-              const uint8_t *arow = lds + L.xt + ((mt - mc) * 16 + li) * L.xt_pitch + kq * 8;
-              for (uint32_t pp = 0; pp < nseg; ++pp) {
-                const short4v a = *reinterpret_cast<const short4v *>(arow + pp * 32);
-                const short4v bb = *reinterpret_cast<const short4v *>(brow + pp * 32);
-#if defined(__HIP_DEVICE_COMPILE__)
-                acc[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, bb, acc[j], 0, 0, 0);
-#else
-                (void)a;
-                (void)bb;
-#endif
-              }
-            }
-          }
-        }
-      }
-      __syncthreads();  // tiles are overwritten by the next group
+      gemm_contract<MT>(acc, xa, lo);
+      xl += m_pad;
+      gemm_load_x<MT>(xa, xl, feeds);
+      if (active) w.template half<1>(q, hi);
+      gemm_contract<MT>(acc, xa, hi);
+      xl += m_pad;
+      gemm_load_x<MT>(xa, xl, feeds && t + 16 < S);
     }
     if (active && !w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
   }
 
-  if (contracts) {
-    const uint32_t n_local = nt * 16 + li;
+  // partial sums of every wave -> LDS, then each output element adds its quads in order
+  __syncthreads();
+  float *sums = reinterpret_cast<float *>(lds);
+#pragma unroll
+  for (int j = 0; j < MT; ++j)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) sums[((wave * MT + j) * 4 + v) * 64 + lane] = acc[j][v];
+  __syncthreads();
+  const uint32_t per_block = MT * 256;  // values of one row block: [tile j][v][lane]
+  for (uint32_t i = tid; i < shape.row_blocks * per_block; i += nthreads) {
+    const uint32_t blk = i / per_block, within = i % per_block;
+    const uint32_t j = within / 256, v = (within / 64) % 4, ln = within % 64;
+    const uint32_t n_local = blk * 16 + ln % 16, m = j * 16 + (ln / 16) * 4 + v;
     const uint32_t orow = n_local < R ? g.tile_rows[tile * R + n_local] : grf::kNoRow;
-    if (orow != grf::kNoRow) {
-      const float bv = bias ? __uint_as_float((uint32_t)bias[orow] << 16) : 0.f;
-#pragma unroll
-      for (uint32_t j = 0; j < kMaxAcc; ++j) {
-        const uint32_t mt = mslot + j * MW;
-        if (mt < MT) {
-#pragma unroll
-          for (uint32_t i = 0; i < 4; ++i) {
-            const uint32_t m = mt * 16 + kq * 4 + i;
-            if (m < m_rows) y[(size_t)m * ldy + orow] = round_bf16(acc[j][i] + bv);
-          }
-        }
-      }
-    }
+    if (orow == grf::kNoRow || m >= m_rows) continue;
+    // wave index of (quad, block) is quad * row_blocks + block
+    float sum = sums[(blk * MT) * 256 + within];
+    for (uint32_t qd = 1; qd < shape.quads; ++qd) sum += sums[((qd * shape.row_blocks + blk) * MT) * 256 + within];
+    if (bias) sum += __uint_as_float((uint32_t)bias[orow] << 16);
+    y[(size_t)m * ldy + orow] = round_bf16(sum);
   }
   if (bad) atomicOr(error, (int)bad);
 }
 
 template <class Walk, int MT>
 int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
-           uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error, hipStream_t s) {
-  const GemmLdsLayout L(f, g, (MT < kChunkTiles ? MT : kChunkTiles) * 16);
+                     uint16_t *y, uint32_t ldy, const uint16_t *bias, uint4 *xp, int32_t *error, hipStream_t s) {
+  const GemmLdsLayout L(f, g);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused GEMM: LDS demand exceeds 160 KiB");
-  const uint32_t nwaves = g.threads / 64, NT = (g.rows_per_tile + 15) / 16;
-  if (NT > nwaves) return grf::set_error(GRF_BAD_ARGUMENT, "fused GEMM: more column blocks than waves");
-  const uint32_t MW = nwaves / NT;
-  if ((MT + MW - 1) / MW > kMaxAcc)
-    return grf::set_error(GRF_BAD_ARGUMENT, "fused GEMM: tiling leaves more than 4 row tiles per wave");
+  const uint32_t chunks = f.cols / 8, m_pad = MT * 16;
+  const uint32_t pack_threads = (chunks + 7) / 8 * 8 * m_pad;
+  hipLaunchKernelGGL(pack_activations_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, x, ldx, m_rows, m_pad,
+                     chunks, xp);
   auto kernel = fused_gemm_kernel<Walk, MT>;
   if (L.total > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
     if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("LDS attribute: ") + hipGetErrorString(e));
   }
-  hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, x, ldx, m_rows, y, ldy, bias, error);
+  hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, xp, m_rows, y, ldy, bias, error);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused GEMM: ") + hipGetErrorString(e));
   return GRF_OK;
 }
 
-// y = x W^T (+ bias) for any number of activation rows, 128 per launch
+// bytes of the packed copy of the activations one launch needs
+inline size_t gemm_workspace_bytes(uint32_t cols, uint32_t m_rows) {
+  const uint32_t m = m_rows > kMaxRowsPerLaunch ? kMaxRowsPerLaunch : m_rows;
+  const uint32_t tiles = m <= 16 ? 1 : m <= 32 ? 2 : kMaxTiles;
+  return (size_t)(cols / 8) * tiles * 16 * 16;
+}
+
+// y = x W^T (+ bias) for any number of activation rows, 64 per launch.  `workspace` holds
+// the packed activations of one launch; launches follow one another on the stream.
 template <class Walk>
 int launch_gemm(const char *who, const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx,
-                uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error, hipStream_t s) {
+                uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
+                size_t workspace_bytes, int32_t *error, hipStream_t s) {
   if (!m_rows) return GRF_OK;
   if (ldx < f.cols || ldy < f.rows || (ldx & 3) || ((uintptr_t)x & 7))
     return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) +
                                                 ": x must be 8-byte aligned with a leading dimension that is a multiple of 4");
+  if (GemmShape(g).threads != g.threads || g.threads > (uint32_t)grf::kFusedMaxThreads)
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) +
+                                                ": tiling threads must be 64 x ceil(rows_per_tile / 16) x ceil(lanes_per_row / 4)");
+  if (!workspace || ((uintptr_t)workspace & 15) || workspace_bytes < gemm_workspace_bytes(f.cols, m_rows))
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": workspace missing, misaligned or too small");
+  uint4 *xp = static_cast<uint4 *>(workspace);
   for (uint32_t m0 = 0; m0 < m_rows; m0 += kMaxRowsPerLaunch) {
     const uint32_t m = m_rows - m0 < kMaxRowsPerLaunch ? m_rows - m0 : kMaxRowsPerLaunch;
     const uint16_t *xs = x + (size_t)m0 * ldx;
     uint16_t *ys = y + (size_t)m0 * ldy;
     int rc;
-    if (m <= 16) rc = launch_gemm_rows<Walk, 1>(f, g, xs, ldx, m, ys, ldy, bias, error, s);
-    else if (m <= 32) rc = launch_gemm_rows<Walk, 2>(f, g, xs, ldx, m, ys, ldy, bias, error, s);
-    else if (m <= 64) rc = launch_gemm_rows<Walk, 4>(f, g, xs, ldx, m, ys, ldy, bias, error, s);
-    else rc = launch_gemm_rows<Walk, 8>(f, g, xs, ldx, m, ys, ldy, bias, error, s);
+    if (m <= 16) rc = launch_gemm_rows<Walk, 1>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
+    else if (m <= 32) rc = launch_gemm_rows<Walk, 2>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
+    else rc = launch_gemm_rows<Walk, 4>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
     if (rc) return rc;
   }
   return GRF_OK;
 }
 
-inline uint32_t gemm_lds_bytes(const grf_bctx_fused &f, const grf_fused_tiling &g, uint32_t m_rows) {
-  const uint32_t m = m_rows > kMaxRowsPerLaunch ? kMaxRowsPerLaunch : m_rows;
-  const uint32_t mt = m <= 16 ? 1 : m <= 32 ? 2 : 4;  // activations are staged 64 rows at a time
-  return GemmLdsLayout(f, g, mt * 16).total;
-}
+inline uint32_t gemm_lds_bytes(const grf_bctx_fused &f, const grf_fused_tiling &g) { return GemmLdsLayout(f, g).total; }
 
 }  // namespace grf

@@ -107,6 +107,8 @@ struct PpcxWalk {
   const uint2 *binp;      // the segment's bins, 8 bytes per 16 symbols
   uint32_t n0, n1, n2;
   uint2 nb;
+  Raw5x16 rr;      // the group being decoded
+  uint32_t bw[2];
 
   __device__ __forceinline__ static const uint32_t *group_dwords(const uint8_t *rawp, uint32_t g) {
     return reinterpret_cast<const uint32_t *>(rawp + ((10 * g) & ~3u));
@@ -129,31 +131,37 @@ struct PpcxWalk {
     c.j = ip0;
   }
 
-  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const grf::FusedParams &q, uint32_t (&pair)[8]) {
-    Raw5x16 rr;
+  __device__ __forceinline__ void begin16(uint32_t t, uint32_t S) {
     rr.set(n0, n1, n2, (t & 16u) ? 16u : 0u);
-    const uint32_t bw[2] = {nb.x, nb.y};
-    {  // the last group loads itself again rather than branch around the loads
-      const uint32_t next = min(t / 16 + 1, S / 16 - 1);
-      const uint32_t *d = group_dwords(rawp, next);
-      n0 = d[0];
-      n1 = d[1];
-      n2 = d[2];
-      nb = binp[next];
-    }
-    uint32_t bits[16];
-#define GRF_STEP(k)                                                                                   \
+    bw[0] = nb.x;
+    bw[1] = nb.y;
+    // the last group loads itself again rather than branch around the loads
+    const uint32_t next = min(t / 16 + 1, S / 16 - 1);
+    const uint32_t *d = group_dwords(rawp, next);
+    n0 = d[0];
+    n1 = d[1];
+    n2 = d[2];
+    nb = binp[next];
+  }
+  template <int H>
+  __device__ __forceinline__ void half(const grf::FusedParams &q, uint32_t (&pair)[4]) {
+    uint32_t bits[8];
+#define GRF_STEP(i)                                                                                   \
   {                                                                                                   \
-    const uint32_t bin = __builtin_amdgcn_ubfe(bw[(k) / 8], 4 * ((k) % 8), 4);                        \
-    const uint32_t hi = grf::fused_symbol_in<k>(c, __umul24(bin, q.block_pitch), q);                  \
-    bits[k] = hi | rr.field<k>();                                                                     \
+    const uint32_t bin = __builtin_amdgcn_ubfe(bw[H], 4 * (i), 4);                                    \
+    const uint32_t hi = grf::fused_symbol_in<8 * H + (i)>(c, __umul24(bin, q.block_pitch), q);        \
+    bits[i] = hi | rr.field<8 * H + (i)>();                                                           \
   }
     GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
-    GRF_STEP(8) GRF_STEP(9) GRF_STEP(10) GRF_STEP(11) GRF_STEP(12) GRF_STEP(13) GRF_STEP(14) GRF_STEP(15)
 #undef GRF_STEP
-    c.end_group();
+    if (H == 1) c.end_group();
 #pragma unroll
-    for (int k = 0; k < 8; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
+    for (int k = 0; k < 4; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
+  }
+  __device__ __forceinline__ void decode16(uint32_t t, uint32_t S, const grf::FusedParams &q, uint32_t (&pair)[8]) {
+    begin16(t, S);
+    half<0>(q, reinterpret_cast<uint32_t (&)[4]>(pair[0]));
+    half<1>(q, reinterpret_cast<uint32_t (&)[4]>(pair[4]));
   }
 
   __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
@@ -232,13 +240,13 @@ int grf_ppcx_gemv(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, c
 }
 
 int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const uint16_t *x,
-                  uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
-                  void *hip_stream) {
+                  uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
+                  size_t workspace_bytes, int32_t *error, void *hip_stream) {
   if (!x || !y || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemm: null argument");
   grf_bctx_fused f;
   if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_gemm", f)) return rc;
-  return grf::launch_gemm<PpcxWalk>("grf_ppcx_gemm", f, *tiling, x, ldx, m_rows, y, ldy, bias, error,
-                                    (hipStream_t)hip_stream);
+  return grf::launch_gemm<PpcxWalk>("grf_ppcx_gemm", f, *tiling, x, ldx, m_rows, y, ldy, bias, workspace,
+                                    workspace_bytes, error, (hipStream_t)hip_stream);
 }
 
 }  // extern "C"

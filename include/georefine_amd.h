@@ -214,11 +214,19 @@ int grf_bctx_fused_decode(const grf_bctx_fused *frame, const grf_fused_tiling *t
 /* Fused decode-GEMM on the matrix cores for any number of activation rows; same operand
  * meaning as grf_bctx_gemv.  Batch-invariant in the sense of GS/bi_csrc/bi_gemm.cuh:1-17:
  * with one tiling, row m of y is a function of row m of x and of W only.  x must be
- * 8-byte aligned with ldx a multiple of 4.  More than 128 rows run as several launches. */
+ * 8-byte aligned with ldx a multiple of 4.  More than 64 rows run as several launches.
+ *
+ * A tiling for this function has threads = 64 * ceil(rows_per_tile / 16) *
+ * ceil(lanes_per_row / 4): a wave walks four lane-segments of 16 rows and feeds the words
+ * it decodes to the matrix cores from its registers.  workspace: device memory, 16-byte
+ * aligned, at least grf_gemm_workspace_bytes(cols, m_rows) bytes; each launch first writes
+ * its activation rows there in operand order (a copy of x: cols * 32 bytes per 16 rows),
+ * so calls that share a workspace must be ordered on one stream. */
 int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, const uint16_t *x, uint32_t ldx,
-                  uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
-                  void *hip_stream);
-uint32_t grf_bctx_gemm_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint32_t m_rows);
+                  uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
+                  size_t workspace_bytes, int32_t *error, void *hip_stream);
+size_t grf_gemm_workspace_bytes(uint32_t cols, uint32_t m_rows);
+uint32_t grf_bctx_gemm_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling);
 
 /* LDS bytes a launch needs for the given m_rows (0 for the store sink). */
 uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint32_t m_rows);
@@ -270,8 +278,8 @@ int grf_ppcx_gemv(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, c
                   uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
                   void *hip_stream);
 int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const uint16_t *x,
-                  uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
-                  void *hip_stream);
+                  uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
+                  size_t workspace_bytes, int32_t *error, void *hip_stream);
 
 const char *grf_last_error(void);
 int grf_abi_version(void);

@@ -93,6 +93,55 @@ def test_attention_matrices_gemm_rows_do_not_depend_on_batch(name, shape):
     _check_products(t, x, (1, 8, 32, 64, 128), lambda v: t.linear(v, check=True, batch_invariant=True))
 
 
+def test_whole_stack_resident_one_pass_at_batch_64():
+    """64 layers x (q, k, v, o, gate, up, down) resident at once, one pass through every coded
+    linear at batch 64.  One layer is encoded; the other 63 are device copies with buffers of
+    their own, so the pass runs 448 launches over about 30 GB of coded weights.  Every copy
+    must give the first layer's rows bit for bit, and the first layer's rows agree with the
+    dense product of its decoded weights."""
+    import torch
+    from concurrent.futures import ThreadPoolExecutor
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd.bitexact_context_gpu import HipContextTensor
+    shapes = {"q": (6144, 5120), "k": (1024, 5120), "v": (1024, 5120), "o": (5120, 6144),
+              "gate": (17408, 5120), "up": (17408, 5120), "down": (5120, 17408)}
+
+    def coded(item):
+        j, (name, shape) = item
+        return name, codec.encode(weight_like(np.random.default_rng(4000 + j), *shape))
+
+    with ThreadPoolExecutor(max_workers=7) as pool:
+        frames = dict(pool.map(coded, enumerate(shapes.items())))
+    first = {name: HipContextTensor(frames[name], stride=1024, device="cuda:0") for name in shapes}
+    assert all(t.fused is not None for t in first.values())
+    layers = [first] + [{name: t.clone() for name, t in first.items()} for _ in range(63)]
+    dense_bytes = 64 * sum(2 * r * c for r, c in shapes.values())
+    resident = sum(t.resident_bytes for layer in layers for t in layer.values())
+    assert dense_bytes == 43_620_761_600 and 0.6 * dense_bytes < resident < 0.75 * dense_bytes
+    assert torch.cuda.memory_allocated() >= resident - 64 * 7 * 4096
+    rng = np.random.default_rng(11)
+    x = {k: torch.from_numpy(bf16_words(rng.normal(0, 1, size=(64, k)))).view(torch.bfloat16).cuda()
+         for k in (5120, 6144, 17408)}
+    outs = [{name: t.linear(x[shapes[name][1]], check=False) for name, t in layer.items()} for layer in layers]
+    torch.cuda.synchronize()
+    for layer in layers:
+        for t in layer.values():
+            assert t.error.item() == 0
+    for name, shape in shapes.items():
+        w = first[name].decode(check=True).float()
+        ref = torch.nn.functional.linear(x[shape[1]].float(), w)
+        scale = torch.nn.functional.linear(x[shape[1]].float().abs(), w.abs())
+        assert _close(outs[0][name], ref, scale), name
+        for i in range(1, 64):
+            assert torch.equal(outs[i][name].view(torch.uint16), outs[0][name].view(torch.uint16)), (i, name)
+    # a copy stands on its own: it decodes to the source words after the first layer is gone
+    keep = layers[63]["k"]
+    want = first["k"].source_sha256
+    del layers, first, outs
+    torch.cuda.empty_cache()
+    assert _digest(keep.decode(check=True)) == want
+
+
 def test_predictive_frame_full_size_decode_and_batch_96():
     """A 5120 x 17408 target coded against a near-identical reference; the product takes
     16 users x (5 speculative + 1) = 96 rows."""

@@ -71,17 +71,21 @@ def test_gemv_matches_float64_and_is_m_invariant(oracle, shape):
     x = torch.from_numpy(xw).view(torch.bfloat16).cuda()
     ref = words_to_float(xw).astype(np.float64) @ w64.T
     scale = np.abs(words_to_float(xw).astype(np.float64)) @ np.abs(w64).T
-    y8 = t.linear(x, check=True)
+    y8 = t.gemv(x, check=True)
     got = words_to_float(y8.view(torch.uint16).cpu().numpy()).astype(np.float64)
     # relative to the magnitude of the terms: 1e-2 is the stated bar, BF16 rounding is ~4e-3 of |y|
     assert np.all(np.abs(got - ref) <= 1e-2 * np.maximum(np.abs(ref), 1e-3 * scale) + 1e-30)
     dense = torch.nn.functional.linear(x.float(), t.decode().float()).double().cpu().numpy()
     assert np.all(np.abs(got - dense) <= 1e-2 * np.maximum(np.abs(dense), 1e-3 * scale) + 1e-30)
     for m in (1, 2, 3, 5, 8):
-        ym = t.linear(x[:m], check=True)
+        ym = t.gemv(x[:m], check=True)
         assert torch.equal(ym.view(torch.uint16), y8[:m].view(torch.uint16)), f"M={m} rows differ from M=8"
-    y1 = torch.cat([t.linear(x[i:i + 1]) for i in range(8)])
+    y1 = torch.cat([t.linear(x[i:i + 1]) for i in range(8)])  # linear() gives single rows to the GEMV
     assert torch.equal(y1.view(torch.uint16), y8.view(torch.uint16))
+    # from three rows on linear() takes the matrix-core kernel: same product, its own rounding
+    y_mm = words_to_float(t.linear(x, check=True).view(torch.uint16).cpu().numpy()).astype(np.float64)
+    assert np.all(np.abs(y_mm - ref) <= 1e-2 * np.maximum(np.abs(ref), 1e-3 * scale) + 1e-30)
+    assert torch.equal(t.linear(x).view(torch.uint16), t.gemm(x).view(torch.uint16))
 
 
 def test_gemv_bias_and_batched_input(oracle):
