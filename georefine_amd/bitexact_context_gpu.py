@@ -117,7 +117,7 @@ class HipContextTensor:
     """A BCTX-coded BF16 matrix resident on one MI355X."""
 
     GEMV_UP_TO = 2    # activation rows linear() gives to the vector-ALU kernel
-    DENSE_ABOVE = 64  # activation rows above which linear() decodes to a dense transient
+    DENSE_ABOVE = 128  # activation rows above which linear() decodes to a dense transient
 
     def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None):
         import torch
@@ -250,7 +250,8 @@ class HipContextTensor:
             count = blocks.numel()
             ids = blocks.data_ptr()
         result = torch.empty(count * self.stride, device=self.device, dtype=torch.uint16)
-        self.error.zero_()
+        if check:  # between checks the word keeps what earlier launches reported
+            self.error.zero_()
         with torch.cuda.device(self.device):
             stream = torch.cuda.current_stream(self.device).cuda_stream
             status = self._lib.grf_bctx_decode(ctypes.byref(self._frame), ids, count, result.data_ptr(),
@@ -283,7 +284,8 @@ class HipContextTensor:
         if self.fused is None or general:
             return self._decode_blocks(check=check)[:self.n].reshape(self.shape)
         out = torch.empty(self.n, device=self.device, dtype=torch.uint16)
-        self.error.zero_()
+        if check:  # between checks the word keeps what earlier launches reported
+            self.error.zero_()
         self._launch(self._lib.grf_bctx_fused_decode, ctypes.byref(self.fused), ctypes.byref(self._tiling(0)[0]),
                      out.data_ptr(), self.error.data_ptr())
         self._check(check)
@@ -320,7 +322,8 @@ class HipContextTensor:
         lead = x.shape[:-1]
         x2, bias, y = self._prepare_activations(x, bias, 4)
         if x2.shape[0]:
-            self.error.zero_()
+            if check:  # between checks the word keeps what earlier launches reported
+                self.error.zero_()
             extra = ()
             if workspace:  # transient: the activations in the matrix cores' operand order
                 size = self._lib.grf_gemm_workspace_bytes(self.shape[1], x2.shape[0])
@@ -352,10 +355,10 @@ class HipContextTensor:
     def linear(self, x, bias=None, *, check=False, batch_invariant=False):
         """y = x @ W.T (+ bias) with W decoded inside the kernel; x is BF16 [..., K].
 
-        One or two activation rows run the fused decode-GEMV, up to 64 the fused decode-GEMM
+        One or two activation rows run the fused decode-GEMV, up to 128 the fused decode-GEMM
         (one launch; from three rows on it is faster than the GEMV, whose cost grows with every
         row); above that a fused decode to a dense transient followed by the library matmul is
-        faster (measured crossover between 64 and 96 rows).  ``batch_invariant=True`` sends
+        faster (a second GEMM launch would decode the matrix again).  ``batch_invariant=True`` sends
         every row count through the GEMM so that a row's output never depends on the batch
         it arrives in.  Frames the fused kernels cannot take are decoded on the device and
         multiplied densely.  ``check=True`` reads the error word back (a host sync)."""

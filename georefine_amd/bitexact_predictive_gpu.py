@@ -133,7 +133,7 @@ class HipPredictiveTensor:
     """A PPCX-coded BF16 matrix resident on one MI355X; decoding needs the reference matrix."""
 
     GEMV_UP_TO = 1    # activation rows linear() gives to the vector-ALU kernel
-    DENSE_ABOVE = 64  # activation rows above which linear() decodes to a dense transient
+    DENSE_ABOVE = 128  # activation rows above which linear() decodes to a dense transient
 
     def __init__(self, frame, reference_uint16_numpy, stride=1024, device="cuda:0", *, fused=True,
                  fused_segment=None):
@@ -254,7 +254,7 @@ class HipPredictiveTensor:
 
     def linear(self, reference_bf16_device, x, bias=None, *, check=False, batch_invariant=False):
         """y = x W^T + bias with W decoded on the fly against the reference: the fused GEMV for
-        one activation row, the fused GEMM (matrix cores, one launch) for up to 64; above that
+        one activation row, the fused GEMM (matrix cores, one launch) for up to 128; above that
         the fused decode to a dense transient plus the library matmul is faster, unless
         ``batch_invariant`` asks for the fused GEMM throughout, whose rows do not depend on
         the batch.  Frames the tile walker cannot take are decoded and multiplied densely."""
@@ -293,7 +293,8 @@ class HipPredictiveTensor:
             bias = bias.to(device=self.device, dtype=torch.bfloat16).contiguous()
         y = torch.empty((m, self.shape[0]), device=self.device, dtype=torch.bfloat16)
         if m:
-            self.error.zero_()
+            if check:  # between checks the word keeps what earlier launches reported
+                self.error.zero_()
             with torch.cuda.device(self.device):
                 bins, status = self._bins(ref)
                 if not status:
@@ -330,7 +331,8 @@ class HipPredictiveTensor:
         ref = self._reference(reference_bf16_device)
         if self.fused is not None and not general:
             out = torch.empty(self.shape, device=self.device, dtype=torch.uint16)
-            self.error.zero_()
+            if check:  # between checks the word keeps what earlier launches reported
+                self.error.zero_()
             with torch.cuda.device(self.device):
                 bins, status = self._bins(ref)
                 if not status:
@@ -342,7 +344,8 @@ class HipPredictiveTensor:
             return out.view(torch.bfloat16)
         count = (self.n + self.stride - 1) // self.stride
         out = torch.empty(count * self.stride, device=self.device, dtype=torch.uint16)
-        self.error.zero_()
+        if check:  # between checks the word keeps what earlier launches reported
+            self.error.zero_()
         with torch.cuda.device(self.device):
             status = self._lib.grf_ppcx_decode(ctypes.byref(self._frame), ref.data_ptr(), out.data_ptr(),
                                                self.error.data_ptr(),

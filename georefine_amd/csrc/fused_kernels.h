@@ -12,13 +12,14 @@
 // to BF16 once.
 //
 // GEMM, batch invariance (the contract of GS/bi_csrc/bi_gemm.cuh:1-17): output element
-// (m, n) is one accumulator fed by a fixed sequence of MFMA operations -- slabs in
-// increasing order, inside a slab the 16-column groups in increasing order, inside a
-// group the P lane-segments p = 0..P-1 -- whose A operand row is x[m] and whose B
+// (m, n) is the sum, in quad order, of one fp32 accumulator per quad of lane-segments;
+// each accumulator is fed by a fixed sequence of MFMA operations -- slabs in increasing
+// order, inside a slab the 8-column half groups in increasing order, one operation per
+// half group over the quad's four segments -- whose A operand row is x[m] and whose B
 // operand column is W[n].  Neither the number of activation rows, nor the tile a row
 // sits in, nor what the other rows hold enters that sequence: every M runs the same
-// kernel (M < 16 is padded with zero rows), and more than 128 rows are cut into
-// launches of 128, which only repeats the same per-row arithmetic.
+// tiling (rows up to the next multiple of 16 are zero), and more than 128 rows are cut
+// into launches of 128, which only repeats the same per-row arithmetic.
 #pragma once
 #include <hip/hip_runtime.h>
 
@@ -215,8 +216,8 @@ int launch_gemv(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-constexpr uint32_t kMaxRowsPerLaunch = 64;  // four 16-row activation tiles per launch
-constexpr uint32_t kMaxTiles = kMaxRowsPerLaunch / 16;
+constexpr uint32_t kMaxRowsPerLaunch = 128;  // eight 16-row activation tiles per launch
+constexpr uint32_t kSumTiles = 4;            // tiles whose partial sums pass through LDS at a time
 
 // Workgroup shape of the GEMM kernel for a tiling: row blocks x quads of lane-segments.
 struct GemmShape {
@@ -237,7 +238,7 @@ struct GemmLdsLayout {
     block_pitch = grf::fused_table_bytes(f) + (1u << f.lognb);
     stream = grf::align_up(f.nc * block_pitch, 16);
     total = grf::align_up(stream + g.rows_per_tile * g.piece_cap, 16);
-    const uint32_t sums = GemmShape(g).threads / 64 * kMaxTiles * 1024;
+    const uint32_t sums = GemmShape(g).threads / 64 * kSumTiles * 1024;
     if (total < sums) total = sums;
   }
 };
@@ -284,11 +285,9 @@ __device__ __forceinline__ void gemm_contract(float4v (&acc)[MT], const uint4 (&
 
 // MT: 16-row activation tiles of this launch (m_rows <= 16 * MT, xp packed with m_pad = 16 * MT)
 template <class Walk, int MT>
-__global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_gemm_kernel(grf_bctx_fused f, grf_fused_tiling g,
-                                                                            const uint4 *xp, uint32_t m_rows,
-                                                                            uint16_t *y, uint32_t ldy,
-                                                                            const uint16_t *bias, int32_t *error) {
-  extern __shared__ __align__(16) uint8_t lds[];
+__device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fused &f, const grf_fused_tiling &g,
+                                                const uint4 *xp, uint32_t m_rows, uint16_t *y, uint32_t ldy,
+                                                const uint16_t *bias, int32_t *error) {
   const GemmLdsLayout L(f, g);
   const GemmShape shape(g);
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
@@ -352,28 +351,53 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_
     if (active && !w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
   }
 
-  // partial sums of every wave -> LDS, then each output element adds its quads in order
-  __syncthreads();
+  // partial sums of every wave -> LDS, then each output element adds its quads in order;
+  // four activation tiles at a time, which is what the LDS allocation is sized for
+  constexpr int CT = MT < (int)kSumTiles ? MT : (int)kSumTiles;
   float *sums = reinterpret_cast<float *>(lds);
 #pragma unroll
-  for (int j = 0; j < MT; ++j)
+  for (int c0 = 0; c0 < MT; c0 += CT) {
+    __syncthreads();  // tables and stream bytes (or the previous chunk's sums) are done with
 #pragma unroll
-    for (int v = 0; v < 4; ++v) sums[((wave * MT + j) * 4 + v) * 64 + lane] = acc[j][v];
-  __syncthreads();
-  const uint32_t per_block = MT * 256;  // values of one row block: [tile j][v][lane]
-  for (uint32_t i = tid; i < shape.row_blocks * per_block; i += nthreads) {
-    const uint32_t blk = i / per_block, within = i % per_block;
-    const uint32_t j = within / 256, v = (within / 64) % 4, ln = within % 64;
-    const uint32_t n_local = blk * 16 + ln % 16, m = j * 16 + (ln / 16) * 4 + v;
-    const uint32_t orow = n_local < R ? g.tile_rows[tile * R + n_local] : grf::kNoRow;
-    if (orow == grf::kNoRow || m >= m_rows) continue;
-    // wave index of (quad, block) is quad * row_blocks + block
-    float sum = sums[(blk * MT) * 256 + within];
-    for (uint32_t qd = 1; qd < shape.quads; ++qd) sum += sums[((qd * shape.row_blocks + blk) * MT) * 256 + within];
-    if (bias) sum += __uint_as_float((uint32_t)bias[orow] << 16);
-    y[(size_t)m * ldy + orow] = round_bf16(sum);
+    for (int jj = 0; jj < CT; ++jj)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) sums[((wave * CT + jj) * 4 + v) * 64 + lane] = acc[c0 + jj][v];
+    __syncthreads();
+    const uint32_t per_block = CT * 256;  // values of one row block: [tile jj][v][lane]
+    for (uint32_t i = tid; i < shape.row_blocks * per_block; i += nthreads) {
+      const uint32_t blk = i / per_block, within = i % per_block;
+      const uint32_t jj = within / 256, v = (within / 64) % 4, ln = within % 64;
+      const uint32_t n_local = blk * 16 + ln % 16, m = (c0 + jj) * 16 + (ln / 16) * 4 + v;
+      const uint32_t orow = n_local < R ? g.tile_rows[tile * R + n_local] : grf::kNoRow;
+      if (orow == grf::kNoRow || m >= m_rows) continue;
+      // wave index of (quad, block) is quad * row_blocks + block
+      float sum = sums[(blk * CT) * 256 + within];
+      for (uint32_t qd = 1; qd < shape.quads; ++qd) sum += sums[((qd * shape.row_blocks + blk) * CT) * 256 + within];
+      if (bias) sum += __uint_as_float((uint32_t)bias[orow] << 16);
+      y[(size_t)m * ldy + orow] = round_bf16(sum);
+    }
   }
   if (bad) atomicOr(error, (int)bad);
+}
+
+// Up to four activation tiles: 80 vector registers, six waves per SIMD.
+template <class Walk, int MT>
+__global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_gemm_kernel(
+    grf_bctx_fused f, grf_fused_tiling g, const uint4 *xp, uint32_t m_rows, uint16_t *y, uint32_t ldy,
+    const uint16_t *bias, int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  fused_gemm_body<Walk, MT>(lds, f, g, xp, m_rows, y, ldy, bias, error);
+}
+
+// Eight activation tiles: the accumulators and operands alone take 64 registers, so fewer
+// waves are resident; still cheaper than decoding the matrix twice.
+template <class Walk, int MT>
+__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_wide_kernel(grf_bctx_fused f, grf_fused_tiling g,
+                                                                                 const uint4 *xp, uint32_t m_rows,
+                                                                                 uint16_t *y, uint32_t ldy,
+                                                                                 const uint16_t *bias, int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  fused_gemm_body<Walk, MT>(lds, f, g, xp, m_rows, y, ldy, bias, error);
 }
 
 template <class Walk, int MT>
@@ -385,7 +409,10 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
   const uint32_t pack_threads = (chunks + 7) / 8 * 8 * m_pad;
   hipLaunchKernelGGL(pack_activations_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, x, ldx, m_rows, m_pad,
                      chunks, xp);
-  auto kernel = fused_gemm_kernel<Walk, MT>;
+  void (*kernel)(grf_bctx_fused, grf_fused_tiling, const uint4 *, uint32_t, uint16_t *, uint32_t, const uint16_t *,
+                 int32_t *);
+  if constexpr (MT <= 4) kernel = fused_gemm_kernel<Walk, MT>;
+  else kernel = fused_gemm_wide_kernel<Walk, MT>;
   if (L.total > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
@@ -400,11 +427,11 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
 // bytes of the packed copy of the activations one launch needs
 inline size_t gemm_workspace_bytes(uint32_t cols, uint32_t m_rows) {
   const uint32_t m = m_rows > kMaxRowsPerLaunch ? kMaxRowsPerLaunch : m_rows;
-  const uint32_t tiles = m <= 16 ? 1 : m <= 32 ? 2 : kMaxTiles;
+  const uint32_t tiles = m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8;
   return (size_t)(cols / 8) * tiles * 16 * 16;
 }
 
-// y = x W^T (+ bias) for any number of activation rows, 64 per launch.  `workspace` holds
+// y = x W^T (+ bias) for any number of activation rows, 128 per launch.  `workspace` holds
 // the packed activations of one launch; launches follow one another on the stream.
 template <class Walk>
 int launch_gemm(const char *who, const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx,
@@ -427,7 +454,8 @@ int launch_gemm(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
     int rc;
     if (m <= 16) rc = launch_gemm_rows<Walk, 1>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
     else if (m <= 32) rc = launch_gemm_rows<Walk, 2>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
-    else rc = launch_gemm_rows<Walk, 4>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
+    else if (m <= 64) rc = launch_gemm_rows<Walk, 4>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
+    else rc = launch_gemm_rows<Walk, 8>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
     if (rc) return rc;
   }
   return GRF_OK;

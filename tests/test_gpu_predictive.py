@@ -184,13 +184,13 @@ def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle,
         assert torch.equal(t.gemv(ref_dev, x[:m], bias).view(torch.uint16), y8[:m].view(torch.uint16))
     assert torch.equal(t.linear(ref_dev, x[:1], bias).view(torch.uint16), y8[:1].view(torch.uint16))  # one row: the GEMV
     y40 = t.linear(ref_dev, x, bias, check=True, batch_invariant=True)  # the matrix-core kernel
-    assert torch.equal(t.linear(ref_dev, x, bias, check=True).view(torch.uint16), y40.view(torch.uint16))  # default to 64 rows
+    assert torch.equal(t.linear(ref_dev, x, bias, check=True).view(torch.uint16), y40.view(torch.uint16))  # default to 128 rows
     assert close(y40, 40)
-    many = torch.cat([x, x, x[:10]])                                     # 90 rows: decode + dense by default
+    many = torch.cat([x, x, x, x[:10]])                                  # 130 rows: decode + dense by default
     assert close(t.linear(ref_dev, many, bias, check=True)[:40], 40)
-    y90 = t.linear(ref_dev, many, bias, batch_invariant=True)            # two launches of the GEMM
-    assert torch.equal(y90[:40].view(torch.uint16), y40.view(torch.uint16))
-    assert torch.equal(y90[80:].view(torch.uint16), y40[:10].view(torch.uint16))
+    y130 = t.linear(ref_dev, many, bias, batch_invariant=True)           # two launches of the GEMM
+    assert torch.equal(y130[:40].view(torch.uint16), y40.view(torch.uint16))
+    assert torch.equal(y130[120:].view(torch.uint16), y40[:10].view(torch.uint16))
     for m in (1, 8, 17, 32):
         ym = t.linear(ref_dev, x[:m], bias, batch_invariant=True)
         assert torch.equal(ym.view(torch.uint16), y40[:m].view(torch.uint16)), m
