@@ -11,6 +11,10 @@ every step streams its compressed bytes from HBM.
 Prints ONE JSON line: metric = compressed bytes consumed per second (GB/s), with
 the achieved fraction of the 8 TB/s HBM roofline for the dominant kernel and a
 CPU baseline (the CPU oracle's decode + matvec on the host cores).
+
+After the warm-up, K eager steps give the per-launch durations (HIP events on the
+launch stream); the K timed steps are then replays of one HIP graph of a step
+(--no-graph times the eager steps instead).
 """
 from __future__ import annotations
 
@@ -190,6 +194,23 @@ def run_stack(args):
                     probes[name].append((a, b))
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
+    launch = "eager"
+    if args.graph:
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            graph.replay()
+            torch.cuda.synchronize()
+        except Exception as exc:
+            log(f"graph capture failed ({exc}); reporting the eager steps")
+        else:
+            wall0 = time.perf_counter()
+            for _ in range(args.steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - wall0
+            launch = "hip graph replay"
     for layer in layers:
         for name, t in layer.items():
             if t.error.item():
@@ -211,7 +232,7 @@ def run_stack(args):
         "config": {"workload": f"whole stack resident: {args.layers} layers x (q 5120->6144, k/v 5120->1024, o 6144->5120, "
                                f"gate/up 5120->17408, down 17408->5120), one pass through every coded linear at batch {m}",
                    "batch": m, "layers": args.layers, "distinct_layers": args.distinct_layers,
-                   "linears": args.layers * len(LAYER)},
+                   "linears": args.layers * len(LAYER), "launch": launch},
         "dense_bf16_bytes": dense, "frame_bytes": frame_bytes, "resident_device_bytes": resident,
         "algorithmic_bytes_per_step": step_bytes,
         "effective_bf16_GBps": round(dense / (ms_per_step * 1e-3) / 1e9, 2),
@@ -232,6 +253,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1, help="activation rows; 1..8 run the fused GEMV (the headline figure is batch 1), more the fused GEMM")
     ap.add_argument("--segment", type=int, default=0, help="fused segment length (0 = automatic)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", dest="graph", action="store_false",
+                    help="time K eager steps; by default the K timed steps are replays of one captured HIP graph "
+                         "of a step (per-kernel durations always come from K eager steps before it)")
     ap.add_argument("--only", default="", help="comma list of gate,up,down (profiling aid)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB read + 128 MiB write elementwise kernel three times, so that a "
@@ -309,6 +333,25 @@ def main():
             ends[s][j].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
+    launch = "eager"
+    if args.graph:
+        # the same step captured once and replayed: the launches of a step are submitted together,
+        # which takes the host's per-launch latency out of the gaps between kernels
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            graph.replay()
+            torch.cuda.synchronize()
+        except Exception as exc:  # keep the eager figure
+            log(f"graph capture failed ({exc}); reporting the eager steps")
+        else:
+            wall0 = time.perf_counter()
+            for _ in range(args.steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - wall0
+            launch = "hip graph replay"
     for name in names:
         if tensors[name].error.item():
             sys.exit(f"bench.py: decoder error word set for {name}")
@@ -354,7 +397,7 @@ def main():
         "config": {"workload": "fused decode-" + ("GEMV" if m <= 8 else "GEMM") + ", batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
                                "BCTX (16,4) frames, residuals resident in packed 6-bit form" % m,
                    "batch": m, "matrices": names,
-                   "segment": tensors[names[0]].fused_plan["seg_len"]},
+                   "segment": tensors[names[0]].fused_plan["seg_len"], "launch": launch},
         "effective_bf16_GBps": round(eff_bf16, 2),
         "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3),
         "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),

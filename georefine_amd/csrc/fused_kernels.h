@@ -23,6 +23,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <string>
 
 #include "fused_device.h"
@@ -30,6 +31,22 @@
 namespace grf {
 int set_error(int code, const std::string &what);                                          // decode_general.hip
 int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who);  // fused_gemv.hip
+
+// A kernel may ask for more than 64 KiB of dynamic LDS only after its limit has been raised;
+// done once per kernel and device (not per launch: it is a driver call, and a launch that
+// is being captured into a graph should consist of the launch alone).
+template <auto Kernel>
+int allow_full_lds() {
+  static std::atomic<uint64_t> done{0};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+  if (dev >= 0 && ((done.load(std::memory_order_relaxed) >> dev) & 1u)) return GRF_OK;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                     160 * 1024);
+  if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("LDS attribute: ") + hipGetErrorString(e));
+  if (dev >= 0) done.fetch_or(1ull << dev, std::memory_order_relaxed);
+  return GRF_OK;
+}
 
 // ---------------------------------------------------------------- GEMV and store sinks
 
@@ -167,12 +184,9 @@ int launch_walk(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16
                 uint32_t ldy, const uint16_t *bias, uint16_t *out, int32_t *error, hipStream_t s) {
   const FusedLdsLayout L(f, g, STORE ? 0 : M);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
-  auto kernel = fused_walk_kernel<Walk, M, STORE>;
-  if (L.total > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
-    if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("LDS attribute: ") + hipGetErrorString(e));
-  }
+  constexpr auto kernel = &fused_walk_kernel<Walk, M, STORE>;
+  if (L.total > 64 * 1024)
+    if (int rc = allow_full_lds<kernel>()) return rc;
   hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, x, ldx, y, ldy, bias, out, error);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
@@ -409,15 +423,12 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
   const uint32_t pack_threads = (chunks + 7) / 8 * 8 * m_pad;
   hipLaunchKernelGGL(pack_activations_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, x, ldx, m_rows, m_pad,
                      chunks, xp);
-  void (*kernel)(grf_bctx_fused, grf_fused_tiling, const uint4 *, uint32_t, uint16_t *, uint32_t, const uint16_t *,
-                 int32_t *);
-  if constexpr (MT <= 4) kernel = fused_gemm_kernel<Walk, MT>;
-  else kernel = fused_gemm_wide_kernel<Walk, MT>;
-  if (L.total > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)L.total);
-    if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("LDS attribute: ") + hipGetErrorString(e));
-  }
+  constexpr auto kernel = [] {
+    if constexpr (MT <= 4) return &fused_gemm_kernel<Walk, MT>;
+    else return &fused_gemm_wide_kernel<Walk, MT>;
+  }();
+  if (L.total > 64 * 1024)
+    if (int rc = allow_full_lds<kernel>()) return rc;
   hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, xp, m_rows, y, ldy, bias, error);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused GEMM: ") + hipGetErrorString(e));
