@@ -77,38 +77,133 @@ def algorithmic_bytes(t, m):
     return dict(total=payload + index + tables + labels + io, payload=payload, index=index, tables=tables)
 
 
+def host_description():
+    model = ""
+    try:
+        for line in Path("/proc/cpuinfo").read_text().splitlines():
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    return {"cpu": model, "logical_cpus": os.cpu_count(), "oracle_flags": "gcc -O3 (oracle/Makefile)"}
+
+
+def measured_copy_gbps(torch):
+    """Device-to-device copy of 1 GiB (read + write counted), the achievable HBM rate on this
+    box next to the 8 TB/s nameplate."""
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(5):
+        dst.copy_(src)
+    b.record()
+    torch.cuda.synchronize()
+    return 5 * 2 * src.numel() / (a.elapsed_time(b) * 1e-3) / 1e9
+
+
+def reference_core():
+    """The reference's own C++ coder, compiled from its sources into oracle/_ref by the oracle's
+    Makefile; None where that build is absent."""
+    import ctypes
+    path = ROOT / "oracle" / "_ref" / "libref_context.so"
+    if not path.exists():
+        return None
+    L = ctypes.CDLL(str(path))
+    U8P, U16P, U32P = (ctypes.POINTER(t) for t in (ctypes.c_uint8, ctypes.c_uint16, ctypes.c_uint32))
+    sz, u32, u64 = ctypes.c_size_t, ctypes.c_uint32, ctypes.c_uint64
+    L.bcx_decode.argtypes = [U8P, sz, u64, u32, u32, U8P, U8P, u32, u32, u32, U16P, U32P, U16P]
+    L.bcx_unpack6.argtypes = [U8P, sz, u64, U16P]
+    L.bcx_decode.restype = L.bcx_unpack6.restype = ctypes.c_int
+    return L
+
+
+def reference_decode(L, orc, frame):
+    """A frame decoded by the reference's bcx_decode / bcx_unpack6 (full 65536-slot lookup);
+    the container around them (header, inflate, digests) is read by the oracle's parser."""
+    import ctypes
+    import hashlib
+    s = orc.bctx_sections(frame)
+    if s["mode"] == 1:
+        return s["raw"]
+    rows, cols = s["shape"]
+    n = rows * cols
+    p = lambda a, t: a.ctypes.data_as(ctypes.POINTER(t))
+    u8, u16, u32 = ctypes.c_uint8, ctypes.c_uint16, ctypes.c_uint32
+
+    def entropy(stream, freq, kind, main):
+        data = np.frombuffer(stream, dtype=np.uint8)
+        out = np.empty(n, dtype=np.uint16)
+        freq = np.ascontiguousarray(freq, dtype=np.uint32).ravel()
+        rc = L.bcx_decode(p(data, u8), len(stream), n, rows, cols, p(s["rc"], u8), p(s["cc"], u8), s["nr"], s["nc"],
+                          kind, p(main, u16) if main is not None else None, p(freq, u32), p(out, u16))
+        if rc:
+            raise RuntimeError(f"reference bcx_decode failed ({rc})")
+        return out
+
+    main = entropy(s["main_stream"], s["main_freq"], 0, None)
+    if s["mode"] == 128:
+        residual = entropy(s["res_stream"], s["res_freq"], 1, main)
+    else:
+        raw = np.frombuffer(s["res_stream"], dtype=np.uint8)
+        residual = np.empty(n, dtype=np.uint16)
+        if L.bcx_unpack6(p(raw, u8), len(raw), n, p(residual, u16)):
+            raise RuntimeError("reference bcx_unpack6 failed")
+    out = np.ascontiguousarray(orc.join_words(main, residual).reshape(rows, cols))
+    if hashlib.sha256(out.tobytes()).digest() != s["digest"]:
+        raise RuntimeError("reference decode does not reproduce the frame's digest")
+    return out
+
+
 def cpu_baseline(frames, words_of, x_words, min_seconds=10.0, max_frames=12):
-    """The CPU oracle (full 65536-slot lookup, one thread, as the reference decodes a
-    frame) on whole frames of the workload, each followed by an fp32 matvec on the host;
-    frames are taken in turn until min_seconds of work are done."""
+    """CPU decode + fp32 matvec of whole frames of the workload, one thread, as the reference
+    decodes a frame; frames are taken in turn until min_seconds of work are done.  Timed with
+    the reference's own compiled coder where oracle/_ref holds it (kind "reference"), and
+    with the CPU oracle (kind "port"); the reference figure is the headline when present."""
     from oracle import codec_oracle as orc
-    coded = produced = done = 0
-    checksum = 0.0
     names = list(frames)
-    t0 = time.perf_counter()
-    while done < max_frames and (done == 0 or time.perf_counter() - t0 < min_seconds):
-        name = names[done % len(names)]
-        dec = orc.bctx_decode(frames[name])
-        wf = (dec.astype(np.uint32) << 16).view(np.float32)
-        xf = (x_words[dec.shape[1]][0].astype(np.uint32) << 16).view(np.float32)
-        checksum += float(np.sum(wf @ xf))
-        assert np.array_equal(dec, words_of[name]), "CPU oracle decode is not bit-exact"
-        coded += len(frames[name])
-        produced += dec.nbytes
-        done += 1
-        del dec, wf
-    dt = time.perf_counter() - t0
-    result = dict(value=round(coded / dt / 1e9, 4), unit="GB/s", cores=1, kind="port",
-                  sample=f"{done} whole frames in turn from {', '.join(names)} ({coded} coded bytes): frame parse + "
-                         f"sha256 + full-LUT rANS decode of both streams + bit-exact check + fp32 matvec in {dt:.1f}s "
-                         f"({produced / dt / 1e6:.1f} MB/s of BF16 produced)",
-                  checksum=checksum)
+
+    def timed(decode, what):
+        coded = produced = done = 0
+        checksum = 0.0
+        t0 = time.perf_counter()
+        while done < max_frames and (done == 0 or time.perf_counter() - t0 < min_seconds):
+            name = names[done % len(names)]
+            dec = decode(frames[name])
+            wf = (dec.astype(np.uint32) << 16).view(np.float32)
+            xf = (x_words[dec.shape[1]][0].astype(np.uint32) << 16).view(np.float32)
+            checksum += float(np.sum(wf @ xf))
+            assert np.array_equal(dec, words_of[name]), "CPU decode is not bit-exact"
+            coded += len(frames[name])
+            produced += dec.nbytes
+            done += 1
+            del dec, wf
+        dt = time.perf_counter() - t0
+        return dict(value=round(coded / dt / 1e9, 4), unit="GB/s", cores=1,
+                    sample=f"{done} whole frames in turn from {', '.join(names)} ({coded} coded bytes): frame parse + "
+                           f"sha256 + {what} + bit-exact check + fp32 matvec in {dt:.1f}s "
+                           f"({produced / dt / 1e6:.1f} MB/s of BF16 produced)",
+                    checksum=checksum)
+
+    port = dict(timed(orc.bctx_decode, "the oracle's full-LUT rANS decode of the main stream and 6-bit unpack"), kind="port")
+    core = reference_core()
+    if core is not None:
+        result = dict(timed(lambda f: reference_decode(core, orc, f),
+                            "the reference's bcx_decode (full LUT) and bcx_unpack6, compiled from its sources"),
+                      kind="reference")
+        result["oracle_port"] = port
+    else:
+        result = port
     if len(names) > 1:
         # the reference decodes one frame per thread; the same frames, one thread each, once
         from concurrent.futures import ThreadPoolExecutor
+        decode = (lambda f: reference_decode(core, orc, f)) if core is not None else orc.bctx_decode
         t0 = time.perf_counter()
         with ThreadPoolExecutor(max_workers=len(names)) as pool:
-            sizes = list(pool.map(lambda n: orc.bctx_decode(frames[n]).nbytes, names))
+            sizes = list(pool.map(lambda n: decode(frames[n]).nbytes, names))
         dt = time.perf_counter() - t0
         total = sum(len(frames[n]) for n in names)
         result["one_frame_per_thread"] = dict(value=round(total / dt / 1e9, 4), unit="GB/s", cores=len(names),
@@ -410,9 +505,13 @@ def main():
                      "kernel": (f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, false>" if m <= 8
                                 else "grf::fused_gemm_kernel<grf::SegmentWalk, MT>") + f" on {dom}"},
     }
+    copy_rate = measured_copy_gbps(torch)
+    result["hbm_copy_measured_GBps"] = round(copy_rate, 1)
+    result["pct_of_measured_copy"] = round(100 * value / copy_rate, 2)
     if not args.no_cpu_baseline:
         log("timing the CPU oracle on whole frames ...")
         result["cpu_baseline"] = cpu_baseline(frames, words_of, x_words)
+        result["cpu_baseline"]["host"] = host_description()
     print(json.dumps(result), flush=True)
 
 
