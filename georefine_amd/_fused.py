@@ -308,6 +308,18 @@ class FramePlan:
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
                                  n_tiles=n_tiles, piece_cap=cap), lds=lds)
 
+    def gather_scalars(self):
+        """Scalars of a tiling that gives every requested row a tile of its own, all of its
+        segments walked at once where a workgroup has the lanes (rows need no grouping by class
+        then); the caller supplies the rows and their classes per call."""
+        p = min(self.spr, 1024)
+        cap = self._cap(p)
+        lds = lds_bytes(self.nc, self.lognb, self.tabn, 0, p, self.seg_len, 1, cap)
+        if lds > MAX_LDS:
+            raise FusedUnsupported("gather tile does not fit in LDS")
+        return dict(threads=-(-p // 64) * 64, lanes_per_row=p, rows_per_tile=1, n_slabs=-(-self.spr // p),
+                    piece_cap=cap), lds
+
     def gemm_tiling(self):
         """The one tiling every fused GEMM launch uses, whatever its row count: the order in
         which an output element accumulates follows the tiling, so it must not change with M."""

@@ -190,6 +190,7 @@ class HipContextTensor:
             f.main.n_bytes = self._main_bytes
             self._frame = f
         self._tilings = {}
+        self._gather = None  # scalars of the row-gather tiling once planned; False: not possible
         if plan is not None:
             d = _hip_abi.GrfBctxFused()
             b = self.buffers
@@ -371,12 +372,37 @@ class HipContextTensor:
         return self.gemv(x, bias, check=check)
 
     def gather_rows(self, ids, *, check=True):
+        """Rows ``ids`` (any shape) as BF16 [*ids.shape, cols]; IndexError for a row the matrix
+        does not have (GCR/bitexact_context_gpu.py:159-168).  Frames the tile walker takes give
+        every requested row a workgroup that walks all of its segments at once; others decode
+        the checkpoint blocks of the rows, one lane each."""
         import torch
         ids = ids.to(device=self.device, dtype=torch.int64)
         if ids.numel() == 0:
             return torch.empty((*ids.shape, self.shape[1]), device=self.device, dtype=torch.bfloat16)
         if torch.any((ids < 0) | (ids >= self.shape[0])).item():
             raise IndexError("embedding row outside tensor")
+        if self.fused is not None and self._gather is not False:
+            if self._gather is None:
+                try:
+                    self._gather = self._plan.gather_scalars()[0]
+                except _fused.FusedUnsupported:
+                    self._gather = False
+            if self._gather:
+                flat = ids.reshape(-1)
+                rows = flat.to(torch.int32)
+                classes = self.buffers["rows"][flat]
+                g = _hip_abi.GrfFusedTiling()
+                g.tile_rows, g.tile_class, g.n_tiles = rows.data_ptr(), classes.data_ptr(), flat.numel()
+                for key, value in self._gather.items():
+                    setattr(g, key, value)
+                out = torch.empty((flat.numel(), self.shape[1]), device=self.device, dtype=torch.uint16)
+                if check:  # between checks the word keeps what earlier launches reported
+                    self.error.zero_()
+                self._launch(self._lib.grf_bctx_fused_gather, ctypes.byref(self.fused), ctypes.byref(g), out.data_ptr(),
+                             self.error.data_ptr())
+                self._check(check)
+                return out.view(torch.bfloat16).reshape(*ids.shape, self.shape[1])
         if self.mode == 1 or self.shape[1] % self.stride:
             return self.decode(check=check)[ids]
         per_row = self.shape[1] // self.stride

@@ -46,8 +46,17 @@ int grf_bctx_fused_decode(const grf_bctx_fused *frame, const grf_fused_tiling *t
   if (!frame || !tiling || !out || !error)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_fused_decode: null argument");
   if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_fused_decode")) return rc;
-  return grf::launch_walk<grf::SegmentWalk, 1, true>(*frame, *tiling, nullptr, 0, nullptr, 0, nullptr, out, error,
+  return grf::launch_walk<grf::SegmentWalk, 1, grf::kStore>(*frame, *tiling, nullptr, 0, nullptr, 0, nullptr, out, error,
                                                      (hipStream_t)hip_stream);
+}
+
+int grf_bctx_fused_gather(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint16_t *out,
+                          int32_t *error, void *hip_stream) {
+  if (!frame || !tiling || !out || !error)
+    return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_fused_gather: null argument");
+  if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_fused_gather")) return rc;
+  return grf::launch_walk<grf::SegmentWalk, 1, grf::kGather>(*frame, *tiling, nullptr, 0, nullptr, 0, nullptr, out,
+                                                             error, (hipStream_t)hip_stream);
 }
 
 }  // extern "C"

@@ -67,13 +67,19 @@ __device__ __forceinline__ uint16_t round_bf16(float v) {
   return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
 }
 
-template <class Walk, int M, bool STORE>
+// What a lane does with the words it decodes: multiply them into M activation rows, store
+// them where the row lies in the dense matrix, or store them in the slot the row has in the
+// tiling (row tile * R + r of a compact [n_tiles * R][cols] output: a gather of rows).
+enum Sink : int { kDot = 0, kStore = 1, kGather = 2 };
+
+template <class Walk, int M, int SINK>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_bctx_fused f, grf_fused_tiling g,
                                                                             const uint16_t *x, uint32_t ldx,
                                                                             uint16_t *y, uint32_t ldy,
                                                                             const uint16_t *bias, uint16_t *out,
                                                                             int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
+  constexpr bool STORE = SINK != kDot;
   const FusedLdsLayout L(f, g, STORE ? 0 : M);
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
@@ -81,7 +87,8 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
 
   const uint32_t r = tid / P, p = tid % P;
-  const uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
+  uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
+  if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
   uint16_t *xs = reinterpret_cast<uint16_t *>(lds + L.xs);
   const uint32_t xpitch = S + grf::kXPad;
   const uint32_t width = P * S;
@@ -132,7 +139,8 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
         uint32_t pair[8];
         w.decode16(t, S, q, pair);
         if (STORE) {
-          uint4 *dst = reinterpret_cast<uint4 *>(out + elem0 + t);
+          const uint64_t at = SINK == kGather ? (uint64_t)(tile * R + r) * K + col0 : elem0;
+          uint4 *dst = reinterpret_cast<uint4 *>(out + at + t);
           dst[0] = make_uint4(pair[0], pair[1], pair[2], pair[3]);
           dst[1] = make_uint4(pair[4], pair[5], pair[6], pair[7]);
         } else {
@@ -178,13 +186,13 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
   if (bad) atomicOr(error, (int)bad);
 }
 
-template <class Walk, int M, bool STORE>
+template <class Walk, int M, int SINK>
 int launch_walk(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx,
                 uint16_t *y,
                 uint32_t ldy, const uint16_t *bias, uint16_t *out, int32_t *error, hipStream_t s) {
-  const FusedLdsLayout L(f, g, STORE ? 0 : M);
+  const FusedLdsLayout L(f, g, SINK != kDot ? 0 : M);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
-  constexpr auto kernel = &fused_walk_kernel<Walk, M, STORE>;
+  constexpr auto kernel = &fused_walk_kernel<Walk, M, SINK>;
   if (L.total > 64 * 1024)
     if (int rc = allow_full_lds<kernel>()) return rc;
   hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, x, ldx, y, ldy, bias, out, error);
@@ -202,14 +210,14 @@ int launch_gemv(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
     return grf::set_error(GRF_BAD_ARGUMENT,
                           std::string(who) + ": x must be 4-byte aligned with an even leading dimension");
   switch (m_rows) {
-    case 1: return launch_walk<Walk, 1, false>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
-    case 2: return launch_walk<Walk, 2, false>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
-    case 3: return launch_walk<Walk, 3, false>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
-    case 4: return launch_walk<Walk, 4, false>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
-    case 5: return launch_walk<Walk, 5, false>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
-    case 6: return launch_walk<Walk, 6, false>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
-    case 7: return launch_walk<Walk, 7, false>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
-    default: return launch_walk<Walk, 8, false>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    case 1: return launch_walk<Walk, 1, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    case 2: return launch_walk<Walk, 2, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    case 3: return launch_walk<Walk, 3, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    case 4: return launch_walk<Walk, 4, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    case 5: return launch_walk<Walk, 5, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    case 6: return launch_walk<Walk, 6, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    case 7: return launch_walk<Walk, 7, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    default: return launch_walk<Walk, 8, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
   }
 }
 

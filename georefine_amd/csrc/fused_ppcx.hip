@@ -225,7 +225,7 @@ int grf_ppcx_fused_decode(const grf_ppcx_fused *frame, const grf_fused_tiling *t
   if (!out || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_fused_decode: null argument");
   grf_bctx_fused f;
   if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_fused_decode", f)) return rc;
-  return grf::launch_walk<PpcxWalk, 1, true>(f, *tiling, nullptr, 0, nullptr, 0, nullptr, out, error,
+  return grf::launch_walk<PpcxWalk, 1, grf::kStore>(f, *tiling, nullptr, 0, nullptr, 0, nullptr, out, error,
                                              (hipStream_t)hip_stream);
 }
 

@@ -211,6 +211,16 @@ int grf_bctx_gemv(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
 int grf_bctx_fused_decode(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint16_t *out,
                           int32_t *error, void *hip_stream);
 
+/* Rows of a coded matrix, decoded by the same walker into a compact output (the embedding
+ * lookup of CudaContextTensor.gather_rows, GCR/bitexact_context_gpu.py:159-168, without
+ * decoding checkpoint blocks one lane each).  The tiling names the rows: slot s = tile *
+ * rows_per_tile + r holds row tile_rows[s] (0xFFFFFFFF = empty; a row may appear in any
+ * number of slots) and is written to out[s][cols]; the rows of a tile must share the row
+ * class tile_class[tile].  One row per tile with lanes_per_row = segs_per_row needs no
+ * grouping at all.  Rows outside the matrix are the caller's to reject. */
+int grf_bctx_fused_gather(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint16_t *out,
+                          int32_t *error, void *hip_stream);
+
 /* Fused decode-GEMM on the matrix cores for any number of activation rows; same operand
  * meaning as grf_bctx_gemv.  Batch-invariant in the sense of GS/bi_csrc/bi_gemm.cuh:1-17:
  * with one tiling, row m of y is a function of row m of x and of W only.  x must be
