@@ -142,6 +142,32 @@ def test_whole_stack_resident_one_pass_at_batch_64():
     assert _digest(keep.decode(check=True)) == want
 
 
+def test_vocabulary_sized_matrix_decode_products_and_row_lookup():
+    """248320 x 5120 (the head and embedding of the 27B model, 1.27 G weights, close to the
+    frame format's 2^32 - 1 elements): element and byte offsets beyond 2^31, 19.9 M segments."""
+    import torch
+    from concurrent.futures import ThreadPoolExecutor
+    rows, cols, step = 248320, 5120, 15520
+
+    def chunk(i):
+        return weight_like(np.random.default_rng(7000 + i), step, cols)
+
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        words = np.concatenate(list(pool.map(chunk, range(rows // step))))
+    assert words.shape == (rows, cols)
+    frame, t = _tensor(words)
+    assert t.fused is not None, t.fused_reason
+    want = hashlib.sha256(words.tobytes()).hexdigest()
+    assert t.source_sha256 == want and len(frame) > 1 << 30
+    assert _digest(t.decode(check=True)) == want
+    x = torch.from_numpy(bf16_words(np.random.default_rng(8).normal(0, 1, size=(16, cols)))).view(torch.bfloat16).cuda()
+    _check_products(t, x[:8], (1, 2), lambda v: t.gemv(v, check=True))
+    _check_products(t, x, (1, 16), lambda v: t.gemm(v, check=True))
+    ids = torch.tensor([0, rows - 1, 123456, 200000, 200000, 131072])
+    got = t.gather_rows(ids, check=True).view(torch.uint16).cpu().numpy()
+    assert np.array_equal(got, words[ids.numpy()])
+
+
 def test_predictive_frame_full_size_decode_and_batch_96():
     """A 5120 x 17408 target coded against a near-identical reference; the product takes
     16 users x (5 speculative + 1) = 96 rows."""
