@@ -104,7 +104,7 @@ def lds_bytes(nc, lognb, tabn, m, p, s, r, piece_cap):
     return total
 
 
-GEMM_MAX_TILES = 4  # 16-row activation tiles of one GEMM launch
+GEMM_MAX_TILES = 4  # 16-row activation tiles whose partial sums pass through LDS at a time
 
 
 def gemm_shape(p, r):
