@@ -318,7 +318,7 @@ def run_stack(args):
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     dom = max(LAYER, key=lambda n_: ms[n_])
     achieved = alg[dom]["total"] / (ms[dom] * 1e-3) / 1e9
-    kernel = "grf::fused_gemm_kernel<grf::SegmentWalk, MT>" if m > 8 else f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, false>"
+    kernel = "grf::fused_gemm_kernel<grf::SegmentWalk, MT>" if m > 8 else f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>"
     print(json.dumps({
         "metric": "compressed-weight decode-GEMV GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
@@ -502,7 +502,7 @@ def main():
                             "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in names},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "kernel": (f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, false>" if m <= 8
+                     "kernel": (f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>" if m <= 8
                                 else "grf::fused_gemm_kernel<grf::SegmentWalk, MT>") + f" on {dom}"},
     }
     copy_rate = measured_copy_gbps(torch)
