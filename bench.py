@@ -61,6 +61,9 @@ def synth_weights(index, rows, cols):
     return out
 
 
+GEMV_UP_TO = 2  # HipContextTensor.GEMV_UP_TO: linear() gives more rows to the matrix-core kernel
+
+
 def algorithmic_bytes(t, m):
     """Bytes one fused GEMV launch has to touch once: both streams, the fused index,
     the per-class lookup tables, labels, activations and outputs."""
@@ -68,7 +71,7 @@ def algorithmic_bytes(t, m):
     n = lambda k: b[k].numel() * b[k].element_size()
     rows, cols = t.shape
     payload = t._main_bytes + n("residual_stream")
-    _, tile_rows, tile_class, _ = t._tiling(m) if m <= 8 else t._gemm_tiling()
+    _, tile_rows, tile_class, _ = t._tiling(m) if m <= GEMV_UP_TO else t._gemm_tiling()
     index = (n("fused_seg_state") + n("fused_seg_offset") + tile_rows.numel() * tile_rows.element_size()
              + tile_class.numel() * tile_class.element_size())
     tables = n("fused_lut") + n("fused_tab")
@@ -254,7 +257,7 @@ def run_stack(args):
         layers.append(src if i < args.distinct_layers else {k: v.clone() for k, v in src.items()})
     for layer in layers:
         for t in layer.values():
-            t._gemm_tiling() if m > 8 else t._tiling(m)
+            t._gemm_tiling() if m > GEMV_UP_TO else t._tiling(m)
     torch.cuda.synchronize()
     frame_bytes = sum(t.frame_bytes for layer in layers for t in layer.values())
     resident = sum(t.resident_bytes for layer in layers for t in layer.values())
@@ -269,7 +272,7 @@ def run_stack(args):
     def step():
         for layer in layers:
             for name, t in layer.items():
-                t.linear(x[LAYER[name][1]], batch_invariant=m > 8)
+                t.linear(x[LAYER[name][1]], batch_invariant=m > GEMV_UP_TO)
 
     for _ in range(args.warmup):
         step()
@@ -283,7 +286,7 @@ def run_stack(args):
                 if i == 0:
                     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                     a.record()
-                t.linear(x[LAYER[name][1]], batch_invariant=m > 8)
+                t.linear(x[LAYER[name][1]], batch_invariant=m > GEMV_UP_TO)
                 if i == 0:
                     b.record()
                     probes[name].append((a, b))
@@ -318,7 +321,7 @@ def run_stack(args):
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     dom = max(LAYER, key=lambda n_: ms[n_])
     achieved = alg[dom]["total"] / (ms[dom] * 1e-3) / 1e9
-    kernel = "grf::fused_gemm_kernel<grf::SegmentWalk, MT>" if m > 8 else f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>"
+    kernel = "grf::fused_gemm_kernel<grf::SegmentWalk, MT>" if m > GEMV_UP_TO else f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>"
     print(json.dumps({
         "metric": "compressed-weight decode-GEMV GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
@@ -345,7 +348,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--batch", type=int, default=1, help="activation rows; 1..8 run the fused GEMV (the headline figure is batch 1), more the fused GEMM")
+    ap.add_argument("--batch", type=int, default=1, help="activation rows; 1..2 run the fused GEMV (the headline figure is batch 1), more the fused GEMM")
     ap.add_argument("--segment", type=int, default=0, help="fused segment length (0 = automatic)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
@@ -393,7 +396,7 @@ def main():
             sys.exit(f"bench.py: {name} is not eligible for the fused kernel: {tensors[name].fused_reason}")
         log(f"{name}: {rows}x{cols} mode {tensors[name].mode} frame {len(frame)} B "
             f"({8 * len(frame) / w.size:.3f} bit/weight) encode {t1 - t0:.1f}s index+upload {t2 - t1:.1f}s "
-            f"plan {tensors[name].fused_plan} tiling {(tensors[name]._tiling(args.batch) if args.batch <= 8 else tensors[name]._gemm_tiling())[3]}")
+            f"plan {tensors[name].fused_plan} tiling {(tensors[name]._tiling(args.batch) if args.batch <= GEMV_UP_TO else tensors[name]._gemm_tiling())[3]}")
         frames[name] = frame
         words_of[name] = w
     log(f"setup {time.perf_counter() - t_setup:.1f}s")
@@ -489,7 +492,7 @@ def main():
         "vs_baseline": None,
         "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
         "data": "synthetic",
-        "config": {"workload": "fused decode-" + ("GEMV" if m <= 8 else "GEMM") + ", batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
+        "config": {"workload": "fused decode-" + ("GEMV" if m <= GEMV_UP_TO else "GEMM") + ", batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
                                "BCTX (16,4) frames, residuals resident in packed 6-bit form" % m,
                    "batch": m, "matrices": names,
                    "segment": tensors[names[0]].fused_plan["seg_len"], "launch": launch},
@@ -502,7 +505,7 @@ def main():
                             "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in names},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "kernel": (f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>" if m <= 8
+                     "kernel": (f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>" if m <= GEMV_UP_TO
                                 else "grf::fused_gemm_kernel<grf::SegmentWalk, MT>") + f" on {dom}"},
     }
     copy_rate = measured_copy_gbps(torch)
