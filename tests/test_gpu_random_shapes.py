@@ -1,6 +1,8 @@
 """Seeded sweep over shapes, class counts, segment lengths and value distributions: every
 sink of the tile walker against the CPU oracle (decode bit-exact) and the dense product of the
 decoded words (GEMV and GEMM within 1e-2 relative, rows independent of the batch)."""
+import os
+
 import numpy as np
 import pytest
 
@@ -30,7 +32,7 @@ def _matrix(rng, rows, cols, kind):
 WALKED = []  # cases that went through the tile walker (filled as the sweep runs)
 CASES = []
 _rng = np.random.default_rng(2024)
-for _i in range(40):
+for _i in range(int(os.environ.get("GEOREFINE_TEST_SWEEP_CASES", "40"))):  # a longer sweep on request
     CASES.append((int(_rng.integers(1, 260)), 16 * int(_rng.integers(1, 96)),
                   [(16, 4), (1, 1), (4, 16), (64, 4), (16, 16)][_i % 5],
                   ["weights", "wide", "two-valued", "special", "row-constant"][(_i // 5) % 5], 3000 + _i))
@@ -58,11 +60,13 @@ def test_every_sink_on_a_random_case(oracle, rows, cols, classes, kind, seed):
         return
     assert np.array_equal(t.decode(check=True).view(torch.uint16).cpu().numpy(), words)
     WALKED.append((rows, cols))
+    ids = torch.from_numpy(rng.integers(0, rows, size=(2, 9)))
+    assert np.array_equal(t.gather_rows(ids, check=True).view(torch.uint16).cpu().numpy(), words[ids.numpy()])
     finite = torch.from_numpy(words).view(torch.bfloat16).float().nan_to_num(0.0, 0.0, 0.0).abs().max() < 1e30
     if kind in ("special", "wide") or not bool(finite):
         return  # non-finite or huge words: products are not comparable within a relative tolerance
     dense_w = t.decode().float()
-    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(20, cols)))).view(torch.bfloat16).cuda()
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(70, cols)))).view(torch.bfloat16).cuda()
     want = torch.nn.functional.linear(x.float(), dense_w)
     scale = torch.nn.functional.linear(x.float().abs(), dense_w.abs())
 
@@ -74,10 +78,10 @@ def test_every_sink_on_a_random_case(oracle, rows, cols, classes, kind, seed):
     assert close(y8)
     for m in (1, 3, 6):
         assert torch.equal(t.gemv(x[:m]).view(torch.uint16), y8[:m].view(torch.uint16))
-    y20 = t.gemm(x, check=True)
-    assert close(y20)
-    for m in (1, 8, 17):
-        assert torch.equal(t.gemm(x[:m]).view(torch.uint16), y20[:m].view(torch.uint16))
+    y70 = t.gemm(x, check=True)  # the eight-tile kernel; fewer rows run the one-, two- and four-tile ones
+    assert close(y70)
+    for m in (1, 8, 17, 40):
+        assert torch.equal(t.gemm(x[:m]).view(torch.uint16), y70[:m].view(torch.uint16))
 
 
 def test_sweep_exercised_the_walker():
