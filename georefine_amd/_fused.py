@@ -147,7 +147,16 @@ def _spread_rows(class_rows, r, capacity, floor=1):
     return r
 
 
-def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
+def _walk_share(n_slabs, seg_len, table_bytes):
+    """Share of a workgroup's life spent walking, in units of decode steps: before the first
+    step a workgroup copies its row class's tables (about a step per 12 KiB, measured on
+    53 KiB tables with one 64-step slab: 10 %) and every slab costs a barrier and a staging
+    round (about two steps)."""
+    steps = n_slabs * seg_len
+    return steps / (steps + 3 + table_bytes / 12288 + 2 * n_slabs)
+
+
+def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=64, table_bytes=0):
     """(threads T, lanes_per_row P, rows_per_tile R, ...): best modelled throughput.
 
     The walk is a chain of dependent steps per lane, so time ~ steps per lane x rounds
@@ -191,7 +200,7 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
             slots = cus * per_cu
             rounds = -(-tiles // slots)
             quant = tiles / (rounds * slots)
-            score = lane_eff * fill * quant * min(1.0, waves / 24)
+            score = lane_eff * fill * quant * min(1.0, waves / 24) * _walk_share(n_slabs, seg_len, table_bytes)
             if best is None or score > best[0] + 1e-9:
                 best = (score, threads, p, r, n_slabs, tiles, cap, lds, rounds * slots)
     if best is None:
@@ -206,7 +215,7 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
 GEMM_WAVES_PER_SIMD = int(os.environ.get("GEOREFINE_GEMM_WAVES", "6"))
 
 
-def choose_gemm_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
+def choose_gemm_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=64, table_bytes=0):
     """Tiling of the GEMM kernel: workgroups of (row blocks of 16) x (quads of 4
     lane-segments) waves.  Same model as choose_tiling, counted in waves: a wave is busy
     for as long as its busiest lane, so idle lanes inside a wave are free, idle waves and
@@ -241,7 +250,7 @@ def choose_gemm_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256):
         work = total_rows * spr
         paid = rounds * slots * (threads // 64) * 16 * 4 * n_slabs
         waves = per_cu * (threads // 64)
-        score = work / paid * min(1.0, waves / 24)
+        score = work / paid * min(1.0, waves / 24) * _walk_share(n_slabs, seg_len, table_bytes)
         if best is None or score > best[0] + 1e-9:
             best = (score, threads, p, r_used, n_slabs, tiles_used, cap, lds_fn(p, r_used, cap))
     if best is None:
@@ -272,13 +281,13 @@ class FramePlan:
     """Frame-level derived arrays (shared by every tiling) and a tiling factory."""
 
     def __init__(self, shape, nr, nc, row_class, main_freq, seg_states, seg_offsets, main_bytes, seg_len,
-                 image=None):
+                 image=None, lut_budget=None):
         rows, cols = shape
         if rows * cols > 0xFFFFFFFF:
             raise FusedUnsupported("matrix too large")
         self.rows, self.cols, self.nr, self.nc, self.seg_len = rows, cols, nr, nc, seg_len
         self.spr = cols // seg_len
-        self.shift = choose_shift(nc)
+        self.shift = choose_shift(nc, lut_budget or LUT_BUDGET)
         self.lognb = 16 - self.shift
         self.lut, self.tab, self.tabn = sparse_tables(main_freq, nr, nc, self.shift, image)
         self.seg_state = np.concatenate((seg_states, [1 << 23])).astype(np.uint32)
@@ -286,6 +295,10 @@ class FramePlan:
         self.row_class = np.asarray(row_class)
         self.class_rows = np.bincount(self.row_class, minlength=nr)
         self._caps = {}
+
+    def table_bytes(self):
+        """LDS bytes of one row class's lookup tables (what every workgroup copies first)."""
+        return self.nc * (((self.tabn + 1) * 8 + 15) // 16 * 16 + (1 << self.lognb))
 
     def scalars(self):
         return dict(rows=self.rows, cols=self.cols, nr=self.nr, nc=self.nc, seg_len=self.seg_len,
@@ -301,7 +314,8 @@ class FramePlan:
         (m = 0: the store sink)."""
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
             self.spr, self.class_rows, self._cap,
-            lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_))
+            lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_),
+            seg_len=self.seg_len, table_bytes=self.table_bytes())
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
@@ -325,7 +339,8 @@ class FramePlan:
         which an output element accumulates follows the tiling, so it must not change with M."""
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_gemm_tiling(
             self.spr, self.class_rows, self._cap,
-            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, p_, r_, cap_))
+            lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, p_, r_, cap_),
+            seg_len=self.seg_len, table_bytes=self.table_bytes())
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
