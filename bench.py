@@ -508,6 +508,11 @@ def main():
                      "kernel": (f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>" if m <= GEMV_UP_TO
                                 else "grf::fused_gemm_kernel<grf::SegmentWalk, MT>") + f" on {dom}"},
     }
+    if m > GEMV_UP_TO:
+        # the matrix cores' share: useful flops of the dominant launch against the dense BF16 peak
+        flops = 2.0 * m * SHAPES[dom][0] * SHAPES[dom][1]
+        result["mfma"] = {"achieved": round(flops / (per_kernel_ms[dom] * 1e-3) / 1e12, 2), "peak": 2500.0,
+                          "unit": "TFLOP/s", "frac": round(flops / (per_kernel_ms[dom] * 1e-3) / 2.5e15, 4)}
     copy_rate = measured_copy_gbps(torch)
     result["hbm_copy_measured_GBps"] = round(copy_rate, 1)
     result["pct_of_measured_copy"] = round(100 * value / copy_rate, 2)
