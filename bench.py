@@ -61,7 +61,7 @@ def synth_weights(index, rows, cols):
     return out
 
 
-GEMV_UP_TO = 2  # HipContextTensor.GEMV_UP_TO: linear() gives more rows to the matrix-core kernel
+GEMV_UP_TO = 2  # rows linear() gives to the vector-ALU kernel; read from HipContextTensor once it is imported
 
 
 def algorithmic_bytes(t, m):
@@ -226,6 +226,8 @@ def run_stack(args):
     from concurrent.futures import ThreadPoolExecutor
     from georefine_amd import bitexact_context_codec as codec
     from georefine_amd.bitexact_context_gpu import HipContextTensor
+    global GEMV_UP_TO
+    GEMV_UP_TO = HipContextTensor.GEMV_UP_TO
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: needs a ROCm GPU")
@@ -375,6 +377,8 @@ def main():
     import torch
     from georefine_amd import bitexact_context_codec as codec
     from georefine_amd.bitexact_context_gpu import HipContextTensor
+    global GEMV_UP_TO
+    GEMV_UP_TO = HipContextTensor.GEMV_UP_TO
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: needs a ROCm GPU")
