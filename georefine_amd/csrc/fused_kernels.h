@@ -178,7 +178,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
     for (uint32_t i = tid; i < R * M; i += nthreads) {
       const uint32_t rr = i / M, m = i % M;
       const uint32_t orow = g.tile_rows[tile * R + rr];
-      if (orow == grf::kNoRow) continue;
+      if (orow >= f.rows) continue;  // empty slot or no such row
       float sum = rowsum[i];
       if (bias) sum += __uint_as_float((uint32_t)bias[orow] << 16);
       y[(size_t)m * ldy + orow] = round_bf16(sum);
@@ -322,7 +322,8 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   const uint32_t wave = tid / 64, lane = tid % 64;
   const uint32_t rb = wave % shape.row_blocks, quad = wave / shape.row_blocks;
   const uint32_t r = rb * 16 + lane % 16, p = quad * 4 + lane / 16;
-  const uint32_t row = (r < R && p < P) ? g.tile_rows[tile * R + r] : grf::kNoRow;
+  uint32_t row = (r < R && p < P) ? g.tile_rows[tile * R + r] : grf::kNoRow;
+  if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
   grf::PieceSpan span{0, 0};  // started before the table copy so that the latencies overlap
   if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
@@ -392,7 +393,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
       const uint32_t jj = within / 256, v = (within / 64) % 4, ln = within % 64;
       const uint32_t n_local = blk * 16 + ln % 16, m = (c0 + jj) * 16 + (ln / 16) * 4 + v;
       const uint32_t orow = n_local < R ? g.tile_rows[tile * R + n_local] : grf::kNoRow;
-      if (orow == grf::kNoRow || m >= m_rows) continue;
+      if (orow >= f.rows || m >= m_rows) continue;  // empty slot, no such row, or a padding row
       // wave index of (quad, block) is quad * row_blocks + block
       float sum = sums[(blk * CT) * 256 + within];
       for (uint32_t qd = 1; qd < shape.quads; ++qd) sum += sums[((qd * shape.row_blocks + blk) * CT) * 256 + within];

@@ -197,3 +197,65 @@ def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle,
     wrong = torch.from_numpy(np.roll(ref, 5, axis=1).copy()).view(torch.bfloat16).cuda()
     with pytest.raises(codec.CodecError):
         t.linear(wrong, x[:2], check=True)
+
+
+# ---------------------------------------------------------------- seeded sweep over predictive frames
+SWEEP = []
+_sweep_rng = np.random.default_rng(909)
+for _i in range(30):
+    SWEEP.append((int(_sweep_rng.integers(1, 220)), 32 * int(_sweep_rng.integers(1, 56)), _i % 2,
+                  ["near", "far", "negated rows", "special", "identical"][(_i // 2) % 5], 7000 + _i))
+
+
+@pytest.mark.parametrize("rows,cols,mode,kind,seed", SWEEP, ids=[f"{r}x{c}-mode{m}-{k}" for r, c, m, k, _ in SWEEP])
+def test_every_predictive_sink_on_a_random_case(oracle, rows, cols, mode, kind, seed):
+    """Shapes, reference quality and residual forms at random: every sink of the predictive
+    walker against the CPU oracle (decode bit-exact) and the dense product of the target
+    (1e-2 relative; rows independent of the batch)."""
+    import torch
+    from georefine_amd import bitexact_predictive_codec as codec
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
+    rng = np.random.default_rng(seed)
+    target = weight_like(rng, rows, cols)
+    tf = (target.astype(np.uint32) << 16).view(np.float32)
+    if kind == "near":
+        ref = bf16_words(tf + rng.normal(0, 0.002, target.shape).astype(np.float32))
+    elif kind == "far":
+        ref = weight_like(rng, rows, cols)                     # unrelated: the bins carry no information
+    elif kind == "negated rows":
+        ref = bf16_words(tf * rng.choice([-1.0, 1.0], size=(rows, 1)).astype(np.float32))  # sign flips per row
+    elif kind == "special":
+        ref = bf16_words(tf + rng.normal(0, 0.002, target.shape).astype(np.float32))
+        from conftest import SPECIAL_WORDS
+        mask = rng.random(target.shape) < 0.03
+        ref[mask] = rng.choice(SPECIAL_WORDS, size=int(mask.sum()))  # infinities, NaNs, zeros in the reference
+    else:
+        ref = target.copy()
+    frame = _frame_for_mode(codec, target, ref, mode)
+    assert np.array_equal(oracle.ppcx_decode(frame, ref), target)
+    segments = [s for s in (32, 64, 128, 256) if cols % s == 0]
+    t = HipPredictiveTensor(frame, ref, stride=[64, 256, 1024][seed % 3], device="cuda:0",
+                            fused_segment=segments[seed % len(segments)])
+    ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
+    assert np.array_equal(t.decode(ref_dev, general=True).view(torch.uint16).cpu().numpy(), target)
+    if t.fused is None:
+        assert "255" in str(t.fused_reason), t.fused_reason    # a context with more than 255 live symbols
+        return
+    assert np.array_equal(t.decode(ref_dev).view(torch.uint16).cpu().numpy(), target)
+    dense_w = torch.from_numpy(target).view(torch.bfloat16).cuda().float()
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(70, cols)))).view(torch.bfloat16).cuda()
+    want = torch.nn.functional.linear(x.float(), dense_w)
+    scale = torch.nn.functional.linear(x.float().abs(), dense_w.abs())
+
+    def close(y):
+        n = y.shape[0]
+        return bool((y.float() - want[:n]).abs().le(1e-2 * want[:n].abs().clamp_min(1e-3 * scale[:n]) + 1e-30).all())
+
+    y8 = t.gemv(ref_dev, x[:8], check=True)
+    assert close(y8)
+    for m in (1, 3, 6):
+        assert torch.equal(t.gemv(ref_dev, x[:m]).view(torch.uint16), y8[:m].view(torch.uint16))
+    y70 = t.gemm(ref_dev, x, check=True)
+    assert close(y70)
+    for m in (1, 8, 17, 40):
+        assert torch.equal(t.gemm(ref_dev, x[:m]).view(torch.uint16), y70[:m].view(torch.uint16))
