@@ -233,7 +233,10 @@ __device__ __forceinline__ uint32_t fused_symbol_in(Cursor &c, uint32_t block, c
   fused_pin_bytes(s);
   uint64_t miss;
   uint32_t rel = fused_locate(c.state, s.e0.x, miss);
-  if (__builtin_expect(fused_lane_in(miss), 0)) fused_scan(c.state, s, rel);
+  // a branch on the whole mask first: the common path then leaves EXEC alone
+  if (__builtin_expect(miss != 0, 0)) {
+    if (fused_lane_in(miss)) fused_scan(c.state, s, rel);
+  }
   fused_advance(c, s, rel);
   return s.e0.y;
 }
