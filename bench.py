@@ -200,18 +200,19 @@ def cpu_baseline(frames, words_of, x_words, min_seconds=10.0, max_frames=12):
         result["oracle_port"] = port
     else:
         result = port
-    if len(names) > 1:
-        # the reference decodes one frame per thread; the same frames, one thread each, once
-        from concurrent.futures import ThreadPoolExecutor
-        decode = (lambda f: reference_decode(core, orc, f)) if core is not None else orc.bctx_decode
-        t0 = time.perf_counter()
-        with ThreadPoolExecutor(max_workers=len(names)) as pool:
-            sizes = list(pool.map(lambda n: decode(frames[n]).nbytes, names))
-        dt = time.perf_counter() - t0
-        total = sum(len(frames[n]) for n in names)
-        result["one_frame_per_thread"] = dict(value=round(total / dt / 1e9, 4), unit="GB/s", cores=len(names),
-                                              sample=f"{len(names)} frames decoded concurrently in {dt:.1f}s "
-                                                     f"({sum(sizes) / dt / 1e6:.1f} MB/s of BF16 produced)")
+    # the reference decodes one frame per thread: every host core with a frame of its own, once
+    from concurrent.futures import ThreadPoolExecutor
+    decode = (lambda f: reference_decode(core, orc, f)) if core is not None else orc.bctx_decode
+    threads = max(1, min(os.cpu_count() or 1, 16))
+    jobs = [names[i % len(names)] for i in range(threads)]
+    t0 = time.perf_counter()
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        sizes = list(pool.map(lambda n: decode(frames[n]).nbytes, jobs))
+    dt = time.perf_counter() - t0
+    total = sum(len(frames[n]) for n in jobs)
+    result["one_frame_per_thread"] = dict(value=round(total / dt / 1e9, 4), unit="GB/s", cores=threads,
+                                          sample=f"{threads} frames decoded concurrently, one thread each, in "
+                                                 f"{dt:.1f}s ({sum(sizes) / dt / 1e6:.1f} MB/s of BF16 produced)")
     return result
 
 
