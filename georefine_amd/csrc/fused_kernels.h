@@ -267,17 +267,18 @@ struct GemmLdsLayout {
 };
 
 // Activations in operand order: the 8 columns [8c, 8c+8) of row m at xp[c * m_pad + m]
-// (16 bytes); rows m_rows..m_pad-1 are zero.  A group of 64 threads moves 8 chunks of 8
-// rows, reading 128-byte runs of x and writing 128-byte runs of xp.
+// (16 bytes); rows m_rows..m_pad-1 are zero, and so is one more chunk after the last.  A
+// group of 64 threads moves 8 chunks of 8 rows, reading 128-byte runs of x and writing
+// 128-byte runs of xp.
 static __global__ __launch_bounds__(256) void pack_activations_kernel(const uint16_t *x, uint32_t ldx, uint32_t m_rows,
                                                                 uint32_t m_pad, uint32_t chunks, uint4 *xp) {
   const uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x;
   const uint32_t cc = idx % 8, ml = (idx / 8) % 8, blk = idx / 64;
   const uint32_t m_blocks = m_pad / 8;
   const uint32_t m = (blk % m_blocks) * 8 + ml, c = (blk / m_blocks) * 8 + cc;
-  if (c >= chunks) return;
+  if (c > chunks) return;
   uint4 v = make_uint4(0u, 0u, 0u, 0u);
-  if (m < m_rows) {
+  if (m < m_rows && c < chunks) {
     const uint2 *src = reinterpret_cast<const uint2 *>(x + (size_t)m * ldx + c * 8);
     const uint2 a = src[0], b = src[1];
     v = make_uint4(a.x, a.y, b.x, b.y);
@@ -286,9 +287,9 @@ static __global__ __launch_bounds__(256) void pack_activations_kernel(const uint
 }
 
 template <int MT>
-__device__ __forceinline__ void gemm_load_x(uint4 (&xa)[MT], const uint4 *xl, bool feeds) {
+__device__ __forceinline__ void gemm_load_x(uint4 (&xa)[MT], const uint4 *xl) {
 #pragma unroll
-  for (int j = 0; j < MT; ++j) xa[j] = feeds ? xl[j * 16] : make_uint4(0u, 0u, 0u, 0u);
+  for (int j = 0; j < MT; ++j) xa[j] = xl[j * 16];
 }
 
 template <int MT>
@@ -353,11 +354,14 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     if (__ballot(active) == 0) continue;  // nothing to walk in this wave (the branch is per wave)
     if (active) w.start(piece_off, a0);
     // A lane's k-slots are real columns when its segment exists, whether or not its own
-    // row does; other lanes feed zeros (their weights are zero too, but 0 * NaN is not).
+    // row does; other lanes feed zeros (their weights are zero too, but 0 * NaN is not):
+    // they read the chunk of zeros that ends the packed copy and never move on.  The load
+    // after a segment's last half group reads the chunk that follows it, at most that one.
     const bool feeds = p < nseg;
-    const uint4 *xl = xp + (size_t)(feeds ? col0 / 8 : 0) * m_pad + lane % 16;
+    const uint32_t x_step = feeds ? m_pad : 0;
+    const uint4 *xl = xp + (size_t)(feeds ? col0 / 8 : K / 8) * m_pad + lane % 16;
     uint4 xa[MT];
-    gemm_load_x<MT>(xa, xl, feeds);
+    gemm_load_x<MT>(xa, xl);
     for (uint32_t t = 0; t < S; t += 16) {
       uint32_t lo[4] = {0u, 0u, 0u, 0u}, hi[4] = {0u, 0u, 0u, 0u};
       if (active) {
@@ -365,12 +369,12 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
         w.template half<0>(q, lo);
       }
       gemm_contract<MT>(acc, xa, lo);
-      xl += m_pad;
-      gemm_load_x<MT>(xa, xl, feeds);
+      xl += x_step;
+      gemm_load_x<MT>(xa, xl);
       if (active) w.template half<1>(q, hi);
       gemm_contract<MT>(acc, xa, hi);
-      xl += m_pad;
-      gemm_load_x<MT>(xa, xl, feeds && t + 16 < S);
+      xl += x_step;
+      gemm_load_x<MT>(xa, xl);
     }
     if (active && !w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
   }
@@ -430,7 +434,7 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
   const GemmLdsLayout L(f, g);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused GEMM: LDS demand exceeds 160 KiB");
   const uint32_t chunks = f.cols / 8, m_pad = MT * 16;
-  const uint32_t pack_threads = (chunks + 7) / 8 * 8 * m_pad;
+  const uint32_t pack_threads = (chunks + 1 + 7) / 8 * 8 * m_pad;  // the chunks and the chunk of zeros after them
   hipLaunchKernelGGL(pack_activations_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, x, ldx, m_rows, m_pad,
                      chunks, xp);
   constexpr auto kernel = [] {
@@ -449,7 +453,7 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
 inline size_t gemm_workspace_bytes(uint32_t cols, uint32_t m_rows) {
   const uint32_t m = m_rows > kMaxRowsPerLaunch ? kMaxRowsPerLaunch : m_rows;
   const uint32_t tiles = m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8;
-  return (size_t)(cols / 8) * tiles * 16 * 16;
+  return (size_t)(cols / 8 + 1) * tiles * 16 * 16;
 }
 
 // y = x W^T (+ bias) for any number of activation rows, 128 per launch.  `workspace` holds

@@ -230,7 +230,7 @@ int grf_bctx_fused_gather(const grf_bctx_fused *frame, const grf_fused_tiling *t
  * ceil(lanes_per_row / 4): a wave walks four lane-segments of 16 rows and feeds the words
  * it decodes to the matrix cores from its registers.  workspace: device memory, 16-byte
  * aligned, at least grf_gemm_workspace_bytes(cols, m_rows) bytes; each launch first writes
- * its activation rows there in operand order (a copy of x: cols * 32 bytes per 16 rows),
+ * its activation rows there in operand order (a copy of x: cols * 32 + 256 bytes per 16 rows),
  * so calls that share a workspace must be ordered on one stream. */
 int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, const uint16_t *x, uint32_t ldx,
                   uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
