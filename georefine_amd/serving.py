@@ -432,3 +432,26 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         "consumed_tensors": consumed, "restored_bf16_control": False, "transcoded": False,
     }
     return model, receipt
+
+
+def load_predictive_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
+                          tensor_factory=None, context_factory=None, predictive_factory=None, mix_predictor=None,
+                          host_decoder=None, loader_workers=1, batch_invariant=False, log=print,
+                          progress_callback=None):
+    """The predictive-package loader under the reference's name and keywords
+    (GCR/bitexact_predictive_serving.py:596-619): ``context_factory`` makes the BCTX tensors
+    (``tensor_factory`` is accepted as its older spelling), ``predictive_factory`` the PPCX ones,
+    ``mix_predictor`` the mixed references.  ``load_bctx_model`` already resolves the manifest's
+    ``selected_candidates``, so both names load the same packages; this one insists that the
+    package has candidates to resolve."""
+    from . import bitexact_context_package as pkg
+    if context_factory is not None and tensor_factory is not None and context_factory is not tensor_factory:
+        raise ValueError("pass context_factory or tensor_factory, not two different ones")
+    manifest, _ = pkg.read_manifest(package)
+    if not manifest.get("selected_candidates"):
+        raise ContextServingError("package has no predictive candidates; use load_bctx_model")
+    return load_bctx_model(package, model_factory=model_factory, device=device, dtype=dtype, stride=stride,
+                           tensor_factory=context_factory or tensor_factory, predictive_factory=predictive_factory,
+                           mix_predictor=mix_predictor, host_decoder=host_decoder, loader_workers=loader_workers,
+                           batch_invariant=batch_invariant, log=log, progress_callback=progress_callback)
+

@@ -239,6 +239,28 @@ def _gated_package(tmp_path):
     return path, tensors
 
 
+def test_predictive_loader_name_and_keywords(tmp_path):
+    """load_predictive_model: the reference's name, with context_factory for the BCTX tensors."""
+    path, tensors = _gated_package(tmp_path)
+    made = []
+
+    def context_factory(frame, *, stride, device):
+        made.append(len(frame))
+        return HostContext(frame, stride=stride, device=device)
+
+    model, receipt = serving.load_predictive_model(path, model_factory=GatedNet, device="cpu", context_factory=context_factory,
+                                                   predictive_factory=HostPredictive, log=lambda *_: None)
+    assert made and isinstance(model.down.context_weight, serving.PredictiveContextTensor)
+    assert np.array_equal(model.down.weight.view(torch.uint16).numpy(), tensors["down.weight"])
+    with pytest.raises(ValueError, match="not two different"):
+        serving.load_predictive_model(path, model_factory=GatedNet, device="cpu", context_factory=context_factory,
+                                      tensor_factory=HostContext)
+    plain = tmp_path / "plain"
+    pkg.write_package(plain, {"a.weight": tensors["up.weight"]})
+    with pytest.raises(serving.ContextServingError, match="no predictive candidates"):
+        serving.load_predictive_model(plain, model_factory=GatedNet, device="cpu")
+
+
 def test_loader_resolves_predictive_candidates(tmp_path):
     path, tensors = _gated_package(tmp_path)
     manifest, entries = pkg.read_manifest(path)
