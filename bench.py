@@ -232,7 +232,7 @@ def run_stack(args):
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: needs a ROCm GPU")
-    m = args.batch if args.batch != 1 else 64
+    m = args.batch or 64
     t0 = time.perf_counter()
 
     def coded(job):
@@ -351,7 +351,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--batch", type=int, default=1, help="activation rows; 1..2 run the fused GEMV (the headline figure is batch 1), more the fused GEMM")
+    ap.add_argument("--batch", type=int, default=None, help="activation rows (default 1 for mlp, the headline figure, and 64 for stack); 1..2 run the fused GEMV, more the fused GEMM")
     ap.add_argument("--segment", type=int, default=0, help="fused segment length (0 = automatic)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
@@ -370,6 +370,8 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this decode path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists)")
+    if args.workload == "mlp":
+        args.batch = args.batch or 1  # the stack defaults to 64
     if args.workload == "stack":
         if not 1 <= args.distinct_layers <= args.layers:
             sys.exit("bench.py: --distinct-layers must be between 1 and --layers")
