@@ -208,6 +208,14 @@ class HipContextTensor:
                 self._tiling(0)
             except _fused.FusedUnsupported as exc:
                 self.fused, self.fused_reason = None, str(exc)
+                return
+            # the tilings linear() uses are uploaded now, so that a first call launches and
+            # nothing else (it may be part of a graph capture)
+            try:
+                self._tiling(2)
+                self._gemm_tiling()
+            except _fused.FusedUnsupported:
+                pass  # reported by the call that needs it
 
     def clone(self):
         """A second resident copy of the same coded matrix: every device buffer is duplicated
