@@ -216,6 +216,102 @@ def cpu_baseline(frames, words_of, x_words, min_seconds=10.0, max_frames=12):
     return result
 
 
+def run_predictive(args):
+    """A 5120 x 17408 target coded (PPCX) against a reference that is the target plus N(0, 0.002)
+    noise; the reference is resident dense.  One step = the product of the coded target with
+    `--batch` activation rows (default 96 = 16 users x (5 draft tokens + 1), the verify shape):
+    the bins of the reference, then the fused GEMM (GEMV for one row)."""
+    import torch
+    from georefine_amd import bitexact_predictive_codec as ppcx
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs a ROCm GPU")
+    m = args.batch or 96
+    rows, cols = 5120, 17408
+    target = synth_weights(2, rows, cols)
+    noise = np.random.default_rng(5).normal(0, 0.002, size=target.shape).astype(np.float32)
+    ref = bf16_words((target.astype(np.uint32) << 16).view(np.float32) + noise)
+    del noise
+    t0 = time.perf_counter()
+    frame = ppcx.encode(target, ref)
+    t = HipPredictiveTensor(frame, ref, stride=1024, device="cuda:0")
+    if t.fused is None:
+        sys.exit(f"bench.py: the frame is not eligible for the fused kernels: {t.fused_reason}")
+    log(f"PPCX frame {len(frame)} B ({8 * len(frame) / target.size:.3f} bit/weight) mode {t.mode}; setup {time.perf_counter() - t0:.1f}s")
+    copies = [(t, torch.from_numpy(ref).view(torch.bfloat16).cuda())]
+    for _ in range(2):  # three targets and references in rotation: more bytes than the caches hold
+        other = HipPredictiveTensor(frame, ref, stride=1024, device="cuda:0")
+        copies.append((other, copies[0][1].clone()))
+    x = torch.from_numpy(bf16_words(np.random.default_rng(7).normal(0, 1, size=(m, cols)))).view(torch.bfloat16).cuda()
+
+    def step():
+        return [c.linear(r, x) for c, r in copies]
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    dense = torch.from_numpy(target).view(torch.bfloat16).cuda().float()
+    want = torch.nn.functional.linear(x.float(), dense)
+    scale = torch.nn.functional.linear(x.float().abs(), dense.abs())
+    got = copies[0][0].linear(copies[0][1], x, check=True).float()
+    if not bool((got - want).abs().le(1e-2 * want.abs().clamp_min(1e-3 * scale)).all()):
+        sys.exit("bench.py: the fused product is outside 1e-2 of the dense product")
+    del dense, want, scale, got
+    events = []
+    torch.cuda.synchronize()
+    wall0 = time.perf_counter()
+    for _ in range(args.steps):
+        for c, r in copies:
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            c.linear(r, x)
+            b.record()
+            events.append((a, b))
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - wall0
+    launch = "eager"
+    if args.graph:
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            graph.replay()
+            torch.cuda.synchronize()
+        except Exception as exc:
+            log(f"graph capture failed ({exc}); reporting the eager steps")
+        else:
+            wall0 = time.perf_counter()
+            for _ in range(args.steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - wall0
+            launch = "hip graph replay"
+    for c, _ in copies:
+        if c.error.item():
+            sys.exit("bench.py: decoder error word set")
+    ms_product = float(np.mean([a.elapsed_time(b) for a, b in events]))
+    # bytes one product has to touch once: the coded target, the dense reference, the bins
+    # plane written and read, activations and outputs
+    coded = t.resident_bytes
+    alg = coded + 2 * target.size + 2 * (target.size // 2) + m * cols * 2 + m * rows * 2
+    ms_per_step = wall / args.steps * 1e3
+    value = len(copies) * alg / (ms_per_step * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "compressed-weight decode-GEMV GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
+        "data": "synthetic",
+        "config": {"workload": f"PPCX target 5120x17408 against a dense reference (target + N(0, 0.002)), product with "
+                               f"{m} activation rows; three targets in rotation", "batch": m, "launch": launch},
+        "ms_per_product": round(ms_product, 4), "frame_bytes": len(frame), "resident_coded_bytes": coded,
+        "algorithmic_bytes_per_product": alg, "tok_s_equiv_rows_per_s": round(m * len(copies) / (ms_per_step * 1e-3), 1),
+        "roofline": {"bound": "hbm", "achieved": round(alg / (ms_product * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(alg / (ms_product * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "ppcx_bins_kernel + grf::fused_gemm_kernel<PpcxWalk, MT> (one product, HIP events)"},
+    }), flush=True)
+
+
 def run_stack(args):
     """Every coded linear of a 64-layer stack resident at once, one pass at batch 64.
 
@@ -361,9 +457,10 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB read + 128 MiB write elementwise kernel three times, so that a "
                          "counter profile of this command holds a kernel of known traffic to scale by")
-    ap.add_argument("--workload", choices=("mlp", "stack"), default="mlp",
+    ap.add_argument("--workload", choices=("mlp", "stack", "ppcx"), default="mlp",
                     help="mlp: the three MLP matrices of one layer (the headline); stack: every coded linear of "
-                         "--layers layers resident at once, one pass at batch 64 (or --batch)")
+                         "--layers layers resident at once, one pass at batch 64 (or --batch); ppcx: a predictive "
+                         "frame against its dense reference, product with 96 rows (or --batch)")
     ap.add_argument("--layers", type=int, default=64)
     ap.add_argument("--distinct-layers", type=int, default=1,
                     help="stack: layers encoded from their own seeds; the rest are device copies of these")
@@ -372,6 +469,8 @@ def main():
         sys.exit("bench.py: this decode path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists)")
     if args.workload == "mlp":
         args.batch = args.batch or 1  # the stack defaults to 64
+    if args.workload == "ppcx":
+        return run_predictive(args)
     if args.workload == "stack":
         if not 1 <= args.distinct_layers <= args.layers:
             sys.exit("bench.py: --distinct-layers must be between 1 and --layers")
