@@ -368,10 +368,20 @@ def run_stack(args):
     x = {k: torch.from_numpy(bf16_words(rng.normal(0, 1, size=(m, k)))).view(torch.bfloat16).cuda()
          for k in {c for _, c in LAYER.values()}}
 
+    # q, k, v read the same activations, gate and up too: with the matrix-core kernel their rows
+    # are put into operand order once per group
+    from georefine_amd.bitexact_context_gpu import PackedActivations
+    share = GEMV_UP_TO < m <= PackedActivations.MAX_ROWS and not args.no_shared_pack
+    groups = (("q", "k", "v"), ("o",), ("gate", "up"), ("down",))
+
     def step():
         for layer in layers:
-            for name, t in layer.items():
-                t.linear(x[LAYER[name][1]], batch_invariant=m > GEMV_UP_TO)
+            for group in groups:
+                xin = x[LAYER[group[0]][1]]
+                if share and len(group) > 1:
+                    xin = PackedActivations(xin)
+                for name in group:
+                    layer[name].linear(xin, batch_invariant=m > GEMV_UP_TO)
 
     for _ in range(args.warmup):
         step()
@@ -429,7 +439,8 @@ def run_stack(args):
         "config": {"workload": f"whole stack resident: {args.layers} layers x (q 5120->6144, k/v 5120->1024, o 6144->5120, "
                                f"gate/up 5120->17408, down 17408->5120), one pass through every coded linear at batch {m}",
                    "batch": m, "layers": args.layers, "distinct_layers": args.distinct_layers,
-                   "linears": args.layers * len(LAYER), "launch": launch},
+                   "linears": args.layers * len(LAYER), "launch": launch,
+                   "activations_packed": "once per q/k/v and gate/up group" if share else "per linear"},
         "dense_bf16_bytes": dense, "frame_bytes": frame_bytes, "resident_device_bytes": resident,
         "algorithmic_bytes_per_step": step_bytes,
         "effective_bf16_GBps": round(dense / (ms_per_step * 1e-3) / 1e9, 2),
@@ -462,6 +473,8 @@ def main():
                          "--layers layers resident at once, one pass at batch 64 (or --batch); ppcx: a predictive "
                          "frame against its dense reference, product with 96 rows (or --batch)")
     ap.add_argument("--layers", type=int, default=64)
+    ap.add_argument("--no-shared-pack", action="store_true",
+                    help="stack: pack the activations for every linear instead of once per group that shares them")
     ap.add_argument("--distinct-layers", type=int, default=1,
                     help="stack: layers encoded from their own seeds; the rest are device copies of these")
     args = ap.parse_args()

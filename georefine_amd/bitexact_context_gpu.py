@@ -113,6 +113,34 @@ def _device_stream(buffers, name, vocab, nctx):
     return s
 
 
+class PackedActivations:
+    """Activation rows copied once into the operand order of the matrix-core kernels, for
+    several coded matrices that take the same input (q/k/v, gate/up): ``gemm`` and
+    ``linear`` of the device tensors accept it in place of ``x``.  At most 128 rows."""
+
+    MAX_ROWS = 128
+
+    def __init__(self, x):
+        import torch
+        if x.dtype != torch.bfloat16 or not x.is_cuda:
+            raise ValueError("activations must be bfloat16 on the device")
+        self.lead, self.cols = tuple(x.shape[:-1]), x.shape[-1]
+        x2 = x.reshape(-1, self.cols)
+        self.rows = x2.shape[0]
+        if not 1 <= self.rows <= self.MAX_ROWS or self.cols % 16:
+            raise ValueError("1..128 rows of a width that is a multiple of 16")
+        if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 8:
+            x2 = x2.clone(memory_format=torch.contiguous_format)
+        lib = _native.hip()
+        size = lib.grf_gemm_workspace_bytes(self.cols, self.rows)
+        self.buffer = torch.empty(size, device=x.device, dtype=torch.uint8)
+        with torch.cuda.device(x.device):
+            status = lib.grf_pack_activations(x2.data_ptr(), x2.stride(0), self.rows, self.cols, self.buffer.data_ptr(),
+                                              size, torch.cuda.current_stream(x.device).cuda_stream)
+        if status:
+            raise base.CodecError(f"device launch failed ({status}): " + lib.grf_last_error().decode(errors="replace"))
+
+
 class HipContextTensor:
     """A BCTX-coded BF16 matrix resident on one MI355X."""
 
@@ -326,6 +354,22 @@ class HipContextTensor:
         y = torch.empty((x2.shape[0], self.shape[0]), device=self.device, dtype=torch.bfloat16)
         return x2, bias, y
 
+    def _packed_call(self, packed, bias, check):
+        """The GEMM on rows that were packed before (x == NULL in the C call)."""
+        import torch
+        if packed.cols != self.shape[1] or packed.buffer.device != self.device:
+            raise ValueError("packed activations of another width or device")
+        if bias is not None:
+            bias = bias.to(device=self.device, dtype=torch.bfloat16).contiguous()
+        y = torch.empty((packed.rows, self.shape[0]), device=self.device, dtype=torch.bfloat16)
+        if check:  # between checks the word keeps what earlier launches reported
+            self.error.zero_()
+        self._launch(self._lib.grf_bctx_gemm, ctypes.byref(self.fused), ctypes.byref(self._gemm_tiling()[0]), None, 0,
+                     packed.rows, y.data_ptr(), y.stride(0), bias.data_ptr() if bias is not None else None,
+                     packed.buffer.data_ptr(), packed.buffer.numel(), self.error.data_ptr())
+        self._check(check)
+        return y.reshape(*packed.lead, self.shape[0])
+
     def _fused_call(self, fn, tiling, x, bias, check, *, workspace=False):
         import torch
         lead = x.shape[:-1]
@@ -359,6 +403,8 @@ class HipContextTensor:
         a row's output bits are the same whatever else is in the batch."""
         if self.fused is None:
             raise base.CodecError("frame is not eligible for the fused kernels: " + self.fused_reason)
+        if isinstance(x, PackedActivations):
+            return self._packed_call(x, bias, check)
         return self._fused_call(self._lib.grf_bctx_gemm, self._gemm_tiling()[0], x, bias, check, workspace=True)
 
     def linear(self, x, bias=None, *, check=False, batch_invariant=False):
@@ -372,6 +418,8 @@ class HipContextTensor:
         it arrives in.  Frames the fused kernels cannot take are decoded on the device and
         multiplied densely.  ``check=True`` reads the error word back (a host sync)."""
         import torch.nn.functional as F
+        if isinstance(x, PackedActivations):  # packed for the matrix-core kernel, which is what it gets
+            return self.gemm(x, bias, check=check)
         m = math.prod(x.shape[:-1])
         if self.fused is None or (m > self.DENSE_ABOVE and not batch_invariant):
             return F.linear(x.to(self.device), self.decode(check=check), bias)

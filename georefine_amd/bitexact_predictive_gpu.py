@@ -264,6 +264,9 @@ class HipPredictiveTensor:
         ``batch_invariant`` asks for the fused GEMM throughout, whose rows do not depend on
         the batch.  Frames the tile walker cannot take are decoded and multiplied densely."""
         import torch
+        from .bitexact_context_gpu import PackedActivations
+        if isinstance(x, PackedActivations):  # packed for the matrix-core kernel, which is what it gets
+            return self._product(reference_bf16_device, x, bias, check, True)
         m = math.prod(x.shape[:-1])
         if self.fused is None or x.dtype != torch.bfloat16 or (m > self.DENSE_ABOVE and not batch_invariant):
             return torch.nn.functional.linear(x, self.decode(reference_bf16_device, check=check), bias)
@@ -284,16 +287,23 @@ class HipPredictiveTensor:
         import torch
         if self.fused is None:
             raise codec.CodecError("frame is not eligible for the fused kernels: " + str(self.fused_reason))
-        if x.dtype != torch.bfloat16:
-            raise ValueError("activation must be bfloat16")
-        m = math.prod(x.shape[:-1])
+        from .bitexact_context_gpu import PackedActivations
+        packed = x if isinstance(x, PackedActivations) else None
         ref = self._reference(reference_bf16_device)
-        x2 = x.reshape(-1, x.shape[-1]).to(self.device)
-        if x2.shape[-1] != self.shape[1]:
-            raise ValueError("activation width does not match the weight")
-        align = 4 if use_gemm else 2  # elements: the GEMM reads 8 bytes at a time, the GEMV 4
-        if x2.stride(-1) != 1 or x2.stride(0) % align or x2.data_ptr() % (2 * align):
-            x2 = x2.contiguous()
+        if packed is not None:
+            if not use_gemm or packed.cols != self.shape[1] or packed.buffer.device != self.device:
+                raise ValueError("packed activations go to the GEMM of a weight of their width on their device")
+            m, lead, x2 = packed.rows, packed.lead, None
+        else:
+            if x.dtype != torch.bfloat16:
+                raise ValueError("activation must be bfloat16")
+            m, lead = math.prod(x.shape[:-1]), tuple(x.shape[:-1])
+            x2 = x.reshape(-1, x.shape[-1]).to(self.device)
+            if x2.shape[-1] != self.shape[1]:
+                raise ValueError("activation width does not match the weight")
+            align = 4 if use_gemm else 2  # elements: the GEMM reads 8 bytes at a time, the GEMV 4
+            if x2.stride(-1) != 1 or x2.stride(0) % align or x2.data_ptr() % (2 * align):
+                x2 = x2.contiguous()
         if bias is not None:
             bias = bias.to(device=self.device, dtype=torch.bfloat16).contiguous()
         y = torch.empty((m, self.shape[0]), device=self.device, dtype=torch.bfloat16)
@@ -306,19 +316,22 @@ class HipPredictiveTensor:
                     extra = ()
                     if use_gemm:
                         fn, tiling = self._lib.grf_ppcx_gemm, self._tiling_for("gemm")[0]
-                        # transient: the activations in the matrix cores' operand order
-                        size = self._lib.grf_gemm_workspace_bytes(self.shape[1], m)
-                        packed = torch.empty(size, device=self.device, dtype=torch.uint8)
-                        extra = (packed.data_ptr(), size)
+                        if packed is not None:
+                            space = packed.buffer
+                        else:  # transient: the activations in the matrix cores' operand order
+                            space = torch.empty(self._lib.grf_gemm_workspace_bytes(self.shape[1], m),
+                                                device=self.device, dtype=torch.uint8)
+                        extra = (space.data_ptr(), space.numel())
                     else:
                         fn = self._lib.grf_ppcx_gemv
                         tiling = self._tiling_for(next(v for v in (1, 2, 4, 8) if v >= m))[0]
-                    status = fn(ctypes.byref(self.fused), ctypes.byref(tiling), bins.data_ptr(), x2.data_ptr(),
-                                x2.stride(0), m, y.data_ptr(), y.stride(0),
+                    status = fn(ctypes.byref(self.fused), ctypes.byref(tiling), bins.data_ptr(),
+                                x2.data_ptr() if x2 is not None else None, x2.stride(0) if x2 is not None else 0,
+                                m, y.data_ptr(), y.stride(0),
                                 bias.data_ptr() if bias is not None else None, *extra, self.error.data_ptr(),
                                 torch.cuda.current_stream(self.device).cuda_stream)
             self._status(status, check)
-        return y.reshape(*x.shape[:-1], self.shape[0])
+        return y.reshape(*lead, self.shape[0])
 
     def _status(self, status, check):
         if status:

@@ -286,6 +286,16 @@ static __global__ __launch_bounds__(256) void pack_activations_kernel(const uint
   xp[(size_t)c * m_pad + m] = v;
 }
 
+inline uint32_t gemm_tiles(uint32_t m_rows) { return m_rows <= 16 ? 1 : m_rows <= 32 ? 2 : m_rows <= 64 ? 4 : 8; }
+
+inline void launch_pack(const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint32_t cols, uint32_t m_pad, uint4 *xp,
+                        hipStream_t s) {
+  const uint32_t chunks = cols / 8;
+  const uint32_t pack_threads = (chunks + 1 + 7) / 8 * 8 * m_pad;  // the chunks and the chunk of zeros after them
+  hipLaunchKernelGGL(pack_activations_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, x, ldx, m_rows, m_pad,
+                     chunks, xp);
+}
+
 template <int MT>
 __device__ __forceinline__ void gemm_load_x(uint4 (&xa)[MT], const uint4 *xl) {
 #pragma unroll
@@ -433,10 +443,7 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
                      uint16_t *y, uint32_t ldy, const uint16_t *bias, uint4 *xp, int32_t *error, hipStream_t s) {
   const GemmLdsLayout L(f, g);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused GEMM: LDS demand exceeds 160 KiB");
-  const uint32_t chunks = f.cols / 8, m_pad = MT * 16;
-  const uint32_t pack_threads = (chunks + 1 + 7) / 8 * 8 * m_pad;  // the chunks and the chunk of zeros after them
-  hipLaunchKernelGGL(pack_activations_kernel, dim3((pack_threads + 255) / 256), dim3(256), 0, s, x, ldx, m_rows, m_pad,
-                     chunks, xp);
+  if (x) launch_pack(x, ldx, m_rows, f.cols, MT * 16, xp, s);  // else the caller packed these rows already
   constexpr auto kernel = [] {
     if constexpr (MT <= 4) return &fused_gemm_kernel<Walk, MT>;
     else return &fused_gemm_wide_kernel<Walk, MT>;
@@ -452,18 +459,21 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
 // bytes of the packed copy of the activations one launch needs
 inline size_t gemm_workspace_bytes(uint32_t cols, uint32_t m_rows) {
   const uint32_t m = m_rows > kMaxRowsPerLaunch ? kMaxRowsPerLaunch : m_rows;
-  const uint32_t tiles = m <= 16 ? 1 : m <= 32 ? 2 : m <= 64 ? 4 : 8;
-  return (size_t)(cols / 8 + 1) * tiles * 16 * 16;
+  return (size_t)(cols / 8 + 1) * gemm_tiles(m) * 16 * 16;
 }
 
 // y = x W^T (+ bias) for any number of activation rows, 128 per launch.  `workspace` holds
-// the packed activations of one launch; launches follow one another on the stream.
+// the packed activations of one launch; launches follow one another on the stream.  With
+// x == nullptr the workspace already holds these rows (pack_rows, same cols and m_rows).
 template <class Walk>
 int launch_gemm(const char *who, const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx,
                 uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
                 size_t workspace_bytes, int32_t *error, hipStream_t s) {
   if (!m_rows) return GRF_OK;
-  if (ldx < f.cols || ldy < f.rows || (ldx & 3) || ((uintptr_t)x & 7))
+  if (ldy < f.rows) return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": ldy is smaller than the row count");
+  if (!x && m_rows > kMaxRowsPerLaunch)
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": packed activations hold at most 128 rows");
+  if (x && (ldx < f.cols || (ldx & 3) || ((uintptr_t)x & 7)))
     return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) +
                                                 ": x must be 8-byte aligned with a leading dimension that is a multiple of 4");
   if (GemmShape(g).threads != g.threads || g.threads > (uint32_t)grf::kFusedMaxThreads)
@@ -474,7 +484,7 @@ int launch_gemm(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
   uint4 *xp = static_cast<uint4 *>(workspace);
   for (uint32_t m0 = 0; m0 < m_rows; m0 += kMaxRowsPerLaunch) {
     const uint32_t m = m_rows - m0 < kMaxRowsPerLaunch ? m_rows - m0 : kMaxRowsPerLaunch;
-    const uint16_t *xs = x + (size_t)m0 * ldx;
+    const uint16_t *xs = x ? x + (size_t)m0 * ldx : nullptr;
     uint16_t *ys = y + (size_t)m0 * ldy;
     int rc;
     if (m <= 16) rc = launch_gemm_rows<Walk, 1>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
@@ -483,6 +493,23 @@ int launch_gemm(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
     else rc = launch_gemm_rows<Walk, 8>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
     if (rc) return rc;
   }
+  return GRF_OK;
+}
+
+// The rows of x in operand order into `workspace`, for products of several matrices with
+// the same activations.
+inline int pack_rows(const char *who, const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint32_t cols, void *workspace,
+                     size_t workspace_bytes, hipStream_t s) {
+  if (!x || !m_rows || m_rows > kMaxRowsPerLaunch || !cols || (cols & 15))
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": 1..128 rows of a width that is a multiple of 16");
+  if (ldx < cols || (ldx & 3) || ((uintptr_t)x & 7))
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) +
+                                                ": x must be 8-byte aligned with a leading dimension that is a multiple of 4");
+  if (!workspace || ((uintptr_t)workspace & 15) || workspace_bytes < gemm_workspace_bytes(cols, m_rows))
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": workspace missing, misaligned or too small");
+  launch_pack(x, ldx, m_rows, cols, gemm_tiles(m_rows) * 16, static_cast<uint4 *>(workspace), s);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string(who) + ": " + hipGetErrorString(e));
   return GRF_OK;
 }
 

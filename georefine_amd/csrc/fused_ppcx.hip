@@ -242,7 +242,7 @@ int grf_ppcx_gemv(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, c
 int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const uint16_t *x,
                   uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
                   size_t workspace_bytes, int32_t *error, void *hip_stream) {
-  if (!x || !y || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemm: null argument");
+  if (!y || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemm: null argument");  // x may be null: packed rows
   grf_bctx_fused f;
   if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_gemm", f)) return rc;
   return grf::launch_gemm<PpcxWalk>("grf_ppcx_gemm", f, *tiling, x, ldx, m_rows, y, ldy, bias, workspace,

@@ -236,6 +236,13 @@ int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
                   uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
                   size_t workspace_bytes, int32_t *error, void *hip_stream);
 size_t grf_gemm_workspace_bytes(uint32_t cols, uint32_t m_rows);
+
+/* For several matrices that take the same activations (q/k/v, gate/up): writes 1..128 rows
+ * of x into workspace in operand order once; grf_bctx_gemm / grf_ppcx_gemm called with
+ * x == NULL, the same m_rows, a frame of this width and that workspace then multiply
+ * without packing again.  No reference counterpart. */
+int grf_pack_activations(const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint32_t cols, void *workspace,
+                         size_t workspace_bytes, void *hip_stream);
 uint32_t grf_bctx_gemm_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling);
 
 /* LDS bytes a launch needs for the given m_rows (0 for the store sink). */

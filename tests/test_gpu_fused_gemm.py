@@ -75,3 +75,41 @@ def test_gemm_checkpoint_mismatch_sets_error(oracle):
     x = torch.zeros(32, 512, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(codec.CodecError):
         t.gemm(x, check=True)
+
+
+def test_packed_activations_serve_several_matrices(oracle):
+    """Rows packed once multiply any matrix of their width, bit for bit what gemm(x) gives
+    (context and predictive frames), from strided and batched inputs, for every launch size."""
+    import torch
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd import bitexact_predictive_codec as ppcx
+    from georefine_amd.bitexact_context_gpu import HipContextTensor, PackedActivations
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
+    rng = np.random.default_rng(31)
+    a_words, b_words = weight_like(rng, 96, 768), weight_like(rng, 200, 768)
+    a = HipContextTensor(codec.encode(a_words), stride=1024, device="cuda:0")
+    b = HipContextTensor(codec.encode(b_words), stride=1024, device="cuda:0")
+    ref = bf16_words(words_to_float(b_words) + rng.normal(0, 0.002, b_words.shape).astype(np.float32))
+    p = HipPredictiveTensor(ppcx.encode(b_words, ref), ref, stride=1024, device="cuda:0")
+    ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
+    bias = torch.from_numpy(bf16_words(rng.normal(0, 1, size=200))).view(torch.bfloat16).cuda()
+    base = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(128, 2, 768)))).view(torch.bfloat16).cuda()
+    for rows in (1, 16, 17, 64, 100, 128):
+        x = base[:rows, 1, :]  # a strided view
+        packed = PackedActivations(x)
+        assert packed.rows == rows and packed.cols == 768
+        assert torch.equal(a.gemm(packed, check=True).view(torch.uint16), a.gemm(x).view(torch.uint16))
+        assert torch.equal(b.linear(packed, bias, check=True).view(torch.uint16), b.gemm(x, bias).view(torch.uint16))
+        assert torch.equal(p.linear(ref_dev, packed, bias, check=True).view(torch.uint16),
+                           p.gemm(ref_dev, x, bias).view(torch.uint16))
+    batched = PackedActivations(base[:5])  # [5, 2, 768] -> 10 rows
+    assert a.gemm(batched).shape == (5, 2, 96)
+    assert torch.equal(a.gemm(batched).view(torch.uint16), a.gemm(base[:5]).view(torch.uint16))
+    with pytest.raises(ValueError):
+        PackedActivations(torch.zeros(129, 768, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(ValueError):
+        PackedActivations(torch.zeros(4, 768, dtype=torch.float32, device="cuda"))
+    narrow = HipContextTensor(codec.encode(weight_like(rng, 32, 256)), stride=1024, device="cuda:0")
+    with pytest.raises(ValueError):
+        narrow.gemm(packed)
+
