@@ -343,7 +343,8 @@ def run_stack(args):
     t0 = time.perf_counter()
     base = {}
     for job in jobs:
-        t = HipContextTensor(frames[job], stride=1024, device="cuda:0")
+        # one segment length for every matrix, so that q/k/v and gate/up can share a launch
+        t = HipContextTensor(frames[job], stride=1024, device="cuda:0", fused_segment=64)
         if t.fused is None:
             sys.exit(f"bench.py: {job} is not eligible for the fused kernels: {t.fused_reason}")
         t._gemm_tiling()
@@ -368,20 +369,23 @@ def run_stack(args):
     x = {k: torch.from_numpy(bf16_words(rng.normal(0, 1, size=(m, k)))).view(torch.bfloat16).cuda()
          for k in {c for _, c in LAYER.values()}}
 
-    # q, k, v read the same activations, gate and up too: with the matrix-core kernel their rows
-    # are put into operand order once per group
-    from georefine_amd.bitexact_context_gpu import PackedActivations
-    share = GEMV_UP_TO < m <= PackedActivations.MAX_ROWS and not args.no_shared_pack
-    groups = (("q", "k", "v"), ("o",), ("gate", "up"), ("down",))
+    # q, k, v read the same activations, gate and up too: each group is one launch
+    from georefine_amd.bitexact_context_gpu import HipLinearGroup
+    names = (("q", "k", "v"), ("o",), ("gate", "up"), ("down",))
+    grouped = not args.no_groups
+    groups = [[HipLinearGroup([layer[n] for n in g]) if grouped and len(g) > 1 else None for g in names]
+              for layer in layers] if grouped else None
+    torch.cuda.synchronize()
 
     def step():
-        for layer in layers:
-            for group in groups:
-                xin = x[LAYER[group[0]][1]]
-                if share and len(group) > 1:
-                    xin = PackedActivations(xin)
-                for name in group:
-                    layer[name].linear(xin, batch_invariant=m > GEMV_UP_TO)
+        for i, layer in enumerate(layers):
+            for j, g in enumerate(names):
+                xin = x[LAYER[g[0]][1]]
+                if grouped and len(g) > 1:
+                    groups[i][j].linear(xin, batch_invariant=m > GEMV_UP_TO)
+                else:
+                    for name in g:
+                        layer[name].linear(xin, batch_invariant=m > GEMV_UP_TO)
 
     for _ in range(args.warmup):
         step()
@@ -440,7 +444,7 @@ def run_stack(args):
                                f"gate/up 5120->17408, down 17408->5120), one pass through every coded linear at batch {m}",
                    "batch": m, "layers": args.layers, "distinct_layers": args.distinct_layers,
                    "linears": args.layers * len(LAYER), "launch": launch,
-                   "activations_packed": "once per q/k/v and gate/up group" if share else "per linear"},
+                   "launches": "q/k/v and gate/up grouped" if grouped else "one per linear"},
         "dense_bf16_bytes": dense, "frame_bytes": frame_bytes, "resident_device_bytes": resident,
         "algorithmic_bytes_per_step": step_bytes,
         "effective_bf16_GBps": round(dense / (ms_per_step * 1e-3) / 1e9, 2),
@@ -473,8 +477,8 @@ def main():
                          "--layers layers resident at once, one pass at batch 64 (or --batch); ppcx: a predictive "
                          "frame against its dense reference, product with 96 rows (or --batch)")
     ap.add_argument("--layers", type=int, default=64)
-    ap.add_argument("--no-shared-pack", action="store_true",
-                    help="stack: pack the activations for every linear instead of once per group that shares them")
+    ap.add_argument("--no-groups", action="store_true",
+                    help="stack: one launch per linear instead of one for q/k/v and one for gate/up")
     ap.add_argument("--distinct-layers", type=int, default=1,
                     help="stack: layers encoded from their own seeds; the rest are device copies of these")
     args = ap.parse_args()

@@ -346,3 +346,33 @@ class FramePlan:
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
                                  n_tiles=n_tiles, piece_cap=cap), lds=lds)
+
+
+def plan_group(plans, m=None, gemm=False):
+    """Tilings of several frames of one width for one grouped launch: planned as if the
+    members' row classes belonged to one matrix (so a small member's tiles fill the
+    workgroup slots a large one leaves), with one thread count, lanes per row and rows per
+    tile for all; returns one tiling (as ``FramePlan.tiling``) per member."""
+    first = plans[0]
+    if any(pl.spr != first.spr or pl.seg_len != first.seg_len or pl.cols != first.cols for pl in plans):
+        raise FusedUnsupported("group members need one width and one segment length")
+    class_rows = np.concatenate([pl.class_rows for pl in plans])
+    cap_fn = lambda lanes: max(pl._cap(lanes) for pl in plans)
+    table = max(pl.table_bytes() for pl in plans)
+    if gemm:
+        lds_fn = lambda p_, r_, cap_: max(lds_bytes_gemm(pl.nc, pl.lognb, pl.tabn, p_, r_, cap_) for pl in plans)
+        threads, p, r, n_slabs, _, cap, lds = choose_gemm_tiling(first.spr, class_rows, cap_fn, lds_fn,
+                                                                 seg_len=first.seg_len, table_bytes=table)
+    else:
+        lds_fn = lambda p_, r_, cap_: max(lds_bytes(pl.nc, pl.lognb, pl.tabn, m, p_, first.seg_len, r_, cap_)
+                                          for pl in plans)
+        threads, p, r, n_slabs, _, cap, lds = choose_tiling(first.spr, class_rows, cap_fn, lds_fn,
+                                                            seg_len=first.seg_len, table_bytes=table)
+    tilings = []
+    for pl in plans:
+        tile_rows, tile_class = build_tiles(pl.row_class, pl.nr, r)
+        tilings.append(dict(tile_rows=tile_rows, tile_class=tile_class,
+                            scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
+                                         n_tiles=len(tile_class), piece_cap=cap), lds=lds))
+    return tilings
+

@@ -466,5 +466,114 @@ class HipContextTensor:
         return self._decode_blocks(blocks, check=check).reshape(*ids.shape, self.shape[1])
 
 
+class HipLinearGroup:
+    """Coded matrices of one width that take the same activations (q/k/v, gate/up), multiplied
+    in one launch: the members' tiles share the grid, so a small matrix fills the workgroup
+    slots a large one leaves, and the launch overhead is paid once.  The members stay usable
+    on their own.  They must have been indexed with one segment length
+    (``HipContextTensor(..., fused_segment=...)``)."""
+
+    GEMV_UP_TO = HipContextTensor.GEMV_UP_TO
+    DENSE_ABOVE = HipContextTensor.DENSE_ABOVE
+
+    def __init__(self, tensors):
+        import torch
+        self.tensors = list(tensors)
+        if not 1 <= len(self.tensors) <= 4:
+            raise ValueError("a group has 1..4 members")
+        first = self.tensors[0]
+        for t in self.tensors:
+            if t.fused is None:
+                raise base.CodecError("frame is not eligible for the fused kernels: " + t.fused_reason)
+            if t.shape[1] != first.shape[1] or t.device != first.device:
+                raise ValueError("group members need one width and one device")
+        self.device, self._lib = first.device, first._lib
+        self.error = torch.zeros((), device=self.device, dtype=torch.int32)
+        self._tilings = {}
+        for key in (1, 2, "gemm"):
+            self._tiling(key)  # raises FusedUnsupported when the members cannot share a tiling
+
+    def _tiling(self, key):
+        """Per member: (structure, device arrays) of the joint tiling for ``key`` (GEMV row
+        bucket 1/2/4/8, or "gemm")."""
+        import torch
+        if key not in self._tilings:
+            plans = [t._plan for t in self.tensors]
+            hosts = _fused.plan_group(plans, gemm=True) if key == "gemm" else _fused.plan_group(plans, m=key)
+            made = []
+            for host in hosts:
+                rows = torch.from_numpy(host["tile_rows"]).to(self.device)
+                classes = torch.from_numpy(host["tile_class"]).to(self.device)
+                g = _hip_abi.GrfFusedTiling()
+                g.tile_rows, g.tile_class = rows.data_ptr(), classes.data_ptr()
+                for name, value in host["scalars"].items():
+                    setattr(g, name, value)
+                made.append((g, rows, classes, dict(host["scalars"], lds=host["lds"])))
+            self._tilings[key] = made
+        return self._tilings[key]
+
+    def _arrays(self, tilings, outs, biases):
+        n = len(self.tensors)
+        frames = (ctypes.POINTER(_hip_abi.GrfBctxFused) * n)(*[ctypes.pointer(t.fused) for t in self.tensors])
+        tiles = (ctypes.POINTER(_hip_abi.GrfFusedTiling) * n)(*[ctypes.pointer(g[0]) for g in tilings])
+        ys = (ctypes.c_void_p * n)(*[y.data_ptr() for y in outs])
+        ldy = (ctypes.c_uint32 * n)(*[y.stride(0) for y in outs])
+        bias = (ctypes.c_void_p * n)(*[b.data_ptr() if b is not None else None for b in biases])
+        return frames, tiles, ys, ldy, bias
+
+    def linear(self, x, biases=None, *, check=False, batch_invariant=False):
+        """[x @ W.T (+ bias) for every member]; x is BF16 [..., K] or ``PackedActivations``.
+        Row counts are routed as in ``HipContextTensor.linear``: the GEMV to 2 rows, the
+        matrix-core kernel to 128 (every count with ``batch_invariant``), the members' own
+        decode + matmul above."""
+        import torch
+        n = len(self.tensors)
+        biases = list(biases) if biases is not None else [None] * n
+        if len(biases) != n:
+            raise ValueError("one bias (or None) per member")
+        packed = x if isinstance(x, PackedActivations) else None
+        m = packed.rows if packed else math.prod(x.shape[:-1])
+        lead = packed.lead if packed else tuple(x.shape[:-1])
+        cols = self.tensors[0].shape[1]
+        if packed is None and m > self.DENSE_ABOVE and not batch_invariant:
+            return [t.linear(x, b, check=check) for t, b in zip(self.tensors, biases)]
+        if packed is not None:
+            if packed.cols != cols or packed.buffer.device != self.device:
+                raise ValueError("packed activations of another width or device")
+            x2 = None
+        else:
+            if x.dtype != torch.bfloat16 or x.shape[-1] != cols:
+                raise ValueError("activation must be bfloat16 with the weights' input width")
+            x2 = x.reshape(-1, cols).to(self.device)
+            if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 8:
+                x2 = x2.clone(memory_format=torch.contiguous_format)
+        biases = [b.to(device=self.device, dtype=torch.bfloat16).contiguous() if b is not None else None for b in biases]
+        outs = [torch.empty((m, t.shape[0]), device=self.device, dtype=torch.bfloat16) for t in self.tensors]
+        if m:
+            if check:
+                self.error.zero_()
+            use_gemm = packed is not None or batch_invariant or m > self.GEMV_UP_TO
+            with torch.cuda.device(self.device):
+                stream = torch.cuda.current_stream(self.device).cuda_stream
+                if use_gemm:
+                    arrays = self._arrays(self._tiling("gemm"), outs, biases)
+                    space = packed.buffer if packed else torch.empty(
+                        self._lib.grf_gemm_workspace_bytes(cols, m), device=self.device, dtype=torch.uint8)
+                    status = self._lib.grf_bctx_gemm_group(
+                        n, arrays[0], arrays[1], x2.data_ptr() if x2 is not None else None,
+                        x2.stride(0) if x2 is not None else 0, m, arrays[2], arrays[3], arrays[4], space.data_ptr(),
+                        space.numel(), self.error.data_ptr(), stream)
+                else:
+                    arrays = self._arrays(self._tiling(next(v for v in (1, 2, 4, 8) if v >= m)), outs, biases)
+                    status = self._lib.grf_bctx_gemv_group(n, arrays[0], arrays[1], x2.data_ptr(), x2.stride(0), m,
+                                                           arrays[2], arrays[3], arrays[4], self.error.data_ptr(), stream)
+            if status:
+                raise base.CodecError(f"device launch failed ({status}): "
+                                      + self._lib.grf_last_error().decode(errors="replace"))
+            if check and self.error.item() != 0:
+                raise base.CodecError("HIP decoder checkpoint mismatch")
+        return [y.reshape(*lead, t.shape[0]) for y, t in zip(outs, self.tensors)]
+
+
 # The loaders name the class they expect; keep that name importable.
 CudaContextTensor = HipContextTensor

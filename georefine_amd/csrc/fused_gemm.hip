@@ -27,4 +27,23 @@ int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
                                             workspace_bytes, error, (hipStream_t)hip_stream);
 }
 
+int grf_bctx_gemv_group(uint32_t n, const grf_bctx_fused *const *frames, const grf_fused_tiling *const *tilings,
+                        const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint16_t *const *y, const uint32_t *ldy,
+                        const uint16_t *const *bias, int32_t *error, void *hip_stream) {
+  if (!error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemv_group: null argument");
+  const grf::GroupSpec spec{n, frames, tilings, y, ldy, bias};
+  return grf::launch_gemv_group<grf::SegmentWalk>("grf_bctx_gemv_group", spec, x, ldx, m_rows, error,
+                                                  (hipStream_t)hip_stream);
+}
+
+int grf_bctx_gemm_group(uint32_t n, const grf_bctx_fused *const *frames, const grf_fused_tiling *const *tilings,
+                        const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint16_t *const *y, const uint32_t *ldy,
+                        const uint16_t *const *bias, void *workspace, size_t workspace_bytes, int32_t *error,
+                        void *hip_stream) {
+  if (!error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemm_group: null argument");
+  const grf::GroupSpec spec{n, frames, tilings, y, ldy, bias};
+  return grf::launch_gemm_group<grf::SegmentWalk>("grf_bctx_gemm_group", spec, x, ldx, m_rows, workspace,
+                                                  workspace_bytes, error, (hipStream_t)hip_stream);
+}
+
 }  // extern "C"

@@ -24,6 +24,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <atomic>
 #include <string>
 
@@ -73,16 +74,14 @@ __device__ __forceinline__ uint16_t round_bf16(float v) {
 // tiling (row tile * R + r of a compact [n_tiles * R][cols] output: a gather of rows).
 enum Sink : int { kDot = 0, kStore = 1, kGather = 2 };
 
+// One workgroup's walk over tile `tile` of a frame.
 template <class Walk, int M, int SINK>
-__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_bctx_fused f, grf_fused_tiling g,
-                                                                            const uint16_t *x, uint32_t ldx,
-                                                                            uint16_t *y, uint32_t ldy,
-                                                                            const uint16_t *bias, uint16_t *out,
-                                                                            int32_t *error) {
-  extern __shared__ __align__(16) uint8_t lds[];
+__device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fused &f, const grf_fused_tiling &g,
+                                                const uint16_t *x, uint32_t ldx, uint16_t *y, uint32_t ldy,
+                                                const uint16_t *bias, uint16_t *out, int32_t *error, uint32_t tile) {
   constexpr bool STORE = SINK != kDot;
   const FusedLdsLayout L(f, g, STORE ? 0 : M);
-  const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
@@ -185,6 +184,48 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_b
     }
   }
   if (bad) atomicOr(error, (int)bad);
+}
+
+template <class Walk, int M, int SINK>
+__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_bctx_fused f, grf_fused_tiling g,
+                                                                            const uint16_t *x, uint32_t ldx,
+                                                                            uint16_t *y, uint32_t ldy,
+                                                                            const uint16_t *bias, uint16_t *out,
+                                                                            int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  fused_walk_body<Walk, M, SINK>(lds, f, g, x, ldx, y, ldy, bias, out, error, blockIdx.x);
+}
+
+// Several frames of one width in one launch (q/k/v, gate/up): the grid is the tiles of the
+// members one after the other, every member with its own tiling, output and bias.  The
+// tilings share one thread count; a member's rows see exactly the arithmetic of a launch of
+// their own with that tiling.
+constexpr uint32_t kMaxGroup = 4;
+struct FusedGroup {
+  grf_bctx_fused f[kMaxGroup];
+  grf_fused_tiling g[kMaxGroup];
+  uint16_t *y[kMaxGroup];
+  const uint16_t *bias[kMaxGroup];
+  uint32_t ldy[kMaxGroup];
+  uint32_t first_tile[kMaxGroup + 1];  // first_tile[n] = tiles of the whole launch
+  uint32_t n;
+};
+
+__device__ __forceinline__ uint32_t group_member(const FusedGroup &a, uint32_t block) {
+  uint32_t i = 0;
+#pragma unroll
+  for (uint32_t k = 1; k < kMaxGroup; ++k)
+    if (k < a.n && block >= a.first_tile[k]) i = k;
+  return i;
+}
+
+template <class Walk, int M>
+__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_group_kernel(FusedGroup a, const uint16_t *x,
+                                                                                  uint32_t ldx, int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t i = group_member(a, blockIdx.x);
+  fused_walk_body<Walk, M, kDot>(lds, a.f[i], a.g[i], x, ldx, a.y[i], a.ldy[i], a.bias[i], nullptr, error,
+                                 blockIdx.x - a.first_tile[i]);
 }
 
 template <class Walk, int M, int SINK>
@@ -321,10 +362,10 @@ __device__ __forceinline__ void gemm_contract(float4v (&acc)[MT], const uint4 (&
 template <class Walk, int MT>
 __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fused &f, const grf_fused_tiling &g,
                                                 const uint4 *xp, uint32_t m_rows, uint16_t *y, uint32_t ldy,
-                                                const uint16_t *bias, int32_t *error) {
+                                                const uint16_t *bias, int32_t *error, uint32_t tile) {
   const GemmLdsLayout L(f, g);
   const GemmShape shape(g);
-  const uint32_t tid = threadIdx.x, nthreads = blockDim.x, tile = blockIdx.x;
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
@@ -424,7 +465,7 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_
     grf_bctx_fused f, grf_fused_tiling g, const uint4 *xp, uint32_t m_rows, uint16_t *y, uint32_t ldy,
     const uint16_t *bias, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  fused_gemm_body<Walk, MT>(lds, f, g, xp, m_rows, y, ldy, bias, error);
+  fused_gemm_body<Walk, MT>(lds, f, g, xp, m_rows, y, ldy, bias, error, blockIdx.x);
 }
 
 // Eight activation tiles: the accumulators and operands alone take 64 registers, so fewer
@@ -435,7 +476,25 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_wide_kernel(
                                                                                  uint16_t *y, uint32_t ldy,
                                                                                  const uint16_t *bias, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  fused_gemm_body<Walk, MT>(lds, f, g, xp, m_rows, y, ldy, bias, error);
+  fused_gemm_body<Walk, MT>(lds, f, g, xp, m_rows, y, ldy, bias, error, blockIdx.x);
+}
+
+template <class Walk, int MT>
+__global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_gemm_group_kernel(
+    FusedGroup a, const uint4 *xp, uint32_t m_rows, int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t i = group_member(a, blockIdx.x);
+  fused_gemm_body<Walk, MT>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], error,
+                            blockIdx.x - a.first_tile[i]);
+}
+
+template <class Walk, int MT>
+__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_wide_group_kernel(FusedGroup a, const uint4 *xp,
+                                                                                       uint32_t m_rows, int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t i = group_member(a, blockIdx.x);
+  fused_gemm_body<Walk, MT>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], error,
+                            blockIdx.x - a.first_tile[i]);
 }
 
 template <class Walk, int MT>
@@ -510,6 +569,128 @@ inline int pack_rows(const char *who, const uint16_t *x, uint32_t ldx, uint32_t 
   launch_pack(x, ldx, m_rows, cols, gemm_tiles(m_rows) * 16, static_cast<uint4 *>(workspace), s);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string(who) + ": " + hipGetErrorString(e));
+  return GRF_OK;
+}
+
+// ---------------------------------------------------------------- grouped launches
+
+struct GroupSpec {  // the arrays of a grouped entry point
+  uint32_t n;
+  const grf_bctx_fused *const *frames;
+  const grf_fused_tiling *const *tilings;
+  uint16_t *const *y;
+  const uint32_t *ldy;
+  const uint16_t *const *bias;  // may be null, and so may any of its elements
+};
+
+inline int build_group(const char *who, const GroupSpec &spec, bool gemm, FusedGroup &a) {
+  auto bad = [&](const char *why) { return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": " + why); };
+  if (spec.n < 1 || spec.n > kMaxGroup) return bad("a group has 1..4 members");
+  if (!spec.frames || !spec.tilings || !spec.y || !spec.ldy) return bad("null argument");
+  a = FusedGroup{};
+  a.n = spec.n;
+  for (uint32_t i = 0; i < spec.n; ++i) {
+    if (!spec.frames[i] || !spec.tilings[i] || !spec.y[i]) return bad("null member");
+    const grf_bctx_fused &f = *spec.frames[i];
+    const grf_fused_tiling &g = *spec.tilings[i];
+    if (int rc = grf::check_fused_frame(f, g, who)) return rc;
+    if (f.cols != spec.frames[0]->cols) return bad("members must have one width");
+    if (g.threads != spec.tilings[0]->threads) return bad("member tilings must share one thread count");
+    if (gemm && GemmShape(g).threads != g.threads)
+      return bad("tiling threads must be 64 x ceil(rows_per_tile / 16) x ceil(lanes_per_row / 4)");
+    if (spec.ldy[i] < f.rows) return bad("ldy is smaller than the row count");
+    a.f[i] = f;
+    a.g[i] = g;
+    a.y[i] = spec.y[i];
+    a.ldy[i] = spec.ldy[i];
+    a.bias[i] = spec.bias ? spec.bias[i] : nullptr;
+    a.first_tile[i + 1] = a.first_tile[i] + g.n_tiles;
+  }
+  return GRF_OK;
+}
+
+template <class Walk, int M>
+int launch_walk_group(const FusedGroup &a, const uint16_t *x, uint32_t ldx, int32_t *error, hipStream_t s) {
+  uint32_t lds = 0;
+  for (uint32_t i = 0; i < a.n; ++i) lds = std::max(lds, FusedLdsLayout(a.f[i], a.g[i], M).total);
+  if (lds > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
+  constexpr auto kernel = &fused_walk_group_kernel<Walk, M>;
+  if (lds > 64 * 1024)
+    if (int rc = allow_full_lds<kernel>()) return rc;
+  hipLaunchKernelGGL(kernel, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, a, x, ldx, error);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
+  return GRF_OK;
+}
+
+// y_i = x W_i^T (+ bias_i) for the members of a group, 1..8 activation rows, one launch
+template <class Walk>
+int launch_gemv_group(const char *who, const GroupSpec &spec, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
+                      int32_t *error, hipStream_t s) {
+  FusedGroup a;
+  if (int rc = build_group(who, spec, false, a)) return rc;
+  if (m_rows < 1 || m_rows > 8) return grf::set_error(GRF_UNSUPPORTED, std::string(who) + ": 1 <= m_rows <= 8");
+  if (!x || ldx < a.f[0].cols || (ldx & 1) || ((uintptr_t)x & 3))
+    return grf::set_error(GRF_BAD_ARGUMENT,
+                          std::string(who) + ": x must be 4-byte aligned with an even leading dimension");
+  switch (m_rows) {
+    case 1: return launch_walk_group<Walk, 1>(a, x, ldx, error, s);
+    case 2: return launch_walk_group<Walk, 2>(a, x, ldx, error, s);
+    case 3: return launch_walk_group<Walk, 3>(a, x, ldx, error, s);
+    case 4: return launch_walk_group<Walk, 4>(a, x, ldx, error, s);
+    case 5: return launch_walk_group<Walk, 5>(a, x, ldx, error, s);
+    case 6: return launch_walk_group<Walk, 6>(a, x, ldx, error, s);
+    case 7: return launch_walk_group<Walk, 7>(a, x, ldx, error, s);
+    default: return launch_walk_group<Walk, 8>(a, x, ldx, error, s);
+  }
+}
+
+template <class Walk, int MT>
+int launch_gemm_group_rows(const FusedGroup &a, uint32_t m_rows, const uint4 *xp, int32_t *error, hipStream_t s) {
+  uint32_t lds = 0;
+  for (uint32_t i = 0; i < a.n; ++i) lds = std::max(lds, GemmLdsLayout(a.f[i], a.g[i]).total);
+  if (lds > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused GEMM: LDS demand exceeds 160 KiB");
+  constexpr auto kernel = [] {
+    if constexpr (MT <= 4) return &fused_gemm_group_kernel<Walk, MT>;
+    else return &fused_gemm_wide_group_kernel<Walk, MT>;
+  }();
+  if (lds > 64 * 1024)
+    if (int rc = allow_full_lds<kernel>()) return rc;
+  hipLaunchKernelGGL(kernel, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, a, xp, m_rows, error);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused GEMM: ") + hipGetErrorString(e));
+  return GRF_OK;
+}
+
+// the same for any number of rows on the matrix cores, 128 rows per launch; x == nullptr:
+// the workspace already holds the rows
+template <class Walk>
+int launch_gemm_group(const char *who, const GroupSpec &spec, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
+                      void *workspace, size_t workspace_bytes, int32_t *error, hipStream_t s) {
+  FusedGroup a;
+  if (int rc = build_group(who, spec, true, a)) return rc;
+  if (!m_rows) return GRF_OK;
+  const uint32_t cols = a.f[0].cols;
+  if (!x && m_rows > kMaxRowsPerLaunch)
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": packed activations hold at most 128 rows");
+  if (x && (ldx < cols || (ldx & 3) || ((uintptr_t)x & 7)))
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) +
+                                                ": x must be 8-byte aligned with a leading dimension that is a multiple of 4");
+  if (!workspace || ((uintptr_t)workspace & 15) || workspace_bytes < gemm_workspace_bytes(cols, m_rows))
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": workspace missing, misaligned or too small");
+  uint4 *xp = static_cast<uint4 *>(workspace);
+  for (uint32_t m0 = 0; m0 < m_rows; m0 += kMaxRowsPerLaunch) {
+    const uint32_t m = m_rows - m0 < kMaxRowsPerLaunch ? m_rows - m0 : kMaxRowsPerLaunch;
+    FusedGroup part = a;
+    for (uint32_t i = 0; i < a.n; ++i) part.y[i] = a.y[i] + (size_t)m0 * a.ldy[i];
+    if (x) launch_pack(x + (size_t)m0 * ldx, ldx, m, cols, gemm_tiles(m) * 16, xp, s);
+    int rc;
+    if (m <= 16) rc = launch_gemm_group_rows<Walk, 1>(part, m, xp, error, s);
+    else if (m <= 32) rc = launch_gemm_group_rows<Walk, 2>(part, m, xp, error, s);
+    else if (m <= 64) rc = launch_gemm_group_rows<Walk, 4>(part, m, xp, error, s);
+    else rc = launch_gemm_group_rows<Walk, 8>(part, m, xp, error, s);
+    if (rc) return rc;
+  }
   return GRF_OK;
 }
 

@@ -245,6 +245,21 @@ int grf_pack_activations(const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint3
                          size_t workspace_bytes, void *hip_stream);
 uint32_t grf_bctx_gemm_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling);
 
+/* Up to four coded matrices of one width that take the same activations (q/k/v, gate/up) in
+ * one launch: y[i] = x W_i^T (+ bias[i]).  The grid is the members' tiles one after the
+ * other, so small members fill the machine beside large ones; every member keeps its own
+ * tiling, and a member's rows see exactly the arithmetic of grf_bctx_gemv / grf_bctx_gemm
+ * with that tiling.  The tilings must share one thread count.  bias may be NULL, and so
+ * may any bias[i]; the other arguments are those of the single-matrix entry points (for
+ * the GEMM: x == NULL for rows packed by grf_pack_activations).  No reference counterpart. */
+int grf_bctx_gemv_group(uint32_t n, const grf_bctx_fused *const *frames, const grf_fused_tiling *const *tilings,
+                        const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint16_t *const *y, const uint32_t *ldy,
+                        const uint16_t *const *bias, int32_t *error, void *hip_stream);
+int grf_bctx_gemm_group(uint32_t n, const grf_bctx_fused *const *frames, const grf_fused_tiling *const *tilings,
+                        const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint16_t *const *y, const uint32_t *ldy,
+                        const uint16_t *const *bias, void *workspace, size_t workspace_bytes, int32_t *error,
+                        void *hip_stream);
+
 /* LDS bytes a launch needs for the given m_rows (0 for the store sink). */
 uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint32_t m_rows);
 

@@ -96,7 +96,8 @@ def test_attention_matrices_gemm_rows_do_not_depend_on_batch(name, shape):
 def test_whole_stack_resident_one_pass_at_batch_64():
     """64 layers x (q, k, v, o, gate, up, down) resident at once, one pass through every coded
     linear at batch 64.  One layer is encoded; the other 63 are device copies with buffers of
-    their own, so the pass runs 448 launches over about 30 GB of coded weights.  Every copy
+    their own, so the pass covers about 30 GB of coded weights in 256 launches (q/k/v share
+    one, gate/up another).  Every copy
     must give the first layer's rows bit for bit, and the first layer's rows agree with the
     dense product of its decoded weights."""
     import torch
@@ -112,7 +113,8 @@ def test_whole_stack_resident_one_pass_at_batch_64():
 
     with ThreadPoolExecutor(max_workers=7) as pool:
         frames = dict(pool.map(coded, enumerate(shapes.items())))
-    first = {name: HipContextTensor(frames[name], stride=1024, device="cuda:0") for name in shapes}
+    # one segment length throughout, so that q/k/v and gate/up can share a launch
+    first = {name: HipContextTensor(frames[name], stride=1024, device="cuda:0", fused_segment=64) for name in shapes}
     assert all(t.fused is not None for t in first.values())
     layers = [first] + [{name: t.clone() for name, t in first.items()} for _ in range(63)]
     dense_bytes = 64 * sum(2 * r * c for r, c in shapes.values())
@@ -122,7 +124,16 @@ def test_whole_stack_resident_one_pass_at_batch_64():
     rng = np.random.default_rng(11)
     x = {k: torch.from_numpy(bf16_words(rng.normal(0, 1, size=(64, k)))).view(torch.bfloat16).cuda()
          for k in (5120, 6144, 17408)}
-    outs = [{name: t.linear(x[shapes[name][1]], check=False) for name, t in layer.items()} for layer in layers]
+    from georefine_amd.bitexact_context_gpu import HipLinearGroup
+    outs = []
+    for layer in layers:  # q/k/v in one launch, gate/up in one launch, o and down on their own
+        qkv = HipLinearGroup([layer[n] for n in ("q", "k", "v")])
+        mlp = HipLinearGroup([layer[n] for n in ("gate", "up")])
+        out = dict(zip(("q", "k", "v"), qkv.linear(x[5120])))
+        out.update(zip(("gate", "up"), mlp.linear(x[5120])))
+        out["o"], out["down"] = layer["o"].linear(x[6144]), layer["down"].linear(x[17408])
+        outs.append(out)
+        assert qkv.error.item() == 0 and mlp.error.item() == 0
     torch.cuda.synchronize()
     for layer in layers:
         for t in layer.values():
