@@ -2,11 +2,12 @@
 """Headline benchmark: fused decode-GEMV at batch 1 on Qwen-27B-like MLP shapes.
 
 One step = one pass of the hot path over the three coded MLP matrices of a layer
-(gate and up: 17408x5120, down: 5120x17408), i.e. three fused decode-GEMV
-launches on seeded synthetic BF16 weights (N(0,0.02) with per-row log-normal(0,0.5)
-scale and 0.1% outliers at 10x) against an N(0,1) BF16 activation vector.  The
-three matrices together are ~354 MB coded, more than L2 + Infinity Cache, so
-every step streams its compressed bytes from HBM.
+(gate and up: 17408x5120, down: 5120x17408) on seeded synthetic BF16 weights
+(N(0,0.02) with per-row log-normal(0,0.5) scale and 0.1% outliers at 10x) against
+an N(0,1) BF16 activation vector: gate and up take the same vector and run as one
+fused decode-GEMV launch, down as another (--no-groups: three launches).  The three
+matrices together are ~354 MB coded, more than L2 + Infinity Cache, so every step
+streams its compressed bytes from HBM.
 
 Prints ONE JSON line: metric = compressed bytes consumed per second (GB/s), with
 the achieved fraction of the 8 TB/s HBM roofline for the dominant kernel and a
@@ -460,8 +461,9 @@ def run_stack(args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=50, help="untimed steps first (the clocks of an idle GPU take "
+                                                         "some milliseconds of work to come up)")
     ap.add_argument("--batch", type=int, default=None, help="activation rows (default 1 for mlp, the headline figure, and 64 for stack); 1..2 run the fused GEMV, more the fused GEMM")
     ap.add_argument("--segment", type=int, default=0, help="fused segment length (0 = automatic)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -478,7 +480,8 @@ def main():
                          "frame against its dense reference, product with 96 rows (or --batch)")
     ap.add_argument("--layers", type=int, default=64)
     ap.add_argument("--no-groups", action="store_true",
-                    help="stack: one launch per linear instead of one for q/k/v and one for gate/up")
+                    help="one launch per linear instead of one for the matrices that take the same activations "
+                         "(gate/up; in the stack also q/k/v)")
     ap.add_argument("--distinct-layers", type=int, default=1,
                     help="stack: layers encoded from their own seeds; the rest are device copies of these")
     args = ap.parse_args()
@@ -529,11 +532,19 @@ def main():
     x_words = {k: bf16_words(rng.normal(0, 1, size=(m, k))) for k in (5120, 17408)}
     x = {k: torch.from_numpy(v).view(torch.bfloat16).cuda() for k, v in x_words.items()}
 
+    # the launches of a step: gate and up take the same activations and share one launch
+    from georefine_amd.bitexact_context_gpu import HipLinearGroup
+    units = []  # (label, member names, callable)
+    if not args.no_groups and "gate" in names and "up" in names:
+        pair = HipLinearGroup([tensors["gate"], tensors["up"]])
+        units.append(("gate+up", ["gate", "up"], lambda: pair.linear(x[5120])))
+        log(f"gate+up: one launch, tiling {pair._tiling(m if m <= GEMV_UP_TO else 'gemm')[0][3]}")
+    for name in names:
+        if not any(name in u[1] for u in units):
+            units.append((name, [name], lambda name=name: tensors[name].linear(x[SHAPES[name][1]])))
+
     def step():
-        outs = []
-        for name in names:
-            outs.append(tensors[name].linear(x[SHAPES[name][1]]))
-        return outs
+        return [run() for _, _, run in units]
 
     for _ in range(args.warmup):
         step()
@@ -543,14 +554,14 @@ def main():
             sys.exit(f"bench.py: decoder error word set for {name}")
 
     # per-launch durations with events on the stream the kernels run on
-    starts = [[torch.cuda.Event(enable_timing=True) for _ in names] for _ in range(args.steps)]
-    ends = [[torch.cuda.Event(enable_timing=True) for _ in names] for _ in range(args.steps)]
+    starts = [[torch.cuda.Event(enable_timing=True) for _ in units] for _ in range(args.steps)]
+    ends = [[torch.cuda.Event(enable_timing=True) for _ in units] for _ in range(args.steps)]
     torch.cuda.synchronize()
     wall0 = time.perf_counter()
     for s in range(args.steps):
-        for j, name in enumerate(names):
+        for j, (_, _, run) in enumerate(units):
             starts[s][j].record()
-            tensors[name].linear(x[SHAPES[name][1]])
+            run()
             ends[s][j].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - wall0
@@ -584,9 +595,14 @@ def main():
             torch.add(src, 1, out=dst)
         torch.cuda.synchronize()
 
-    per_kernel_ms = {name: float(np.mean([starts[s][j].elapsed_time(ends[s][j]) for s in range(args.steps)]))
-                     for j, name in enumerate(names)}
-    alg = {name: algorithmic_bytes(tensors[name], m) for name in names}
+    per_kernel_ms = {label: float(np.mean([starts[s][j].elapsed_time(ends[s][j]) for s in range(args.steps)]))
+                     for j, (label, _, _) in enumerate(units)}
+    alg = {}
+    for label, members, _ in units:
+        parts = [algorithmic_bytes(tensors[n_], m) for n_ in members]
+        alg[label] = {k: sum(p_[k] for p_ in parts) for k in parts[0]}
+        if len(members) > 1:  # the members read one x
+            alg[label]["total"] -= (len(members) - 1) * m * SHAPES[members[0]][1] * 2
     step_bytes = sum(a["total"] for a in alg.values())
     dense_bytes = sum(2 * SHAPES[n][0] * SHAPES[n][1] for n in names)
     ms_per_step = wall / args.steps * 1e3
@@ -595,12 +611,18 @@ def main():
 
     # HBM bytes per launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE (scaled by a copy
     # kernel of known size); a recorded figure, bench.py cannot read hardware counters itself
+    dom = max(per_kernel_ms, key=lambda n_: per_kernel_ms[n_])
+    grouped = "+" in dom
+    if m <= GEMV_UP_TO:
+        kernel = f"grf::fused_walk_group_kernel<grf::SegmentWalk, {m}>" if grouped else f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>"
+    else:
+        kernel = "grf::fused_gemm_group_kernel<grf::SegmentWalk, MT>" if grouped else "grf::fused_gemm_kernel<grf::SegmentWalk, MT>"
     traffic = None
     recorded = ROOT / "profiles" / "fused_gemv_m1_qwen27b_mlp_traffic.json"
     if m == 1 and recorded.exists():
-        traffic = json.loads(recorded.read_text()).get("traffic_bytes_per_launch")
-
-    dom = max(names, key=lambda n_: per_kernel_ms[n_])
+        per_kernel_traffic = json.loads(recorded.read_text()).get("traffic_bytes_per_launch")
+        if isinstance(per_kernel_traffic, dict):  # by kernel name
+            traffic = per_kernel_traffic.get(kernel.split("<")[0].split("::")[-1])
     achieved = alg[dom]["total"] / (per_kernel_ms[dom] * 1e-3) / 1e9
     result = {
         "metric": "compressed-weight decode-GEMV GB/s",
@@ -617,7 +639,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": "fused decode-" + ("GEMV" if m <= GEMV_UP_TO else "GEMM") + ", batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
                                "BCTX (16,4) frames, residuals resident in packed 6-bit form" % m,
-                   "batch": m, "matrices": names,
+                   "batch": m, "matrices": names, "launches": [u[0] for u in units],
                    "segment": tensors[names[0]].fused_plan["seg_len"], "launch": launch},
         "effective_bf16_GBps": round(eff_bf16, 2),
         "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3),
@@ -625,15 +647,13 @@ def main():
         "per_kernel": {n_: {"ms": round(per_kernel_ms[n_], 4), "alg_bytes": alg[n_]["total"],
                             "payload_bytes": alg[n_]["payload"], "index_bytes": alg[n_]["index"],
                             "table_bytes": alg[n_]["tables"],
-                            "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in names},
+                            "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in per_kernel_ms},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "kernel": (f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>" if m <= GEMV_UP_TO
-                                else "grf::fused_gemm_kernel<grf::SegmentWalk, MT>") + f" on {dom}"},
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "kernel": f"{kernel} on {dom}"},
     }
     if m > GEMV_UP_TO:
         # the matrix cores' share: useful flops of the dominant launch against the dense BF16 peak
-        flops = 2.0 * m * SHAPES[dom][0] * SHAPES[dom][1]
+        flops = sum(2.0 * m * SHAPES[n_][0] * SHAPES[n_][1] for n_ in dom.split("+"))
         result["mfma"] = {"achieved": round(flops / (per_kernel_ms[dom] * 1e-3) / 1e12, 2), "peak": 2500.0,
                           "unit": "TFLOP/s", "frac": round(flops / (per_kernel_ms[dom] * 1e-3) / 2.5e15, 4)}
     copy_rate = measured_copy_gbps(torch)

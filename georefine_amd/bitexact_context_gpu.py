@@ -489,7 +489,7 @@ class HipLinearGroup:
                 raise ValueError("group members need one width and one device")
         self.device, self._lib = first.device, first._lib
         self.error = torch.zeros((), device=self.device, dtype=torch.int32)
-        self._tilings = {}
+        self._tilings, self._pointer_arrays = {}, {}
         for key in (1, 2, "gemm"):
             self._tiling(key)  # raises FusedUnsupported when the members cannot share a tiling
 
@@ -512,10 +512,14 @@ class HipLinearGroup:
             self._tilings[key] = made
         return self._tilings[key]
 
-    def _arrays(self, tilings, outs, biases):
+    def _arrays(self, key, outs, biases):
         n = len(self.tensors)
-        frames = (ctypes.POINTER(_hip_abi.GrfBctxFused) * n)(*[ctypes.pointer(t.fused) for t in self.tensors])
-        tiles = (ctypes.POINTER(_hip_abi.GrfFusedTiling) * n)(*[ctypes.pointer(g[0]) for g in tilings])
+        if key not in self._pointer_arrays:  # the frames and tilings do not change between calls
+            tilings = self._tiling(key)
+            self._pointer_arrays[key] = (
+                (ctypes.POINTER(_hip_abi.GrfBctxFused) * n)(*[ctypes.pointer(t.fused) for t in self.tensors]),
+                (ctypes.POINTER(_hip_abi.GrfFusedTiling) * n)(*[ctypes.pointer(g[0]) for g in tilings]))
+        frames, tiles = self._pointer_arrays[key]
         ys = (ctypes.c_void_p * n)(*[y.data_ptr() for y in outs])
         ldy = (ctypes.c_uint32 * n)(*[y.stride(0) for y in outs])
         bias = (ctypes.c_void_p * n)(*[b.data_ptr() if b is not None else None for b in biases])
@@ -556,7 +560,7 @@ class HipLinearGroup:
             with torch.cuda.device(self.device):
                 stream = torch.cuda.current_stream(self.device).cuda_stream
                 if use_gemm:
-                    arrays = self._arrays(self._tiling("gemm"), outs, biases)
+                    arrays = self._arrays("gemm", outs, biases)
                     space = packed.buffer if packed else torch.empty(
                         self._lib.grf_gemm_workspace_bytes(cols, m), device=self.device, dtype=torch.uint8)
                     status = self._lib.grf_bctx_gemm_group(
@@ -564,7 +568,7 @@ class HipLinearGroup:
                         x2.stride(0) if x2 is not None else 0, m, arrays[2], arrays[3], arrays[4], space.data_ptr(),
                         space.numel(), self.error.data_ptr(), stream)
                 else:
-                    arrays = self._arrays(self._tiling(next(v for v in (1, 2, 4, 8) if v >= m)), outs, biases)
+                    arrays = self._arrays(next(v for v in (1, 2, 4, 8) if v >= m), outs, biases)
                     status = self._lib.grf_bctx_gemv_group(n, arrays[0], arrays[1], x2.data_ptr(), x2.stride(0), m,
                                                            arrays[2], arrays[3], arrays[4], self.error.data_ptr(), stream)
             if status:
