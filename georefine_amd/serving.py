@@ -20,16 +20,39 @@ class ContextServingError(RuntimeError):
     """Malformed or incomplete coded-weight module."""
 
 
-def hip_tensor_factory(frame, *, stride=1024, device="cuda:0"):
-    """The ``tensor_factory`` to hand to ``load_bctx_model`` (GCR/bitexact_context_serving.py:416,560)."""
+def hip_tensor_factory(frame, *, stride=1024, device="cuda:0", fused_segment=None):
+    """The ``tensor_factory`` to hand to ``load_bctx_model`` (GCR/bitexact_context_serving.py:416,560).
+    ``fused_segment`` fixes the segment length of the fused index (matrices that are to share a
+    launch need one length); the loader passes it to factories that take it."""
     from .bitexact_context_gpu import HipContextTensor
-    return HipContextTensor(frame, stride=stride, device=device)
+    return HipContextTensor(frame, stride=stride, device=device, fused_segment=fused_segment)
 
 
 def hip_predictive_factory(frame, reference_uint16_numpy, stride=1024, device="cuda:0"):
     """The ``predictive_factory`` of ``load_predictive_model`` (GCR/bitexact_predictive_serving.py:918-924)."""
     from .bitexact_predictive_gpu import HipPredictiveTensor
     return HipPredictiveTensor(frame, reference_uint16_numpy, stride=stride, device=device)
+
+
+class SharedProducts:
+    """Sibling linears that are applied to the same tensor one after the other (q/k/v
+    projections, gate and up) as one launch: the first member called with a tensor runs the
+    whole group and keeps the outputs, the others pick theirs up.  A call with another tensor
+    (identity, version counter, address or shape) runs the group again."""
+
+    def __init__(self, group, biases, batch_invariant=False):
+        self.group, self.biases, self.batch_invariant = group, list(biases), batch_invariant
+        self.launches = 0
+        self._key = self._x = self._outs = None
+
+    def output(self, index, x):
+        key = (id(x), x._version, x.data_ptr(), tuple(x.shape), tuple(x.stride()))
+        if key != self._key or self._x is None or self._x() is not x:
+            import weakref
+            self._outs = self.group.linear(x, self.biases, batch_invariant=self.batch_invariant)
+            self._key, self._x = key, weakref.ref(x)
+            self.launches += 1
+        return self._outs[index]
 
 
 class BctxLinear(nn.Module):
@@ -45,6 +68,7 @@ class BctxLinear(nn.Module):
         self.batch_invariant = batch_invariant
         self.forward_calls = 0
         self.weight_materializations = 0
+        self.shared = None  # (SharedProducts, index) when siblings share a launch
         self.register_parameter("bias", bias)
 
     @property
@@ -55,6 +79,8 @@ class BctxLinear(nn.Module):
 
     def forward(self, x):
         self.forward_calls += 1
+        if self.shared is not None and x.dtype == torch.bfloat16 and x.is_cuda:
+            return self.shared[0].output(self.shared[1], x)
         fused = getattr(self.context_weight, "linear", None)
         if fused is not None and x.dtype == torch.bfloat16:
             return fused(x, self.bias, batch_invariant=self.batch_invariant)
@@ -164,7 +190,8 @@ def _runtime_dtype(model, name, parameter, requested):
 
 def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
                     tensor_factory=None, predictive_factory=None, mix_predictor=None, host_decoder=None,
-                    loader_workers=1, batch_invariant=False, log=print, progress_callback=None):
+                    loader_workers=1, batch_invariant=False, log=print, progress_callback=None,
+                    share_launches=()):
     """Build ``model_factory()`` on the meta device and fill it from a BCTX package without
     ever holding a dense checkpoint: returns ``(model, receipt)``.
 
@@ -183,7 +210,11 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
     stride=, device=)`` indexes the frame against the reference words (for ``mixbf16`` the
     row-wise mix of two references with the candidate's coefficients, whose digest is
     checked), and the module receives a ``PredictiveContextTensor`` that resolves the
-    references when it decodes.  What this loader leaves to the caller is the model
+    references when it decodes.  ``share_launches`` names sibling linears that are applied to
+    one tensor, e.g. ``[("q_proj", "k_proj", "v_proj"), ("gate_proj", "up_proj")]``: wherever a
+    module has all the children of a tuple as coded linears of one input width (and the device
+    tensors support it), they are indexed with one segment length and multiplied in one
+    launch (``SharedProducts``); the receipt lists them under ``shared_launches``.  What this loader leaves to the caller is the model
     construction itself (the reference reads a Transformers config and generation config
     from the package's sidecars): ``model_factory`` returns the module to fill."""
     import hashlib
@@ -260,7 +291,8 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
 
     def create_context(name):
         row = entries[name]
-        context = tensor_factory(frame_of(name), stride=stride, device=device)
+        extra = {"fused_segment": shared_segment[name]} if name in shared_segment and takes_segment else {}
+        context = tensor_factory(frame_of(name), stride=stride, device=device, **extra)
         if tuple(context.shape) != pkg.frame_shape(row["shape"]):
             raise ContextServingError(f"indexed BCTX shape mismatch: {name}")
         if context.source_sha256 != row["source_sha256"]:
@@ -282,6 +314,37 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
              for module_name, module in list(model.named_modules())
              if isinstance(module, (nn.Linear, nn.Embedding))]
     coded = [item for item in coded if item[2] in entries]
+
+    # sibling linears that are to share a launch: found by attribute names under one parent
+    import inspect
+    try:
+        takes_segment = "fused_segment" in inspect.signature(tensor_factory).parameters
+    except (TypeError, ValueError):
+        takes_segment = False
+    coded_linears = {module_name: (module, weight_name) for module_name, module, weight_name in coded
+                     if isinstance(module, nn.Linear) and weight_name not in selected}
+    sibling_groups, shared_segment = [], {}
+    for names in share_launches or ():
+        names = tuple(names)
+        if not 2 <= len(names) <= 4:
+            raise ValueError("share_launches: groups of 2..4 sibling names")
+        for module_name in list(coded_linears):
+            parent, _, attr = module_name.rpartition(".")
+            if attr != names[0]:
+                continue
+            members = [f"{parent}.{n}" if parent else n for n in names]
+            if all(m in coded_linears for m in members) and \
+                    len({coded_linears[m][0].in_features for m in members}) == 1:
+                sibling_groups.append(members)
+                if takes_segment:
+                    from . import _fused
+                    cols = coded_linears[members[0]][0].in_features
+                    try:
+                        segment = _fused.choose_segment(cols, None, rows=max(coded_linears[m][0].out_features for m in members))
+                    except _fused.FusedUnsupported:
+                        continue
+                    for m in members:
+                        shared_segment[coded_linears[m][1]] = segment
 
     # tensors that need an object on the device: the coded weights and, transitively, the
     # references of predictive candidates; plain frames first (in parallel), then the
@@ -400,6 +463,21 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         else:
             replacements[module_name] = BctxEmbedding(context, padding_idx=module.padding_idx)
             consumed[weight_name] = record(weight_name, "compressed_embedding", resident)
+    shared_launches = []
+    for members in sibling_groups:
+        modules = [replacements[m] for m in members]
+        try:
+            from .bitexact_context_gpu import HipContextTensor, HipLinearGroup
+            if not all(isinstance(m.context_weight, HipContextTensor) for m in modules):
+                continue
+            products = SharedProducts(HipLinearGroup([m.context_weight for m in modules]), [m.bias for m in modules],
+                                      batch_invariant=batch_invariant)
+        except Exception as exc:  # the members stay separate launches
+            log(f"[bctx] {members} keep separate launches: {exc}")
+            continue
+        for index, module in enumerate(modules):
+            module.shared = (products, index)
+        shared_launches.append([coded_linears[m][1] for m in members])
     # parents before children, so that a replaced parent is not looked up through a stale child
     for name, replacement in sorted(replacements.items(), key=lambda item: item[0].count(".")):
         parent, attr = _parent_and_attr(model, name)
@@ -430,6 +508,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         "dense_parameter_bytes": sum(p.numel() * p.element_size() for p in model.parameters()),
         "buffer_bytes": sum(b.numel() * b.element_size() for b in model.buffers()),
         "consumed_tensors": consumed, "restored_bf16_control": False, "transcoded": False,
+        "shared_launches": shared_launches,
     }
     return model, receipt
 
@@ -437,7 +516,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
 def load_predictive_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
                           tensor_factory=None, context_factory=None, predictive_factory=None, mix_predictor=None,
                           host_decoder=None, loader_workers=1, batch_invariant=False, log=print,
-                          progress_callback=None):
+                          progress_callback=None, share_launches=()):
     """The predictive-package loader under the reference's name and keywords
     (GCR/bitexact_predictive_serving.py:596-619): ``context_factory`` makes the BCTX tensors
     (``tensor_factory`` is accepted as its older spelling), ``predictive_factory`` the PPCX ones,
@@ -453,5 +532,6 @@ def load_predictive_model(package, *, model_factory, device="cuda:0", dtype=torc
     return load_bctx_model(package, model_factory=model_factory, device=device, dtype=dtype, stride=stride,
                            tensor_factory=context_factory or tensor_factory, predictive_factory=predictive_factory,
                            mix_predictor=mix_predictor, host_decoder=host_decoder, loader_workers=loader_workers,
-                           batch_invariant=batch_invariant, log=log, progress_callback=progress_callback)
+                           batch_invariant=batch_invariant, log=log, progress_callback=progress_callback,
+                           share_launches=share_launches)
 

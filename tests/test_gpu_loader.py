@@ -98,3 +98,80 @@ def test_package_with_predictive_candidates_on_device(tmp_path):
             dict(dense.named_parameters())[name].copy_(torch.from_numpy(words).view(torch.bfloat16).cuda())
     x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(6, 256)))).view(torch.bfloat16).cuda()
     assert torch.allclose(model(x).float(), dense(x).float(), rtol=2e-2, atol=2e-2)
+
+
+def test_sibling_projections_share_a_launch(tmp_path):
+    """share_launches: q/k/v and gate/up of every block become one launch each; the model's
+    output agrees with the dense model, and with the same model loaded without sharing
+    wherever the vector-ALU kernel runs (one row: its bits do not depend on the tiling)."""
+    import torch
+    from torch import nn
+    from georefine_amd import bitexact_context_package as pkg
+    from georefine_amd import serving
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.q_proj = nn.Linear(256, 384, bias=True)
+            self.k_proj = nn.Linear(256, 64, bias=True)
+            self.v_proj = nn.Linear(256, 64, bias=False)
+            self.o_proj = nn.Linear(384, 256, bias=False)
+            self.gate_proj = nn.Linear(256, 512, bias=False)
+            self.up_proj = nn.Linear(256, 512, bias=False)
+            self.down_proj = nn.Linear(512, 256, bias=False)
+
+        def forward(self, x):
+            q, k, v = self.q_proj(x), self.k_proj(x), self.v_proj(x)
+            h = x + self.o_proj(q * torch.cat([k, v], dim=-1).repeat(*([1] * (x.ndim - 1)), 3))
+            return h + self.down_proj(torch.nn.functional.silu(self.gate_proj(h)) * self.up_proj(h))
+
+    class Net(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.blocks = nn.ModuleList([Block(), Block()])
+
+        def forward(self, x):
+            for block in self.blocks:
+                x = block(x)
+            return x
+
+    rng = np.random.default_rng(5)
+    reference = Net()
+    tensors = {}
+    for name, p in reference.named_parameters():
+        shape = tuple(p.shape)
+        words = weight_like(rng, *shape, sigma=0.05) if len(shape) == 2 else bf16_words(rng.normal(0, 0.1, size=shape))
+        tensors[name] = torch.from_numpy(words).view(torch.bfloat16)
+    path = tmp_path / "package"
+    pkg.write_package(path, tensors)
+    names = [("q_proj", "k_proj", "v_proj"), ("gate_proj", "up_proj")]
+    shared, receipt = serving.load_bctx_model(path, model_factory=Net, device="cuda:0", share_launches=names,
+                                              log=lambda _: None)
+    plain, _ = serving.load_bctx_model(path, model_factory=Net, device="cuda:0", log=lambda _: None)
+    assert sorted(map(tuple, receipt["shared_launches"])) == sorted(
+        [tuple(f"blocks.{i}.{n}.weight" for n in g) for i in range(2) for g in names])
+    for block in shared.blocks:
+        assert block.q_proj.shared[0] is block.k_proj.shared[0] is block.v_proj.shared[0]
+        assert block.gate_proj.shared[0] is block.up_proj.shared[0] and block.o_proj.shared is None
+    dense = Net().to(torch.bfloat16).cuda()
+    with torch.no_grad():
+        for name, t in tensors.items():
+            dict(dense.named_parameters())[name].copy_(t.cuda())
+    for shape in ((1, 256), (2, 3, 256), (70, 256)):
+        x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=shape))).view(torch.bfloat16).cuda()
+        with torch.no_grad():
+            got, want = shared(x), dense(x)
+        assert got.shape == want.shape
+        # two blocks of BF16 intermediates: compared on the scale of the output
+        assert float((got.float() - want.float()).abs().max()) <= 3e-2 * float(want.float().abs().max())
+        if shape == (1, 256):
+            assert torch.equal(got.view(torch.uint16), plain(x).view(torch.uint16))
+    first = shared.blocks[0]
+    assert first.q_proj.shared[0].launches == 3 and first.gate_proj.shared[0].launches == 3  # one per forward
+    assert first.q_proj.forward_calls == first.k_proj.forward_calls == 3
+    # a member called on its own with another tensor runs the group again and gives its own product
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(1, 256)))).view(torch.bfloat16).cuda()
+    alone = first.k_proj(x)
+    assert torch.equal(alone.view(torch.uint16), plain.blocks[0].k_proj(x).view(torch.uint16))
+    x.add_(1)  # the same tensor object with new contents: not served from the kept outputs
+    assert torch.equal(first.k_proj(x).view(torch.uint16), plain.blocks[0].k_proj(x).view(torch.uint16))
