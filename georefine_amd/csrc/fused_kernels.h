@@ -135,23 +135,45 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
       float acc[M];
 #pragma unroll
       for (int m = 0; m < M; ++m) acc[m] = 0.f;
-      for (uint32_t t = 0; t < S; t += 16) {
+      if (STORE) {
+        // a lane keeps two groups of 16 words and stores them as one 64-byte run: a line of
+        // the output is then written in two visits, not four (four groups would finish the
+        // line at once but cost the registers that keep two workgroups on a compute unit)
+        constexpr int kHold = 2;
+        const uint64_t at = SINK == kGather ? (uint64_t)(tile * R + r) * K + col0 : elem0;
+        w.begin16(0, S);
+        for (uint32_t t = 0; t < S; t += 16 * kHold) {
+          uint32_t hold[kHold][8];
+          const uint32_t groups = min((uint32_t)kHold, (S - t) / 16);
+#pragma unroll
+          for (int k = 0; k < kHold; ++k)
+            if (k < groups) {
+              w.template half<0>(q, reinterpret_cast<uint32_t(&)[4]>(hold[k][0]));
+              w.template half<1>(q, reinterpret_cast<uint32_t(&)[4]>(hold[k][4]));
+              // the loads of the group after this one leave before the stores below: memory
+              // operations complete in order, so a wait for a load that followed the stores
+              // would wait for them too
+              if (t + 16 * (k + 1) < S) w.begin16(t + 16 * (k + 1), S);
+            }
+          uint4 *dst = reinterpret_cast<uint4 *>(out + at + t);
+#pragma unroll
+          for (int k = 0; k < kHold; ++k)
+            if (k < groups) {
+              dst[2 * k] = make_uint4(hold[k][0], hold[k][1], hold[k][2], hold[k][3]);
+              dst[2 * k + 1] = make_uint4(hold[k][4], hold[k][5], hold[k][6], hold[k][7]);
+            }
+        }
+      }
+      for (uint32_t t = 0; !STORE && t < S; t += 16) {
         uint32_t pair[8];
         w.decode16(t, S, q, pair);
-        if (STORE) {
-          const uint64_t at = SINK == kGather ? (uint64_t)(tile * R + r) * K + col0 : elem0;
-          uint4 *dst = reinterpret_cast<uint4 *>(out + at + t);
-          dst[0] = make_uint4(pair[0], pair[1], pair[2], pair[3]);
-          dst[1] = make_uint4(pair[4], pair[5], pair[6], pair[7]);
-        } else {
 #pragma unroll
-          for (int m = 0; m < M; ++m) {
-            const uint4 *xm = reinterpret_cast<const uint4 *>(xr + m * P * xpitch + t);
-            const uint4 xa = xm[0], xb = xm[1];
-            const uint32_t xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+        for (int m = 0; m < M; ++m) {
+          const uint4 *xm = reinterpret_cast<const uint4 *>(xr + m * P * xpitch + t);
+          const uint4 xa = xm[0], xb = xm[1];
+          const uint32_t xv[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
 #pragma unroll
-            for (int k = 0; k < 8; ++k) acc[m] = dot2_bf16(pair[k], xv[k], acc[m]);
-          }
+          for (int k = 0; k < 8; ++k) acc[m] = dot2_bf16(pair[k], xv[k], acc[m]);
         }
       }
       if (!STORE) {
@@ -186,8 +208,10 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
   if (bad) atomicOr(error, (int)bad);
 }
 
+// Six waves per SIMD keep two 768-lane workgroups on a compute unit: the store sinks, which
+// hold decoded words back, would otherwise take a few registers too many for that.
 template <class Walk, int M, int SINK>
-__global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_kernel(grf_bctx_fused f, grf_fused_tiling g,
+__global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_walk_kernel(grf_bctx_fused f, grf_fused_tiling g,
                                                                             const uint16_t *x, uint32_t ldx,
                                                                             uint16_t *y, uint32_t ldy,
                                                                             const uint16_t *bias, uint16_t *out,
