@@ -149,3 +149,46 @@ def test_predictive_plan_refuses_rows_that_are_not_a_multiple_of_32():
     ref = target ^ np.uint16(1)
     ix = _read_frame(ppcx.encode(target, ref), ref, 64, fused=True)
     assert ix["mode"] in (0, 1) and "fused_plan" not in ix and "multiple of 32" in ix["fused_reason"]
+
+
+def _synthetic_choice(spr, class_rows, tabn=330, bytes_per_segment=40):
+    """choose_tiling for a frame with 4 column classes and 8 KiB lookups, from its figures
+    alone: a piece of `lanes` segments takes about bytes_per_segment each."""
+    cap = lambda lanes: (16 + bytes_per_segment * lanes + 15) // 16 * 16
+    lds = lambda p, r, c: _fused.lds_bytes(4, 13, tabn, 1, p, 64, r, c)
+    return _fused.choose_tiling(spr, np.asarray(class_rows), cap, lds, seg_len=64,
+                                table_bytes=4 * ((tabn + 1) * 8 + 8192))
+
+
+def test_planner_takes_the_fewest_slabs_among_tilings_it_scores_alike(monkeypatch):
+    """A 17408 x 5120 matrix in 16 equal row classes: 10 and 20 lanes per row fill the chip
+    equally and the model separates them by about one per cent; the wider slab wins because
+    fewer residual lines straddle two slabs."""
+    monkeypatch.delenv("GEOREFINE_FUSED_TILING", raising=False)
+    threads, p, r, n_slabs, n_tiles, cap, lds = _synthetic_choice(80, [1088] * 16)
+    assert (threads, p, r) == (768, 20, 34) and n_slabs == 4 and n_tiles == 512
+    assert lds * 2 <= _fused.MAX_LDS  # two workgroups per compute unit
+
+
+def test_group_plans_share_one_tile_shape_and_keep_every_member_complete():
+    rng = np.random.default_rng(5)
+    plans, frames = [], []
+    for rows in (96, 32, 32):  # q, k, v of one width
+        ix, plan = _plan(weight_like(rng, rows, 640))
+        plans.append(plan)
+        frames.append(ix)
+    for kwargs in (dict(m=1), dict(m=8), dict(gemm=True)):
+        tilings = _fused.plan_group(plans, **kwargs)
+        shapes = {(t["scalars"]["threads"], t["scalars"]["lanes_per_row"], t["scalars"]["rows_per_tile"],
+                   t["scalars"]["n_slabs"], t["scalars"]["piece_cap"]) for t in tilings}
+        assert len(shapes) == 1 and len(tilings) == 3
+        for ix, plan, t in zip(frames, plans, tilings):
+            s = t["scalars"]
+            rows = t["tile_rows"].reshape(s["n_tiles"], s["rows_per_tile"])
+            assert sorted(rows[rows != 0xFFFFFFFF].tolist()) == list(range(plan.rows))
+            for tile, cls in zip(rows, t["tile_class"]):
+                assert np.all(ix["rows"][tile[tile != 0xFFFFFFFF]] == cls)
+            assert t["lds"] <= _fused.MAX_LDS
+    other = _plan(weight_like(rng, 32, 1280))[1]
+    with pytest.raises(_fused.FusedUnsupported):
+        _fused.plan_group([plans[0], other], m=1)
