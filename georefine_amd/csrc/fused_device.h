@@ -315,13 +315,19 @@ __device__ __forceinline__ uint32_t fused_word_bits(uint32_t hi, uint32_t r6_sig
 }
 
 // A lane's walk over one segment: rANS cursor, plus the registers that hold the packed
-// residuals and the column classes of the next 16 symbols.
-struct SegmentWalk {
+// residuals and the column classes of the next 16 symbols.  AHEAD (segments of 64 symbols
+// only): the residuals of the whole segment, 48 bytes, are read when the segment starts; a
+// line of the residual section is then fetched once instead of on four visits a group
+// apart, between which the L2 may have dropped it.
+template <bool AHEAD>
+struct SegmentWalkT {
+  static constexpr bool kAhead = AHEAD;
   Cursor c;
   uint32_t ip0, gofs, seg;
   const uint32_t *rawp;
   const uint4 *ccp;
-  uint32_t n0, n1, n2;
+  uint32_t n0, n1, n2;             // !AHEAD: the next group's residual words
+  uint32_t rw[AHEAD ? 12 : 1];     // AHEAD: the segment's residual words
   uint4 nc4;
   Raw6x16 rr;      // the group being decoded
   uint32_t cw[4];
@@ -334,9 +340,17 @@ struct SegmentWalk {
     c.state = f.seg_state[seg];
     rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
     ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
-    n0 = rawp[0];
-    n1 = rawp[1];
-    n2 = rawp[2];
+    if constexpr (AHEAD) {
+      const uint4 *r4 = reinterpret_cast<const uint4 *>(rawp);  // 48-byte groups: 16-byte aligned
+      const uint4 a = r4[0], b = r4[1], d = r4[2];
+      rw[0] = a.x, rw[1] = a.y, rw[2] = a.z, rw[3] = a.w;
+      rw[4] = b.x, rw[5] = b.y, rw[6] = b.z, rw[7] = b.w;
+      rw[8] = d.x, rw[9] = d.y, rw[10] = d.z, rw[11] = d.w;
+    } else {
+      n0 = rawp[0];
+      n1 = rawp[1];
+      n2 = rawp[2];
+    }
     nc4 = ccp[0];
   }
   // the row piece was staged at piece_off from global offset a0
@@ -348,18 +362,24 @@ struct SegmentWalk {
   // Start the group of symbols [t, t+16): unpack its residuals and column classes, and load
   // the registers of the following group meanwhile.
   __device__ __forceinline__ void begin16(uint32_t t, uint32_t S) {
-    rr.set(n0, n1, n2);
     cw[0] = nc4.x;
     cw[1] = nc4.y;
     cw[2] = nc4.z;
     cw[3] = nc4.w;
     // the last group loads itself again rather than branch around the loads
     const uint32_t next = min(t / 16 + 1, S / 16 - 1);
-    const uint32_t *nx = rawp + next * 3;
-    n0 = nx[0];
-    n1 = nx[1];
-    n2 = nx[2];
     nc4 = ccp[next];
+    if constexpr (AHEAD) {  // the words of the groups still to come move down one group
+      rr.set(rw[0], rw[1], rw[2]);
+#pragma unroll
+      for (int i = 0; i < 9; ++i) rw[i] = rw[i + 3];
+    } else {
+      rr.set(n0, n1, n2);
+      const uint32_t *nx = rawp + next * 3;
+      n0 = nx[0];
+      n1 = nx[1];
+      n2 = nx[2];
+    }
   }
   // Half H (0 or 1) of the group: eight symbols into four BF16 pairs (word k in the low
   // half, k+1 in the high half).
@@ -385,5 +405,7 @@ struct SegmentWalk {
     return c.state == f.seg_state[seg + 1] && gofs + (c.j - ip0) == f.seg_offset[seg + 1];
   }
 };
+using SegmentWalk = SegmentWalkT<false>;
+using SegmentWalkAhead = SegmentWalkT<true>;
 
 }  // namespace grf

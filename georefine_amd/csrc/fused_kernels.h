@@ -28,6 +28,8 @@
 #include <atomic>
 #include <string>
 
+#include <type_traits>
+
 #include "fused_device.h"
 
 namespace grf {
@@ -73,6 +75,16 @@ __device__ __forceinline__ uint16_t round_bf16(float v) {
 // them where the row lies in the dense matrix, or store them in the slot the row has in the
 // tiling (row tile * R + r of a compact [n_tiles * R][cols] output: a gather of rows).
 enum Sink : int { kDot = 0, kStore = 1, kGather = 2 };
+
+// the walker to use for the same frame when its segments have 64 symbols and few enough
+// activation rows leave it the registers (itself where there is no such variant)
+template <class Walk>
+struct ahead_of { using type = Walk; };
+template <>
+struct ahead_of<grf::SegmentWalk> { using type = grf::SegmentWalkAhead; };
+constexpr uint32_t kAheadMaxRows = 4;
+// a segment's residuals are 48 bytes, read as three 16-byte vectors
+inline bool reads_ahead(const grf_bctx_fused &f) { return f.seg_len == 64 && !((uintptr_t)f.raw6 & 15); }
 
 // One workgroup's walk over tile `tile` of a frame.
 template <class Walk, int M, int SINK>
@@ -135,7 +147,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
       float acc[M];
 #pragma unroll
       for (int m = 0; m < M; ++m) acc[m] = 0.f;
-      if (STORE) {
+      if constexpr (STORE) {
         // a lane keeps two groups of 16 words and stores them as one 64-byte run: a line of
         // the output is then written in two visits, not four (four groups would finish the
         // line at once but cost the registers that keep two workgroups on a compute unit)
@@ -275,6 +287,13 @@ int launch_gemv(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
   if (ldx < f.cols || ldy < f.rows || (ldx & 1) || ((uintptr_t)x & 3))
     return grf::set_error(GRF_BAD_ARGUMENT,
                           std::string(who) + ": x must be 4-byte aligned with an even leading dimension");
+  using Ahead = typename ahead_of<Walk>::type;
+  if (!std::is_same<Ahead, Walk>::value && reads_ahead(f) && m_rows <= kAheadMaxRows) switch (m_rows) {
+      case 1: return launch_walk<Ahead, 1, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+      case 2: return launch_walk<Ahead, 2, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+      case 3: return launch_walk<Ahead, 3, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+      default: return launch_walk<Ahead, 4, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
+    }
   switch (m_rows) {
     case 1: return launch_walk<Walk, 1, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
     case 2: return launch_walk<Walk, 2, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
@@ -657,6 +676,15 @@ int launch_gemv_group(const char *who, const GroupSpec &spec, const uint16_t *x,
   if (!x || ldx < a.f[0].cols || (ldx & 1) || ((uintptr_t)x & 3))
     return grf::set_error(GRF_BAD_ARGUMENT,
                           std::string(who) + ": x must be 4-byte aligned with an even leading dimension");
+  using Ahead = typename ahead_of<Walk>::type;
+  bool ahead = !std::is_same<Ahead, Walk>::value && m_rows <= kAheadMaxRows;
+  for (uint32_t i = 0; i < a.n; ++i) ahead = ahead && reads_ahead(a.f[i]);
+  if (ahead) switch (m_rows) {
+      case 1: return launch_walk_group<Ahead, 1>(a, x, ldx, error, s);
+      case 2: return launch_walk_group<Ahead, 2>(a, x, ldx, error, s);
+      case 3: return launch_walk_group<Ahead, 3>(a, x, ldx, error, s);
+      default: return launch_walk_group<Ahead, 4>(a, x, ldx, error, s);
+    }
   switch (m_rows) {
     case 1: return launch_walk_group<Walk, 1>(a, x, ldx, error, s);
     case 2: return launch_walk_group<Walk, 2>(a, x, ldx, error, s);

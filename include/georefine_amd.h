@@ -166,7 +166,9 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  *                                            (freq & 0xFFFF)<<16 (0 stands for 65536),
  *                                            high32 = symbol<<5; unused entries: 0
  *   col_class   u8  [cols]
- * main_bytes must be readable for 16 bytes past main_n_bytes. */
+ * main_bytes must be readable for 16 bytes past main_n_bytes.  raw6 is 4-byte aligned;
+ * with seg_len 64 and 16-byte alignment the GEMV reads a segment's 48 residual bytes
+ * once, as it starts, instead of 12 at a time. */
 typedef struct grf_bctx_fused {
   const uint8_t *main_bytes;
   const uint8_t *raw6;
