@@ -46,8 +46,11 @@ int grf_bctx_fused_decode(const grf_bctx_fused *frame, const grf_fused_tiling *t
   if (!frame || !tiling || !out || !error)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_fused_decode: null argument");
   if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_fused_decode")) return rc;
+  if (grf::reads_ahead(*frame))
+    return grf::launch_walk<grf::SegmentWalkAhead, 1, grf::kStore>(*frame, *tiling, nullptr, 0, nullptr, 0, nullptr,
+                                                                   out, error, (hipStream_t)hip_stream);
   return grf::launch_walk<grf::SegmentWalk, 1, grf::kStore>(*frame, *tiling, nullptr, 0, nullptr, 0, nullptr, out, error,
-                                                     (hipStream_t)hip_stream);
+                                                            (hipStream_t)hip_stream);
 }
 
 int grf_bctx_fused_gather(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint16_t *out,
