@@ -112,3 +112,25 @@ def test_fused_checkpoint_mismatch_sets_error(oracle):
         t.linear(x, check=True)
     assert t.linear(x).shape == (1, 64)
     assert t.error.item() != 0
+
+
+def test_residual_buffer_off_a_16_byte_boundary_gives_the_same_bits():
+    """Segments of 64 symbols read their 48 residual bytes as three 16-byte vectors when the
+    buffer allows it; a caller's buffer that is only 4-byte aligned takes the 12-bytes-a-group
+    walker.  Same words, same products."""
+    import copy
+    import torch
+    words = weight_like(np.random.default_rng(21), 100, 768)
+    frame, t = _tensor(words, fused_segment=64)
+    assert t.fused is not None and t.fused.raw6 % 16 == 0
+    other = copy.copy(t)
+    other.buffers = dict(t.buffers)
+    padded = torch.zeros(t.buffers["residual_stream"].numel() + 4, dtype=torch.uint8, device="cuda:0")
+    padded[4:] = t.buffers["residual_stream"]
+    other.buffers["residual_stream"] = padded[4:]
+    other._bind()
+    assert other.fused.raw6 % 16 == 4
+    assert np.array_equal(other.decode().view(torch.uint16).cpu().numpy(), words)
+    for m in (1, 2, 4):
+        x = torch.from_numpy(bf16_words(np.random.default_rng(m).normal(0, 1, size=(m, 768)))).view(torch.bfloat16).cuda()
+        assert torch.equal(other.gemv(x, check=True), t.gemv(x, check=True))
