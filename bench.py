@@ -435,7 +435,8 @@ def run_stack(args):
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     dom = max(LAYER, key=lambda n_: ms[n_])
     achieved = alg[dom]["total"] / (ms[dom] * 1e-3) / 1e9
-    kernel = "grf::fused_gemm_kernel<grf::SegmentWalk, MT>" if m > GEMV_UP_TO else f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>"
+    kernel = ("grf::fused_gemm_kernel<grf::SegmentWalkT<false>, MT>" if m > GEMV_UP_TO
+              else f"grf::fused_walk_kernel<grf::SegmentWalkT<true>, {m}, 0>")  # the stack's segments have 64 symbols
     print(json.dumps({
         "metric": "compressed-weight decode-GEMV GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
@@ -474,10 +475,11 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB read + 128 MiB write elementwise kernel three times, so that a "
                          "counter profile of this command holds a kernel of known traffic to scale by")
-    ap.add_argument("--workload", choices=("mlp", "stack", "ppcx"), default="mlp",
+    ap.add_argument("--workload", choices=("mlp", "stack", "ppcx", "decode"), default="mlp",
                     help="mlp: the three MLP matrices of one layer (the headline); stack: every coded linear of "
                          "--layers layers resident at once, one pass at batch 64 (or --batch); ppcx: a predictive "
-                         "frame against its dense reference, product with 96 rows (or --batch)")
+                         "frame against its dense reference, product with 96 rows (or --batch); decode: the "
+                         "three MLP matrices decoded to dense BF16 (decode(), the fused store sink)")
     ap.add_argument("--layers", type=int, default=64)
     ap.add_argument("--no-groups", action="store_true",
                     help="one launch per linear instead of one for the matrices that take the same activations "
@@ -489,6 +491,9 @@ def main():
         sys.exit("bench.py: this decode path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists)")
     if args.workload == "mlp":
         args.batch = args.batch or 1  # the stack defaults to 64
+    decode_only = args.workload == "decode"
+    if decode_only:
+        args.batch, args.no_groups = 0, True  # no activations: rows = 0 selects the store sink's tiling
     if args.workload == "ppcx":
         return run_predictive(args)
     if args.workload == "stack":
@@ -529,7 +534,7 @@ def main():
 
     m = args.batch
     rng = np.random.default_rng(7)
-    x_words = {k: bf16_words(rng.normal(0, 1, size=(m, k))) for k in (5120, 17408)}
+    x_words = {k: bf16_words(rng.normal(0, 1, size=(max(m, 1), k))) for k in (5120, 17408)}
     x = {k: torch.from_numpy(v).view(torch.bfloat16).cuda() for k, v in x_words.items()}
 
     # the launches of a step: gate and up take the same activations and share one launch
@@ -540,7 +545,9 @@ def main():
         units.append(("gate+up", ["gate", "up"], lambda: pair.linear(x[5120])))
         log(f"gate+up: one launch, tiling {pair._tiling(m if m <= GEMV_UP_TO else 'gemm')[0][3]}")
     for name in names:
-        if not any(name in u[1] for u in units):
+        if decode_only:
+            units.append((name, [name], lambda name=name: tensors[name].decode(check=False)))
+        elif not any(name in u[1] for u in units):
             units.append((name, [name], lambda name=name: tensors[name].linear(x[SHAPES[name][1]])))
 
     def step():
@@ -603,6 +610,8 @@ def main():
         alg[label] = {k: sum(p_[k] for p_ in parts) for k in parts[0]}
         if len(members) > 1:  # the members read one x
             alg[label]["total"] -= (len(members) - 1) * m * SHAPES[members[0]][1] * 2
+        if decode_only:  # the dense matrix is written once
+            alg[label]["total"] += sum(2 * SHAPES[n_][0] * SHAPES[n_][1] for n_ in members)
     step_bytes = sum(a["total"] for a in alg.values())
     dense_bytes = sum(2 * SHAPES[n][0] * SHAPES[n][1] for n in names)
     ms_per_step = wall / args.steps * 1e3
@@ -613,19 +622,27 @@ def main():
     # kernel of known size); a recorded figure, bench.py cannot read hardware counters itself
     dom = max(per_kernel_ms, key=lambda n_: per_kernel_ms[n_])
     grouped = "+" in dom
-    if m <= GEMV_UP_TO:
-        kernel = f"grf::fused_walk_group_kernel<grf::SegmentWalk, {m}>" if grouped else f"grf::fused_walk_kernel<grf::SegmentWalk, {m}, 0>"
+    # 64-symbol segments: the walker that reads a segment's residuals once
+    ahead = "true" if tensors[names[0]].fused_plan["seg_len"] == 64 else "false"
+    if decode_only:
+        kernel = f"grf::fused_walk_kernel<grf::SegmentWalkT<{ahead}>, 1, 1>"
+    elif m <= GEMV_UP_TO:
+        kernel = (f"grf::fused_walk_group_kernel<grf::SegmentWalkT<{ahead}>, {m}>" if grouped
+                  else f"grf::fused_walk_kernel<grf::SegmentWalkT<{ahead}>, {m}, 0>")
     else:
-        kernel = "grf::fused_gemm_group_kernel<grf::SegmentWalk, MT>" if grouped else "grf::fused_gemm_kernel<grf::SegmentWalk, MT>"
+        kernel = ("grf::fused_gemm_group_kernel<grf::SegmentWalkT<false>, MT>" if grouped
+                  else "grf::fused_gemm_kernel<grf::SegmentWalkT<false>, MT>")
     traffic = None
-    recorded = ROOT / "profiles" / "fused_gemv_m1_qwen27b_mlp_traffic.json"
-    if m == 1 and recorded.exists():
+    recorded = ROOT / "profiles" / ("fused_store_decode_qwen27b_mlp_traffic.json" if decode_only
+                                    else "fused_gemv_m1_qwen27b_mlp_traffic.json")
+    if (m == 1 or decode_only) and recorded.exists():
         per_kernel_traffic = json.loads(recorded.read_text()).get("traffic_bytes_per_launch")
         if isinstance(per_kernel_traffic, dict):  # by kernel name
             traffic = per_kernel_traffic.get(kernel.split("<")[0].split("::")[-1])
     achieved = alg[dom]["total"] / (per_kernel_ms[dom] * 1e-3) / 1e9
     result = {
-        "metric": "compressed-weight decode-GEMV GB/s",
+        "metric": "compressed-weight decode GB/s (coded bytes read + dense BF16 written)" if decode_only
+                  else "compressed-weight decode-GEMV GB/s",
         "value": round(value, 2),
         "unit": "GB/s",
         "n_gpus": 1,
@@ -637,12 +654,14 @@ def main():
         "vs_baseline": None,
         "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
         "data": "synthetic",
-        "config": {"workload": "fused decode-" + ("GEMV" if m <= GEMV_UP_TO else "GEMM") + ", batch %d, Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
-                               "BCTX (16,4) frames, residuals resident in packed 6-bit form" % m,
+        "config": {"workload": ("fused decode to dense BF16 (decode())" if decode_only else
+                                "fused decode-" + ("GEMV" if m <= GEMV_UP_TO else "GEMM") + ", batch %d" % m)
+                               + ", Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
+                               "BCTX (16,4) frames, residuals resident in packed 6-bit form",
                    "batch": m, "matrices": names, "launches": [u[0] for u in units],
                    "segment": tensors[names[0]].fused_plan["seg_len"], "launch": launch},
         "effective_bf16_GBps": round(eff_bf16, 2),
-        "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3),
+        "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3) if m else None,
         "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
         "per_kernel": {n_: {"ms": round(per_kernel_ms[n_], 4), "alg_bytes": alg[n_]["total"],
                             "payload_bytes": alg[n_]["payload"], "index_bytes": alg[n_]["index"],
