@@ -104,6 +104,17 @@ def lds_bytes(nc, lognb, tabn, m, p, s, r, piece_cap):
     return total
 
 
+def lds_bytes_waves(nc, lognb, tabn, m, threads, p, r, n_slabs, piece_cap):
+    """LDS of the wave-unit GEMV: tables, one row piece per row of every wave's unit, the unit
+    sums of every (row, slab), the tile's rows."""
+    a16 = lambda v: (v + 15) // 16 * 16
+    total = a16(nc * (a16((tabn + 1) * 8) + (1 << lognb)))
+    total = a16(total + threads // 64 * (64 // p) * piece_cap)
+    total = a16(total + r * n_slabs * m * 4)
+    total = a16(total + r * 4)
+    return total
+
+
 GEMM_MAX_TILES = 4  # 16-row activation tiles whose partial sums pass through LDS at a time
 
 
@@ -121,9 +132,13 @@ def lds_bytes_gemm(nc, lognb, tabn, p, r, piece_cap):
     return max(total, gemm_shape(p, r)[2] // 64 * GEMM_MAX_TILES * 1024)  # later: every wave's partial sums
 
 
+WINDOW = 8  # bytes the refill reads from the 4-byte aligned cursor on
+
+
 def piece_capacity(offsets, rows, spr, p):
     """LDS bytes one row piece may need: the longest (16-byte aligned start .. end) span
-    over every (row, slab), plus two bytes the refill reads ahead, rounded to 16."""
+    over every (row, slab), plus the eight bytes the refill's window may read from the
+    cursor on, rounded to 16."""
     off = offsets[:-1].reshape(rows, spr).astype(np.int64)
     end_of_row = np.concatenate((off[1:, 0], [int(offsets[-1])]))
     longest = 0
@@ -131,7 +146,7 @@ def piece_capacity(offsets, rows, spr, p):
         g0 = off[:, b]
         g1 = off[:, b + p] if b + p < spr else end_of_row
         longest = max(longest, int((g1 - (g0 & ~15)).max()))
-    return (longest + 2 + 15) // 16 * 16
+    return (longest + WINDOW + 15) // 16 * 16
 
 
 def _tiles(class_rows, r):
@@ -215,6 +230,53 @@ def choose_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=64, ta
         r = _spread_rows(class_rows, r, capacity)
         tiles, lds = _tiles(class_rows, r), lds_fn(p, r, cap)
     return threads, p, r, n_slabs, tiles, cap, lds
+
+
+SCHEME_SLABS, SCHEME_WAVES = 0, 1
+WAVE_ROWS_PER_PASS = 2  # activation rows one launch of the wave-unit kernel carries
+WAVE_UNIT_OVERHEAD = 8  # decode steps' worth of staging, reduction and bookkeeping per unit
+
+
+def choose_wave_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=64, table_bytes=0):
+    """Tiling of the wave-unit GEMV: a wave walks units of 64 / P rows x P consecutive
+    segments (P a power of two) and the waves of a workgroup share out the units of its tile
+    without meeting at a barrier.  Modelled time = rounds of workgroups x (table copy + the
+    busiest wave's units x steps per unit), at the speed the resident wave count allows;
+    the score is the share of the paid lane-steps that decode a symbol."""
+    total_rows = sum(int(c) for c in class_rows)
+    forced = os.environ.get("GEOREFINE_FUSED_WAVE_TILING")  # "threads,lanes_per_row,rows": experiments only
+    if forced:
+        t_, p_, r_ = (int(v) for v in forced.split(","))
+        cap = piece_cap_fn(p_)
+        n_slabs = -(-spr // p_)
+        return t_, p_, r_, n_slabs, _tiles(class_rows, r_), cap, lds_fn(t_, p_, r_, n_slabs, cap)
+    best = None
+    unit_steps = seg_len + WAVE_UNIT_OVERHEAD
+    for p in (4, 8, 16, 32, 64):
+        if p > 4 and p // 2 >= spr:
+            continue  # half the lanes of every unit would idle
+        rpw = 64 // p
+        n_slabs = -(-spr // p)
+        cap = piece_cap_fn(p)
+        for threads in (1024, 768, 512):
+            nwaves = threads // 64
+            for r in range(rpw, 129):
+                groups = -(-r // rpw)
+                lds = lds_fn(threads, p, r, n_slabs, cap)
+                if lds > MAX_LDS:
+                    break
+                per_cu = max(1, min(24 // nwaves, MAX_LDS // lds))  # six waves per SIMD by registers
+                slots = cus * per_cu
+                tiles = _tiles(class_rows, r)
+                rounds = -(-tiles // slots)
+                unit_rounds = -(-(groups * n_slabs) // nwaves)
+                paid = rounds * slots * nwaves * 64 * (unit_rounds * unit_steps + 3 + table_bytes / 12288)
+                score = total_rows * spr * seg_len / paid * min(1.0, per_cu * nwaves / 24)
+                if best is None or score > best[0] * 1.0001:
+                    best = (score, threads, p, r, n_slabs, tiles, cap, lds)
+    if best is None:
+        raise FusedUnsupported("no wave-unit tiling fits in LDS")
+    return best[1:]
 
 
 GEMM_WAVES_PER_SIMD = int(os.environ.get("GEOREFINE_GEMM_WAVES", "6"))
@@ -314,18 +376,27 @@ class FramePlan:
             self._caps[p] = piece_capacity(self.seg_offset, self.rows, self.spr, p)
         return self._caps[p]
 
-    def tiling(self, m):
+    def tiling(self, m, waves=False):
         """Host arrays and scalars of a ``grf_fused_tiling`` sized for m activation rows
-        (m = 0: the store sink)."""
-        threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
-            self.spr, self.class_rows, self._cap,
-            lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_),
-            seg_len=self.seg_len, table_bytes=self.table_bytes())
+        (m = 0: the store sink).  ``waves``: the wave-unit scheme of the GEMV, one tiling for
+        every row count (launches carry at most two rows each)."""
+        if waves and m:
+            threads, p, r, n_slabs, n_tiles, cap, lds = choose_wave_tiling(
+                self.spr, self.class_rows, self._cap,
+                lambda t_, p_, r_, s_, cap_: lds_bytes_waves(self.nc, self.lognb, self.tabn, WAVE_ROWS_PER_PASS, t_, p_,
+                                                             r_, s_, cap_),
+                seg_len=self.seg_len, table_bytes=self.table_bytes())
+        else:
+            threads, p, r, n_slabs, n_tiles, cap, lds = choose_tiling(
+                self.spr, self.class_rows, self._cap,
+                lambda p_, r_, cap_: lds_bytes(self.nc, self.lognb, self.tabn, m, p_, self.seg_len, r_, cap_),
+                seg_len=self.seg_len, table_bytes=self.table_bytes())
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                 n_tiles=n_tiles, piece_cap=cap), lds=lds)
+                                 n_tiles=n_tiles, piece_cap=cap,
+                                 scheme=SCHEME_WAVES if waves and m else SCHEME_SLABS), lds=lds)
 
     def gather_scalars(self):
         """Scalars of a tiling that gives every requested row a tile of its own, all of its
@@ -350,10 +421,10 @@ class FramePlan:
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                 n_tiles=n_tiles, piece_cap=cap), lds=lds)
+                                 n_tiles=n_tiles, piece_cap=cap, scheme=SCHEME_SLABS), lds=lds)
 
 
-def plan_group(plans, m=None, gemm=False):
+def plan_group(plans, m=None, gemm=False, waves=False):
     """Tilings of several frames of one width for one grouped launch: planned as if the
     members' row classes belonged to one matrix (so a small member's tiles fill the
     workgroup slots a large one leaves), with one thread count, lanes per row and rows per
@@ -364,9 +435,16 @@ def plan_group(plans, m=None, gemm=False):
     class_rows = np.concatenate([pl.class_rows for pl in plans])
     cap_fn = lambda lanes: max(pl._cap(lanes) for pl in plans)
     table = max(pl.table_bytes() for pl in plans)
+    scheme = SCHEME_SLABS
     if gemm:
         lds_fn = lambda p_, r_, cap_: max(lds_bytes_gemm(pl.nc, pl.lognb, pl.tabn, p_, r_, cap_) for pl in plans)
         threads, p, r, n_slabs, _, cap, lds = choose_gemm_tiling(first.spr, class_rows, cap_fn, lds_fn,
+                                                                 seg_len=first.seg_len, table_bytes=table)
+    elif waves:
+        scheme = SCHEME_WAVES
+        lds_fn = lambda t_, p_, r_, s_, cap_: max(lds_bytes_waves(pl.nc, pl.lognb, pl.tabn, WAVE_ROWS_PER_PASS, t_, p_, r_,
+                                                                  s_, cap_) for pl in plans)
+        threads, p, r, n_slabs, _, cap, lds = choose_wave_tiling(first.spr, class_rows, cap_fn, lds_fn,
                                                                  seg_len=first.seg_len, table_bytes=table)
     else:
         lds_fn = lambda p_, r_, cap_: max(lds_bytes(pl.nc, pl.lognb, pl.tabn, m, p_, first.seg_len, r_, cap_)
@@ -378,6 +456,5 @@ def plan_group(plans, m=None, gemm=False):
         tile_rows, tile_class = build_tiles(pl.row_class, pl.nr, r)
         tilings.append(dict(tile_rows=tile_rows, tile_class=tile_class,
                             scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                         n_tiles=len(tile_class), piece_cap=cap), lds=lds))
+                                         n_tiles=len(tile_class), piece_cap=cap, scheme=scheme), lds=lds))
     return tilings
-

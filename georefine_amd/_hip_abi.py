@@ -35,7 +35,7 @@ class GrfBctxFused(ctypes.Structure):
 class GrfFusedTiling(ctypes.Structure):
     _fields_ = [("tile_rows", ctypes.c_void_p), ("tile_class", ctypes.c_void_p)] + [
         (name, ctypes.c_uint32) for name in (
-            "threads", "lanes_per_row", "rows_per_tile", "n_slabs", "n_tiles", "piece_cap")]
+            "threads", "lanes_per_row", "rows_per_tile", "n_slabs", "n_tiles", "piece_cap", "scheme")]
 
 
 class GrfPpcxFused(ctypes.Structure):

@@ -13,11 +13,16 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import math
+import os
 
 import numpy as np
 
 from . import _fused, _hip_abi, _native, _tables
 from . import bitexact_context_codec as base
+
+# The GEMV's tiling scheme: wave units unless the environment asks for the slab kernels.
+GEMV_WAVES = os.environ.get("GEOREFINE_FUSED_GEMV", "waves") != "slabs"
+WAVE_ROWS = _fused.WAVE_ROWS_PER_PASS
 
 
 def _ptr(a, ctype):
@@ -260,12 +265,19 @@ class HipContextTensor:
         return other
 
     def _tiling(self, m):
-        """Device copy of the tiling used for m activation rows (0 = store sink); tilings
-        are made for m in {0, 1, 2, 4, 8} and shared by the row counts in between."""
+        """Device copy of the tiling used for m activation rows (0 = store sink).  The GEMV has
+        one wave-unit tiling for every row count; under GEOREFINE_FUSED_GEMV=slabs (experiments
+        and tests of the slab kernels) tilings are made for m in {1, 2, 4, 8} and shared by
+        the row counts in between."""
         import torch
-        bucket = 0 if m == 0 else next(v for v in (1, 2, 4, 8) if v >= m)
+        if m == 0:
+            bucket = 0
+        elif GEMV_WAVES:
+            bucket = "waves"
+        else:
+            bucket = next(v for v in (1, 2, 4, 8) if v >= m)
         if bucket not in self._tilings:
-            host = self._plan.tiling(bucket)
+            host = self._plan.tiling(WAVE_ROWS if bucket == "waves" else bucket, waves=bucket == "waves")
             rows = torch.from_numpy(host["tile_rows"]).to(self.device)
             classes = torch.from_numpy(host["tile_class"]).to(self.device)
             g = _hip_abi.GrfFusedTiling()
@@ -373,7 +385,7 @@ class HipContextTensor:
     def _fused_call(self, fn, tiling, x, bias, check, *, workspace=False):
         import torch
         lead = x.shape[:-1]
-        x2, bias, y = self._prepare_activations(x, bias, 4)
+        x2, bias, y = self._prepare_activations(x, bias, 8)
         if x2.shape[0]:
             if check:  # between checks the word keeps what earlier launches reported
                 self.error.zero_()
@@ -499,7 +511,8 @@ class HipLinearGroup:
         import torch
         if key not in self._tilings:
             plans = [t._plan for t in self.tensors]
-            hosts = _fused.plan_group(plans, gemm=True) if key == "gemm" else _fused.plan_group(plans, m=key)
+            hosts = (_fused.plan_group(plans, gemm=True) if key == "gemm"
+                     else _fused.plan_group(plans, m=key, waves=GEMV_WAVES))
             made = []
             for host in hosts:
                 rows = torch.from_numpy(host["tile_rows"]).to(self.device)
@@ -549,7 +562,7 @@ class HipLinearGroup:
             if x.dtype != torch.bfloat16 or x.shape[-1] != cols:
                 raise ValueError("activation must be bfloat16 with the weights' input width")
             x2 = x.reshape(-1, cols).to(self.device)
-            if x2.stride(-1) != 1 or x2.stride(0) % 4 or x2.data_ptr() % 8:
+            if x2.stride(-1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
                 x2 = x2.clone(memory_format=torch.contiguous_format)
         biases = [b.to(device=self.device, dtype=torch.bfloat16).contiguous() if b is not None else None for b in biases]
         outs = [torch.empty((m, t.shape[0]), device=self.device, dtype=torch.bfloat16) for t in self.tensors]

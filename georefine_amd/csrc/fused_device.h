@@ -134,17 +134,27 @@ __device__ __forceinline__ uint32_t fused_fetch_index(uint32_t state, uint32_t b
   const uint32_t bucket = (state & 0xFFFFu) >> q.shift;
   return lds_load_u8(block + bucket + q.table_bytes);
 }
-// Refill bytes are fetched ahead of need with two byte reads.  (An unaligned 16-bit LDS
-// read stalls the LDS pipeline for tens of cycles on this hardware; aligned dwords, or a
-// register window that follows the cursor, cost more instructions than they save.)
+// Refill bytes: one read of the two aligned dwords around the cursor serves two steps (they
+// take at most four bytes), and a funnel shift brings the byte at the cursor to the bottom:
+// `window` = stream bytes [ip, ip + 4), first byte lowest.  The lanes of a wave sit at
+// scattered places of their pieces, so byte-wide reads (two per step) collide in the banks
+// about as often as random addresses would, and were the largest share of the LDS time; a
+// quarter as many reads leave the lookup and the entry read as the main LDS work.  (An
+// unaligned 16- or 32-bit LDS read stalls the pipeline for tens of cycles on this hardware.)
+typedef __attribute__((address_space(3))) uint32_t lds_u32;
 template <int K>
-__device__ __forceinline__ void fused_fetch_bytes(StepFetch &s, const Cursor &c) {
-  // first byte above the second, as they enter the state (a byte permute: only the low
-  // byte of either register is looked at)
-  s.bytes = __builtin_amdgcn_perm(lds_load_u8(c.j + 2 * K), lds_load_u8(c.j + 2 * K + 1), 0x0c0c0400u);
+__device__ __forceinline__ void fused_fetch_window(StepFetch &s, const Cursor &c) {
+  static_assert(K % 2 == 0, "a window is read at even steps");
+  const uint32_t a = c.j & ~3u;  // 2K is a multiple of 4: it goes into the offset field
+  const uint32_t lo = *reinterpret_cast<lds_u32 *>(a + 2 * K), hi = *reinterpret_cast<lds_u32 *>(a + 2 * K + 4);
+  s.bytes = __builtin_amdgcn_alignbit(hi, lo, c.j << 3);  // the shift uses bits 0..4: (j & 3) * 8
 }
-// Keeps the combination of the two bytes in the block that loaded them: left alone, the
-// compiler sinks it past the scan branch and then re-masks both bytes there.
+// the window of the step after one that kept `keep` = 2 - (bytes taken)
+__device__ __forceinline__ void fused_next_window(StepFetch &s, const StepFetch &before, uint32_t keep) {
+  s.bytes = __builtin_amdgcn_alignbyte(0u, before.bytes, 2u - keep);
+}
+// Keeps the window in the block that made it: left alone, the compiler sinks the funnel shift
+// past the scan branch.
 __device__ __forceinline__ void fused_pin_bytes(StepFetch &s) {
 #if defined(__HIP_DEVICE_COMPILE__)
   asm volatile("" : "+v"(s.bytes));
@@ -199,8 +209,9 @@ __device__ __forceinline__ void fused_scan(uint32_t state, StepFetch &s, uint32_
 // state' = freq * (state >> 16) + rel, then the refill: n = 0, 1 or 2 bytes are shifted in
 // while the state is below 2^23.  Without branches or condition registers: the state is
 // below 2^31 and at least 2^7, so c = (24 - clz(state')) >> 3 = 2 - n; the byte selector of
-// v_perm that shifts n bytes in is a window, c bytes up, on the constant 00 01 04 05 06 07.
-__device__ __forceinline__ void fused_advance(Cursor &c, const StepFetch &s, uint32_t rel) {
+// v_perm that shifts n bytes of the window in (first stream byte highest) is a window, c
+// bytes up, on the constant 01 00 04 05 06 07.  Returns c.
+__device__ __forceinline__ uint32_t fused_advance(Cursor &c, const StepFetch &s, uint32_t rel) {
   uint32_t x;
 #if defined(__HIP_DEVICE_COMPILE__)
   asm("v_mad_u32_u16 %0, %1, %2, %3 op_sel:[1,1,0,0]" : "=v"(x) : "v"(s.e0.x), "v"(c.state), "v"(rel));
@@ -208,27 +219,17 @@ __device__ __forceinline__ void fused_advance(Cursor &c, const StepFetch &s, uin
   x = (s.e0.x >> 16) * (c.state >> 16) + rel;
 #endif
   const uint32_t keep = (24u - (uint32_t)__builtin_clz(x)) >> 3;
-  const uint32_t sel = __builtin_amdgcn_alignbyte(0x00000706u, 0x05040100u, keep);
+  const uint32_t sel = __builtin_amdgcn_alignbyte(0x00000706u, 0x05040001u, keep);
   c.state = __builtin_amdgcn_perm(x, s.bytes, sel);
   c.j -= keep;
+  return keep;
 }
 
-// One step (number K of its group of 16) of one segment, for the column class held in byte
-// BYTE of `ccw`.  Returns the image of the symbol's bits in the BF16 word (symbol << 5).
-template <int K>
-__device__ __forceinline__ uint32_t fused_symbol_in(Cursor &c, uint32_t block, const FusedParams &q);
-
-template <int K>
-__device__ __forceinline__ uint32_t fused_symbol(Cursor &c, uint32_t ccw, const FusedParams &q) {
-  return fused_symbol_in<K>(c, fused_block_offset<K % 4>(ccw, q.block_pitch), q);
-}
-
-// The step given the LDS offset `block` of its context's table block.
-template <int K>
-__device__ __forceinline__ uint32_t fused_symbol_in(Cursor &c, uint32_t block, const FusedParams &q) {
-  StepFetch s;
-  const uint32_t idx = fused_fetch_index(c.state, block, q);
-  fused_fetch_bytes<K>(s, c);
+// Two steps (numbers K and K + 1 of their group of 16, K even) of one segment, given the LDS
+// offsets of their contexts' table blocks.  Returns the images of the two symbols' bits in the
+// BF16 word (symbol << 5).
+__device__ __forceinline__ uint32_t fused_finish_step(Cursor &c, StepFetch &s, uint32_t idx, uint32_t block,
+                                                      uint32_t &keep) {
   fused_fetch_entry(s, idx, block);
   fused_pin_bytes(s);
   uint64_t miss;
@@ -237,8 +238,26 @@ __device__ __forceinline__ uint32_t fused_symbol_in(Cursor &c, uint32_t block, c
   if (__builtin_expect(miss != 0, 0)) {
     if (fused_lane_in(miss)) fused_scan(c.state, s, rel);
   }
-  fused_advance(c, s, rel);
+  keep = fused_advance(c, s, rel);
   return s.e0.y;
+}
+template <int K>
+__device__ __forceinline__ void fused_symbol_pair_in(Cursor &c, uint32_t block0, uint32_t block1, const FusedParams &q,
+                                                     uint32_t &hi0, uint32_t &hi1) {
+  StepFetch s0, s1;
+  uint32_t keep;
+  const uint32_t idx0 = fused_fetch_index(c.state, block0, q);
+  fused_fetch_window<K>(s0, c);
+  hi0 = fused_finish_step(c, s0, idx0, block0, keep);
+  const uint32_t idx1 = fused_fetch_index(c.state, block1, q);
+  fused_next_window(s1, s0, keep);
+  hi1 = fused_finish_step(c, s1, idx1, block1, keep);
+}
+template <int K>
+__device__ __forceinline__ void fused_symbol_pair(Cursor &c, uint32_t ccw, const FusedParams &q, uint32_t &hi0,
+                                                  uint32_t &hi1) {
+  fused_symbol_pair_in<K>(c, fused_block_offset<K % 4>(ccw, q.block_pitch), fused_block_offset<K % 4 + 1>(ccw, q.block_pitch),
+                          q, hi0, hi1);
 }
 
 // Sixteen packed 6-bit residuals (12 bytes, MSB first) -> field k, k compile-time, sign
@@ -266,18 +285,27 @@ struct Raw6x16 {
 
 // ---- pieces of the tile walk shared by the GEMV and GEMM kernels ----
 
-// this row class's lookup tables -> LDS, one block per column class: table, then lookup bytes
+// this row class's lookup tables -> LDS, one block per column class: table, then lookup bytes.
+// The copy is two flat loops over 16-byte and 8-byte units, unrolled so that a thread has
+// several loads in flight: copied one context after the other, load by load, the tables cost
+// a workgroup eight round trips to memory before its first step.
 __device__ __forceinline__ void fused_load_tables(uint8_t *lds, uint32_t blocks, uint32_t block_pitch,
                                                   const grf_bctx_fused &f, uint32_t cls, uint32_t tid,
                                                   uint32_t nthreads) {
-  const uint32_t nb = 1u << f.lognb, entries = f.tabn + 1;
-  for (uint32_t c = 0; c < f.nc; ++c) {
-    const uint4 *src = reinterpret_cast<const uint4 *>(f.lut + ((size_t)cls * f.nc + c) * nb);
-    uint4 *dst = reinterpret_cast<uint4 *>(lds + blocks + c * block_pitch + fused_table_bytes(f));
-    for (uint32_t i = tid; i < nb / 16; i += nthreads) dst[i] = src[i];
-    const uint2 *ts = reinterpret_cast<const uint2 *>(f.tab) + ((size_t)cls * f.nc + c) * entries;
-    uint2 *td = reinterpret_cast<uint2 *>(lds + blocks + c * block_pitch);
-    for (uint32_t i = tid; i < entries; i += nthreads) td[i] = ts[i];
+  const uint32_t nb16 = (1u << f.lognb) / 16, entries = f.tabn + 1, tb = fused_table_bytes(f);
+  const uint4 *lut = reinterpret_cast<const uint4 *>(f.lut + (size_t)cls * f.nc * (nb16 * 16));
+  const uint32_t n16 = f.nc * nb16;
+#pragma unroll 4
+  for (uint32_t i = tid; i < n16; i += nthreads) {
+    const uint32_t c = i / nb16, w = i % nb16;
+    *reinterpret_cast<uint4 *>(lds + blocks + c * block_pitch + tb + w * 16) = lut[i];
+  }
+  const uint2 *tab = reinterpret_cast<const uint2 *>(f.tab) + (size_t)cls * f.nc * entries;
+  const uint32_t n8 = f.nc * entries;
+#pragma unroll 2
+  for (uint32_t i = tid; i < n8; i += nthreads) {
+    const uint32_t c = i / entries, w = i % entries;
+    *reinterpret_cast<uint2 *>(lds + blocks + c * block_pitch + w * 8) = tab[i];
   }
 }
 
@@ -307,6 +335,34 @@ __device__ __forceinline__ uint32_t fused_stage_piece(uint8_t *lds, uint32_t pie
   return a0;
 }
 
+// The same copy made by one wave for itself (wave-unit tiling), without vector registers: the
+// loads write the LDS directly.  Such a load puts the 16 bytes of lane l at (base + 16 * l) of
+// a wave-uniform base, whatever address the lane read, so one instruction can fill 256
+// contiguous bytes of one row's piece from that row's 16-lane group (P lanes in general): the
+// rows take turns, each with the base that makes its lanes land on its own piece.  Round i
+// moves chunks [i * P, (i + 1) * P) of every row.  The bytes are in the LDS when the wave's
+// vector-memory counter says so; lanes of the same wave read them afterwards.
+__device__ __forceinline__ uint32_t fused_stage_piece_dma(uint8_t *lds, uint32_t region0, uint32_t cap,
+                                                          const grf_bctx_fused &f, uint32_t g0, uint32_t g1, uint32_t rl,
+                                                          uint32_t p, uint32_t P, uint32_t rows_per_wave) {
+  typedef __attribute__((address_space(3))) void lds_void;
+  const uint32_t a0 = g0 & ~15u;
+  // rounds the longest piece of the wave needs (uniform: every lane takes part in the ballots)
+  uint32_t longest = g1 > a0 ? g1 - a0 : 0;
+  for (uint32_t d = P; d < 64; d <<= 1) longest = max(longest, (uint32_t)__shfl_xor((int)longest, (int)d, 64));
+  const uint32_t rounds = (longest + P * 16 - 1) / (P * 16);
+  for (uint32_t i = 0; i < rounds; ++i) {
+    const uint32_t o = a0 + (i * P + p) * 16;
+    for (uint32_t r = 0; r < rows_per_wave; ++r) {  // uniform
+      // lane l = r * P + p of row r must land on region(r) + (i * P + p) * 16
+      const uint32_t base = region0 + r * cap + i * P * 16 - r * P * 16;
+      if (rl == r && o < g1)
+        __builtin_amdgcn_global_load_lds(f.main_bytes + o, (lds_void *)(lds + base), 16, 0, 0);
+    }
+  }
+  return a0;
+}
+
 // BF16 word in bits 0..15 (bits above are unspecified): symbol bits | mantissa low 5 bits
 // | sign << 15, from the sign-extended residual field: its copy of the sign at bit 15 and
 // its low five bits are kept, one and-or.
@@ -323,7 +379,8 @@ template <bool AHEAD>
 struct SegmentWalkT {
   static constexpr bool kAhead = AHEAD;
   Cursor c;
-  uint32_t ip0, gofs, seg;
+  uint32_t gofs, eofs;        // byte offsets of this segment's and the next segment's checkpoints
+  uint32_t end_state, end_j;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
   const uint32_t *rawp;
   const uint4 *ccp;
   uint32_t n0, n1, n2;             // !AHEAD: the next group's residual words
@@ -335,9 +392,10 @@ struct SegmentWalkT {
   // Global reads for segment `seg_` (elem0 / col0: its first element / column), issued
   // before the workgroup waits for the slab's stream bytes so that their latency overlaps it.
   __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t col0) {
-    seg = seg_;
-    gofs = f.seg_offset[seg];
-    c.state = f.seg_state[seg];
+    gofs = f.seg_offset[seg_];
+    eofs = f.seg_offset[seg_ + 1];
+    c.state = f.seg_state[seg_];
+    end_state = f.seg_state[seg_ + 1];
     rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
     ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
     if constexpr (AHEAD) {
@@ -355,8 +413,8 @@ struct SegmentWalkT {
   }
   // the row piece was staged at piece_off from global offset a0
   __device__ __forceinline__ void start(uint32_t piece_off, uint32_t a0) {
-    ip0 = piece_off + (gofs - a0);
-    c.j = ip0;
+    c.j = piece_off + (gofs - a0);
+    end_j = c.j + (eofs - gofs);
   }
 
   // Start the group of symbols [t, t+16): unpack its residuals and column classes, and load
@@ -386,9 +444,15 @@ struct SegmentWalkT {
   template <int H>
   __device__ __forceinline__ void half(const FusedParams &q, uint32_t (&pair)[4]) {
     uint32_t bits[8];
-#define GRF_STEP(i) bits[i] = fused_word_bits(fused_symbol<8 * H + (i)>(c, cw[(8 * H + (i)) / 4], q), rr.field<8 * H + (i)>());
-    GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
-#undef GRF_STEP
+#define GRF_STEP2(i)                                                                   \
+  {                                                                                    \
+    uint32_t h0, h1;                                                                   \
+    fused_symbol_pair<8 * H + (i)>(c, cw[(8 * H + (i)) / 4], q, h0, h1);               \
+    bits[i] = fused_word_bits(h0, rr.field<8 * H + (i)>());                            \
+    bits[(i) + 1] = fused_word_bits(h1, rr.field<8 * H + (i) + 1>());                  \
+  }
+    GRF_STEP2(0) GRF_STEP2(2) GRF_STEP2(4) GRF_STEP2(6)
+#undef GRF_STEP2
     if (H == 1) c.end_group();
 #pragma unroll
     for (int k = 0; k < 4; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
@@ -402,7 +466,8 @@ struct SegmentWalkT {
 
   // the segment must end exactly on the next checkpoint
   __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
-    return c.state == f.seg_state[seg + 1] && gofs + (c.j - ip0) == f.seg_offset[seg + 1];
+    (void)f;
+    return c.state == end_state && c.j == end_j;
   }
 };
 using SegmentWalk = SegmentWalkT<false>;

@@ -34,7 +34,8 @@
 
 namespace grf {
 int set_error(int code, const std::string &what);                                          // decode_general.hip
-int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who);  // fused_gemv.hip
+// fused_gemv.hip; wave_units: the entry point takes GRF_TILE_WAVES tilings
+int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who, bool wave_units = false);
 
 // A kernel may ask for more than 64 KiB of dynamic LDS only after its limit has been raised;
 // done once per kernel and device (not per launch: it is a driver call, and a launch that
@@ -220,6 +221,216 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
   if (bad) atomicOr(error, (int)bad);
 }
 
+// ---------------------------------------------------------------- GEMV over wave units
+//
+// GRF_TILE_WAVES: the unit of work is one wave: 64/P rows of the tile by P segments (one
+// "slab" of the rows).  A wave copies the stream pieces of its rows itself, reads the
+// activations straight from memory (they are small and stay in the caches), walks, and folds
+// its rows' segment partials; the waves of a workgroup take the tile's units in turn and
+// never wait for each other until the row sums are put together at the end.  What the
+// slab-synchronous tiling loses -- every wave waiting for the slowest at two barriers per
+// slab, copies that nothing overlaps because the workgroups of a compute unit run in step,
+// lanes without a segment -- this one keeps busy: while one wave waits for its bytes the
+// others walk.
+//
+// Reduction order of one output element: the S products of a segment as in the other GEMV;
+// the P segment partials of a unit pairwise, neighbours first (lane distances 1, 2, 4, ...);
+// the units' sums of a row in slab order; bias; one rounding.  The tiling fixes P per matrix,
+// and more than two activation rows run as passes of two, so the order depends neither on the
+// activation row count nor on how rows are dealt to workgroups.
+struct WaveLdsLayout {
+  uint32_t blocks, block_pitch, stream, sub, rows, total;
+  __host__ __device__ WaveLdsLayout(const grf_bctx_fused &f, const grf_fused_tiling &g, uint32_t m) {
+    const uint32_t waves = g.threads / 64, rpw = 64 / g.lanes_per_row;
+    blocks = 0;
+    block_pitch = grf::fused_table_bytes(f) + (1u << f.lognb);
+    stream = grf::align_up(f.nc * block_pitch, 16);                   // [waves][64 / P] row pieces
+    sub = grf::align_up(stream + waves * rpw * g.piece_cap, 16);      // [rows_per_tile][n_slabs][m] unit sums
+    rows = grf::align_up(sub + g.rows_per_tile * g.n_slabs * m * 4, 16);  // [rows_per_tile] the tile's rows
+    total = grf::align_up(rows + g.rows_per_tile * 4, 16);
+  }
+};
+
+template <class Walk, int M>
+__device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fused &f, const grf_fused_tiling &g,
+                                                const uint16_t *x, uint32_t ldx, uint16_t *y, uint32_t ldy,
+                                                const uint16_t *bias, int32_t *error, uint32_t tile) {
+  const WaveLdsLayout L(f, g, M);
+  const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
+  const uint32_t wave = tid / 64, lane = tid % 64, nwaves = nthreads / 64;
+  const uint32_t P = g.lanes_per_row, rpw = 64 / P, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
+  const uint32_t cls = g.tile_class[tile];
+  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
+  const uint32_t rl = lane / P, p = lane % P;
+  float *sub = reinterpret_cast<float *>(lds + L.sub);
+  uint32_t *rows = reinterpret_cast<uint32_t *>(lds + L.rows);
+  const uint32_t piece_off = L.stream + (wave * rpw + rl) * g.piece_cap;
+  const uint32_t groups = (R + rpw - 1) / rpw, units = groups * g.n_slabs;
+  uint32_t bad = 0;
+
+  // The byte range [g0, g1) of a unit's row piece is the first of two dependent reads before
+  // the piece can be copied, so it is read one unit ahead (and the first one before the
+  // tables are copied).
+  auto span_of = [&](uint32_t u, uint32_t row, uint32_t &g0, uint32_t &g1) {
+    g0 = g1 = 0;
+    if (row == grf::kNoRow) return;
+    const uint32_t first_seg = (u % g.n_slabs) * P;
+    const uint32_t seg_base = row * f.segs_per_row + first_seg;
+    g0 = f.seg_offset[seg_base];
+    g1 = f.seg_offset[seg_base + min(P, f.segs_per_row - first_seg)];
+  };
+  uint32_t row, g0, g1;
+  {
+    const uint32_t slot0 = (wave / g.n_slabs) * rpw + rl;
+    row = (wave < units && slot0 < R) ? g.tile_rows[tile * R + slot0] : grf::kNoRow;
+    if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
+    span_of(wave, row, g0, g1);
+  }
+  for (uint32_t i = tid; i < R; i += nthreads) {
+    const uint32_t rw = g.tile_rows[tile * R + i];
+    rows[i] = rw < f.rows ? rw : grf::kNoRow;
+  }
+  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
+  __syncthreads();
+  for (uint32_t u = wave; u < units; u += nwaves) {  // wave-uniform
+#if defined(__HIP_DEVICE_COMPILE__)
+    // Waves with more units still to do go first.  Left alone the arbiter prefers the older
+    // of the two workgroups that share a compute unit, which then finishes long before the
+    // other and leaves it the unit at half occupancy.
+    switch (min(3u, (units - 1 - u) / nwaves + (blockIdx.x >= gridDim.x / 2 ? 1u : 0u))) {  // + the later-started half
+      case 0: __builtin_amdgcn_s_setprio(0); break;
+      case 1: __builtin_amdgcn_s_setprio(1); break;
+      case 2: __builtin_amdgcn_s_setprio(2); break;
+      default: __builtin_amdgcn_s_setprio(3); break;
+    }
+#endif
+    const uint32_t slot = (u / g.n_slabs) * rpw + rl, b = u % g.n_slabs;
+    const uint32_t first_seg = b * P;
+    const uint32_t nseg = min(P, f.segs_per_row - first_seg);
+    if (u != wave) row = slot < R ? rows[slot] : grf::kNoRow;  // (read again: cheaper than a register over the walk)
+    const bool walks = row != grf::kNoRow && p < nseg;
+    const uint32_t col0 = (first_seg + p) * S;
+    Walk w;
+    if (walks) w.prefetch(f, row * f.segs_per_row + first_seg + p, (uint64_t)row * K + col0, col0);
+    const uint32_t a0 = grf::fused_stage_piece_dma(lds, L.stream + wave * rpw * g.piece_cap, g.piece_cap, f, g0, g1, rl, p, P, rpw);
+    if (walks) w.start(piece_off, a0);
+    {  // the next unit's byte range, on its way during this unit's walk
+      const uint32_t un = u + nwaves, sn = (un / g.n_slabs) * rpw + rl;
+      span_of(un, (un < units && sn < R) ? rows[sn] : grf::kNoRow, g0, g1);
+    }
+    __builtin_amdgcn_wave_barrier();
+    float acc[M];
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[m] = 0.f;
+    if (walks) {
+      uint4 xn[M][2];  // the activations of the next group of 16 columns
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const uint4 *xm = reinterpret_cast<const uint4 *>(x + (size_t)m * ldx + col0);
+        xn[m][0] = xm[0];
+        xn[m][1] = xm[1];
+      }
+      for (uint32_t t = 0; t < S; t += 16) {
+        uint32_t xv[M][8];
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          xv[m][0] = xn[m][0].x, xv[m][1] = xn[m][0].y, xv[m][2] = xn[m][0].z, xv[m][3] = xn[m][0].w;
+          xv[m][4] = xn[m][1].x, xv[m][5] = xn[m][1].y, xv[m][6] = xn[m][1].z, xv[m][7] = xn[m][1].w;
+          // the last group loads itself again rather than branch around the loads
+          const uint4 *xm = reinterpret_cast<const uint4 *>(x + (size_t)m * ldx + col0 + min(t + 16, S - 16));
+          xn[m][0] = xm[0];
+          xn[m][1] = xm[1];
+        }
+        uint32_t pair[8];
+        w.decode16(t, S, q, pair);
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+#pragma unroll
+          for (int k = 0; k < 8; ++k) acc[m] = dot2_bf16(pair[k], xv[m][k], acc[m]);
+      }
+      if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
+    }
+    // The unit's sum of a row: its P segment partials (0 for lanes without a segment) added
+    // pairwise, neighbours first -- lane distances 1, 2, 4, ... -- in every lane at once.
+    {
+      // (the lane's coordinates are worked out again rather than kept in registers over the walk)
+      uint32_t ln = __lane_id();
+#if defined(__HIP_DEVICE_COMPILE__)
+      asm volatile("" : "+v"(ln));
+#endif
+      const uint32_t p2 = ln % P, slot2 = (u / g.n_slabs) * rpw + ln / P;
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float sum = acc[m];
+        for (uint32_t d = 1; d < P; d <<= 1) sum += __shfl_xor(sum, d, 64);
+        if (p2 == 0 && slot2 < R) sub[(slot2 * g.n_slabs + u % g.n_slabs) * M + m] = sum;
+      }
+    }
+  }
+  __syncthreads();
+  for (uint32_t i = tid; i < R * M; i += nthreads) {
+    const uint32_t rr = i / M, m = i % M;
+    const uint32_t orow = rows[rr];
+    if (orow == grf::kNoRow) continue;
+    const float *sp = sub + (rr * g.n_slabs) * M + m;
+    float sum = sp[0];
+    for (uint32_t b = 1; b < g.n_slabs; ++b) sum += sp[b * M];
+    if (bias) sum += __uint_as_float((uint32_t)bias[orow] << 16);
+    y[(size_t)m * ldy + orow] = round_bf16(sum);
+  }
+  if (bad) atomicOr(error, (int)bad);
+}
+
+template <class Walk, int M>
+__global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_wave_kernel(
+    grf_bctx_fused f, grf_fused_tiling g, const uint16_t *x, uint32_t ldx, uint16_t *y, uint32_t ldy,
+    const uint16_t *bias, int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  fused_wave_body<Walk, M>(lds, f, g, x, ldx, y, ldy, bias, error, blockIdx.x);
+}
+
+template <class Walk, int M>
+int launch_wave(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint16_t *y,
+                uint32_t ldy, const uint16_t *bias, int32_t *error, hipStream_t s) {
+  const WaveLdsLayout L(f, g, M);
+  if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
+  constexpr auto kernel = &fused_wave_kernel<Walk, M>;
+  if (L.total > 64 * 1024)
+    if (int rc = allow_full_lds<kernel>()) return rc;
+  hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, x, ldx, y, ldy, bias, error);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
+  return GRF_OK;
+}
+
+// The wave-unit GEMV keeps the activations of a group of columns in registers: two rows per
+// pass.  More rows run as further passes over the matrix with exactly the same arithmetic per
+// row; batches beyond two belong to the matrix-core GEMM anyway.
+constexpr uint32_t kWaveRowsPerPass = 2;
+
+inline int check_wave_operands(const char *who, const grf_bctx_fused &f, const uint16_t *x, uint32_t ldx) {
+  if ((ldx & 7) || ((uintptr_t)x & 15))
+    return grf::set_error(GRF_BAD_ARGUMENT,
+                          std::string(who) + ": wave units read x in 16-byte vectors (aligned, ldx a multiple of 8)");
+  if (f.seg_len % 16 || f.cols % 16) return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": segment length");
+  return GRF_OK;
+}
+
+template <class Walk>
+int launch_wave_rows(const char *who, const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx,
+                     uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error, hipStream_t s) {
+  if (int rc = check_wave_operands(who, f, x, ldx)) return rc;
+  for (uint32_t m0 = 0; m0 < m_rows; m0 += kWaveRowsPerPass) {
+    const uint16_t *xs = x + (size_t)m0 * ldx;
+    uint16_t *ys = y + (size_t)m0 * ldy;
+    const int rc = m_rows - m0 == 1 ? launch_wave<Walk, 1>(f, g, xs, ldx, ys, ldy, bias, error, s)
+                                    : launch_wave<Walk, 2>(f, g, xs, ldx, ys, ldy, bias, error, s);
+    if (rc) return rc;
+  }
+  return GRF_OK;
+}
+
+
 // Six waves per SIMD keep two 768-lane workgroups on a compute unit: the store sinks, which
 // hold decoded words back, would otherwise take a few registers too many for that.
 template <class Walk, int M, int SINK>
@@ -264,6 +475,14 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_group_kernel
                                  blockIdx.x - a.first_tile[i]);
 }
 
+template <class Walk, int M>
+__global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_wave_group_kernel(
+    FusedGroup a, const uint16_t *x, uint32_t ldx, int32_t *error) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t i = group_member(a, blockIdx.x);
+  fused_wave_body<Walk, M>(lds, a.f[i], a.g[i], x, ldx, a.y[i], a.ldy[i], a.bias[i], error, blockIdx.x - a.first_tile[i]);
+}
+
 template <class Walk, int M, int SINK>
 int launch_walk(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx,
                 uint16_t *y,
@@ -288,6 +507,7 @@ int launch_gemv(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
     return grf::set_error(GRF_BAD_ARGUMENT,
                           std::string(who) + ": x must be 4-byte aligned with an even leading dimension");
   using Ahead = typename ahead_of<Walk>::type;
+  if (g.scheme == GRF_TILE_WAVES) return launch_wave_rows<Walk>(who, f, g, x, ldx, m_rows, y, ldy, bias, error, s);
   if (!std::is_same<Ahead, Walk>::value && reads_ahead(f) && m_rows <= kAheadMaxRows) switch (m_rows) {
       case 1: return launch_walk<Ahead, 1, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
       case 2: return launch_walk<Ahead, 2, kDot>(f, g, x, ldx, y, ldy, bias, nullptr, error, s);
@@ -636,9 +856,10 @@ inline int build_group(const char *who, const GroupSpec &spec, bool gemm, FusedG
     if (!spec.frames[i] || !spec.tilings[i] || !spec.y[i]) return bad("null member");
     const grf_bctx_fused &f = *spec.frames[i];
     const grf_fused_tiling &g = *spec.tilings[i];
-    if (int rc = grf::check_fused_frame(f, g, who)) return rc;
+    if (int rc = grf::check_fused_frame(f, g, who, !gemm)) return rc;
     if (f.cols != spec.frames[0]->cols) return bad("members must have one width");
     if (g.threads != spec.tilings[0]->threads) return bad("member tilings must share one thread count");
+    if (g.scheme != spec.tilings[0]->scheme) return bad("member tilings must share one scheme");
     if (gemm && GemmShape(g).threads != g.threads)
       return bad("tiling threads must be 64 x ceil(rows_per_tile / 16) x ceil(lanes_per_row / 4)");
     if (spec.ldy[i] < f.rows) return bad("ldy is smaller than the row count");
@@ -676,6 +897,29 @@ int launch_gemv_group(const char *who, const GroupSpec &spec, const uint16_t *x,
   if (!x || ldx < a.f[0].cols || (ldx & 1) || ((uintptr_t)x & 3))
     return grf::set_error(GRF_BAD_ARGUMENT,
                           std::string(who) + ": x must be 4-byte aligned with an even leading dimension");
+  if (a.g[0].scheme == GRF_TILE_WAVES) {
+    uint32_t lds = 0;
+    for (uint32_t i = 0; i < a.n; ++i) {
+      if (int rc = check_wave_operands(who, a.f[i], x, ldx)) return rc;
+      lds = std::max(lds, WaveLdsLayout(a.f[i], a.g[i], kWaveRowsPerPass).total);
+    }
+    if (lds > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
+    for (uint32_t m0 = 0; m0 < m_rows; m0 += kWaveRowsPerPass) {
+      FusedGroup part = a;
+      for (uint32_t i = 0; i < a.n; ++i) part.y[i] = a.y[i] + (size_t)m0 * a.ldy[i];
+      const uint16_t *xs = x + (size_t)m0 * ldx;
+      const bool one = m_rows - m0 == 1;
+      constexpr auto k1 = &fused_wave_group_kernel<Walk, 1>;
+      constexpr auto k2 = &fused_wave_group_kernel<Walk, 2>;
+      if (lds > 64 * 1024)
+        if (int rc = one ? allow_full_lds<k1>() : allow_full_lds<k2>()) return rc;
+      if (one) hipLaunchKernelGGL(k1, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, part, xs, ldx, error);
+      else hipLaunchKernelGGL(k2, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, part, xs, ldx, error);
+      hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
+    }
+    return GRF_OK;
+  }
   using Ahead = typename ahead_of<Walk>::type;
   bool ahead = !std::is_same<Ahead, Walk>::value && m_rows <= kAheadMaxRows;
   for (uint32_t i = 0; i < a.n; ++i) ahead = ahead && reads_ahead(a.f[i]);

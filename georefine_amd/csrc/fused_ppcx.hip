@@ -102,7 +102,8 @@ struct Raw5x16 {
 
 struct PpcxWalk {
   grf::Cursor c;
-  uint32_t ip0, gofs, seg;
+  uint32_t gofs, eofs;        // byte offsets of this segment's and the next segment's checkpoints
+  uint32_t end_state, end_j;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
   const uint8_t *rawp;    // the segment's first residual byte (5 * S / 8 bytes per segment)
   const uint2 *binp;      // the segment's bins, 8 bytes per 16 symbols
   uint32_t n0, n1, n2;
@@ -115,9 +116,10 @@ struct PpcxWalk {
   }
   // global reads of the segment, issued before the wait for the slab's stream bytes
   __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t) {
-    seg = seg_;
-    gofs = f.seg_offset[seg];
-    c.state = f.seg_state[seg];
+    gofs = f.seg_offset[seg_];
+    eofs = f.seg_offset[seg_ + 1];
+    c.state = f.seg_state[seg_];
+    end_state = f.seg_state[seg_ + 1];
     rawp = f.raw6 + elem0 / 8 * 5;
     binp = reinterpret_cast<const uint2 *>(f.col_class) + elem0 / 16;
     const uint32_t *d = group_dwords(rawp, 0);
@@ -127,8 +129,8 @@ struct PpcxWalk {
     nb = binp[0];
   }
   __device__ __forceinline__ void start(uint32_t piece_off, uint32_t a0) {
-    ip0 = piece_off + (gofs - a0);
-    c.j = ip0;
+    c.j = piece_off + (gofs - a0);
+    end_j = c.j + (eofs - gofs);
   }
 
   __device__ __forceinline__ void begin16(uint32_t t, uint32_t S) {
@@ -146,14 +148,17 @@ struct PpcxWalk {
   template <int H>
   __device__ __forceinline__ void half(const grf::FusedParams &q, uint32_t (&pair)[4]) {
     uint32_t bits[8];
-#define GRF_STEP(i)                                                                                   \
+#define GRF_STEP2(i)                                                                                  \
   {                                                                                                   \
-    const uint32_t bin = __builtin_amdgcn_ubfe(bw[H], 4 * (i), 4);                                    \
-    const uint32_t hi = grf::fused_symbol_in<8 * H + (i)>(c, __umul24(bin, q.block_pitch), q);        \
-    bits[i] = hi | rr.field<8 * H + (i)>();                                                           \
+    const uint32_t bin0 = __builtin_amdgcn_ubfe(bw[H], 4 * (i), 4);                                   \
+    const uint32_t bin1 = __builtin_amdgcn_ubfe(bw[H], 4 * (i) + 4, 4);                               \
+    uint32_t h0, h1;                                                                                  \
+    grf::fused_symbol_pair_in<8 * H + (i)>(c, __umul24(bin0, q.block_pitch), __umul24(bin1, q.block_pitch), q, h0, h1); \
+    bits[i] = h0 | rr.field<8 * H + (i)>();                                                           \
+    bits[(i) + 1] = h1 | rr.field<8 * H + (i) + 1>();                                                 \
   }
-    GRF_STEP(0) GRF_STEP(1) GRF_STEP(2) GRF_STEP(3) GRF_STEP(4) GRF_STEP(5) GRF_STEP(6) GRF_STEP(7)
-#undef GRF_STEP
+    GRF_STEP2(0) GRF_STEP2(2) GRF_STEP2(4) GRF_STEP2(6)
+#undef GRF_STEP2
     if (H == 1) c.end_group();
 #pragma unroll
     for (int k = 0; k < 4; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
@@ -165,7 +170,8 @@ struct PpcxWalk {
   }
 
   __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
-    return c.state == f.seg_state[seg + 1] && gofs + (c.j - ip0) == f.seg_offset[seg + 1];
+    (void)f;
+    return c.state == end_state && c.j == end_j;
   }
 };
 

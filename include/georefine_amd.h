@@ -162,9 +162,10 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  *   lut         u8  [nr][nc << lognb]        lognb = 16 - shift; sparse index of a
  *                                            symbol with slots in the bucket (best: the
  *                                            one owning most of them)
- *   tab         u64 [nr][nc][tabn+1]         entry(cc, sparse): low32 = start |
- *                                            (freq & 0xFFFF)<<16 (0 stands for 65536),
- *                                            high32 = symbol<<5; unused entries: 0
+ *   tab         u32 [nr][nc][tabn+1][4]      entry(cc, sparse): start | (freq & 0xFFFF)<<16
+ *                                            (0 stands for 65536); symbol<<5; then (freq<<16 |
+ *                                            symbol<<5) of the previous and of the next live
+ *                                            symbol of the context (0: none); unused entries: 0
  *   col_class   u8  [cols]
  * main_bytes must be readable for 16 bytes past main_n_bytes.  raw6 is 4-byte aligned;
  * with seg_len 64 and 16-byte alignment the GEMV reads a segment's 48 residual bytes
@@ -185,18 +186,28 @@ typedef struct grf_bctx_fused {
 } grf_bctx_fused;
 
 /* How a launch cuts the frame into workgroups.  A tile is up to rows_per_tile rows of
- * one row class; lane (r, p) of the workgroup walks segment b*lanes_per_row + p of the
- * tile's row r in slab b.  threads >= rows_per_tile*lanes_per_row, a multiple of 64,
- * at most 1024.
+ * one row class; threads is a multiple of 64, at most 1024.
  *   tile_rows   u32 [n_tiles*rows_per_tile]  row of each slot, 0xFFFFFFFF = empty
  *   tile_class  u8  [n_tiles]                row class shared by the tile's rows
- *   piece_cap   LDS bytes reserved per row piece of one slab (multiple of 16) */
+ *   piece_cap   LDS bytes reserved per row piece of one slab (multiple of 16)
+ *   scheme      GRF_TILE_SLABS: lane (r, p) of the workgroup walks segment b*lanes_per_row + p
+ *               of the tile's row r in slab b, the whole workgroup slab by slab
+ *               (threads >= rows_per_tile*lanes_per_row).
+ *               GRF_TILE_WAVES (GEMV only): a wave is a unit of 64/lanes_per_row rows by
+ *               lanes_per_row segments (lanes_per_row a power of two, 4..64); the waves of
+ *               the workgroup take the tile's units (row group g, slab b) in turn and share
+ *               nothing but the lookup tables, so there is no barrier between the table copy
+ *               and the final row sums.
+ * n_slabs = ceil(segs_per_row / lanes_per_row) in both schemes. */
+#define GRF_TILE_SLABS 0
+#define GRF_TILE_WAVES 1
 typedef struct grf_fused_tiling {
   const uint32_t *tile_rows;
   const uint8_t *tile_class;
   uint32_t threads;
   uint32_t lanes_per_row, rows_per_tile, n_slabs, n_tiles;
   uint32_t piece_cap;
+  uint32_t scheme;
 } grf_fused_tiling;
 
 /* Fused decode-GEMV, the slot the reference leaves for "a backend with a fused GEMM"
@@ -271,8 +282,8 @@ uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_t
  *   main_bytes  the frame's main rANS stream, readable for 16 bytes past main_n_bytes
  *   raw5        packed 5-bit residuals, MSB first, readable for 16 bytes past the end
  *   seg_state / seg_offset  as in grf_bctx_fused, contexts label[row]*16 + bin
- *   lut  u8 [n_labels][16 << lognb], tab u64 [n_labels][16][tabn+1]   as in grf_bctx_fused,
- *        entry high32 = the symbol's bits in the BF16 word (sign, exponent, mantissa 6..5)
+ *   lut  u8 [n_labels][16 << lognb], tab u32 [n_labels][16][tabn+1][4]   as in grf_bctx_fused,
+ *        with the symbol's bits in the BF16 word (sign, exponent, mantissa 6..5) for symbol<<5
  * seg_len must be a multiple of 32.  Tilings are built over row labels. */
 typedef struct grf_ppcx_fused {
   const uint8_t *main_bytes;

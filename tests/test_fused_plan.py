@@ -60,7 +60,8 @@ def test_lookup_tables_resolve_every_slot(classes):
 def test_tilings_cover_each_row_once_with_one_class_per_tile(shape):
     words = weight_like(np.random.default_rng(shape[0]), *shape)
     ix, plan = _plan(words)
-    tilings = [plan.tiling(m) for m in (0, 1, 8)] + [plan.gemm_tiling()]
+    tilings = [plan.tiling(m) for m in (0, 1, 8)] + [plan.tiling(1, waves=True), plan.gemm_tiling()]
+    assert plan.tiling(0, waves=True)["scalars"]["scheme"] == _fused.SCHEME_SLABS  # the store sink has no wave units
     for t in tilings:
         s = t["scalars"]
         rows = t["tile_rows"].reshape(s["n_tiles"], s["rows_per_tile"])
@@ -69,15 +70,22 @@ def test_tilings_cover_each_row_once_with_one_class_per_tile(shape):
         for tile, cls in zip(rows, t["tile_class"]):
             members = tile[tile != 0xFFFFFFFF]
             assert members.size and np.all(ix["rows"][members] == cls)
-        assert s["threads"] % 64 == 0 and s["lanes_per_row"] * s["rows_per_tile"] <= s["threads"] <= 1024
+        assert s["threads"] % 64 == 0 and s["threads"] <= 1024
+        if s["scheme"] == _fused.SCHEME_WAVES:  # a wave walks 64 / P rows of P segments at a time
+            assert s["lanes_per_row"] in (4, 8, 16, 32, 64) and 1 <= s["rows_per_tile"]
+            assert t is tilings[3] and t["lds"] == _fused.lds_bytes_waves(
+                plan.nc, plan.lognb, plan.tabn, 2, s["threads"], s["lanes_per_row"], s["rows_per_tile"], s["n_slabs"],
+                s["piece_cap"])
+        else:
+            assert s["lanes_per_row"] * s["rows_per_tile"] <= s["threads"]
         assert s["n_slabs"] == -(-plan.spr // s["lanes_per_row"])
         assert t["lds"] <= _fused.MAX_LDS
-        # a row piece of any slab fits its LDS slot together with the two bytes read ahead
+        # a row piece of any slab fits its LDS slot together with the window the refill reads
         off = plan.seg_offset.astype(np.int64)
         for b in range(s["n_slabs"]):
             first = np.arange(shape[0]) * plan.spr + b * s["lanes_per_row"]
             last = first + min(s["lanes_per_row"], plan.spr - b * s["lanes_per_row"])
-            assert np.max(off[last] - (off[first] & ~15)) + 2 <= s["piece_cap"]
+            assert np.max(off[last] - (off[first] & ~15)) + 8 <= s["piece_cap"]
     g = tilings[-1]["scalars"]
     waves, blocks = g["threads"] // 64, -(-g["rows_per_tile"] // 16)
     assert blocks <= waves and -(-8 // (waves // blocks)) <= 4
@@ -170,6 +178,19 @@ def test_planner_takes_the_fewest_slabs_among_tilings_it_scores_alike(monkeypatc
     assert lds * 2 <= _fused.MAX_LDS  # two workgroups per compute unit
 
 
+def test_wave_planner_on_the_benchmark_shapes(monkeypatch):
+    """17408 x 5120 and 5120 x 17408 in four row classes: two workgroups of twelve waves per
+    compute unit, one round of workgroups, the units of a tile shared out evenly."""
+    monkeypatch.delenv("GEOREFINE_FUSED_WAVE_TILING", raising=False)
+    for rows, spr, want in ((17408, 80, (768, 16, 34)), (5120, 272, (768, 32, 10))):
+        cap = lambda lanes: (16 + 54 * lanes + 8 + 15) // 16 * 16
+        lds = lambda t, p, r, s, c: _fused.lds_bytes_waves(16, 9, 200, 2, t, p, r, s, c)
+        threads, p, r, n_slabs, n_tiles, _, total = _fused.choose_wave_tiling(
+            spr, np.asarray([rows // 4] * 4), cap, lds, seg_len=64, table_bytes=53 * 1024)
+        assert (threads, p, r) == want and n_tiles == 512 and n_slabs == -(-spr // p)
+        assert total * 2 <= _fused.MAX_LDS
+
+
 def test_group_plans_share_one_tile_shape_and_keep_every_member_complete():
     rng = np.random.default_rng(5)
     plans, frames = [], []
@@ -177,8 +198,9 @@ def test_group_plans_share_one_tile_shape_and_keep_every_member_complete():
         ix, plan = _plan(weight_like(rng, rows, 640))
         plans.append(plan)
         frames.append(ix)
-    for kwargs in (dict(m=1), dict(m=8), dict(gemm=True)):
+    for kwargs in (dict(m=1), dict(m=8), dict(m=2, waves=True), dict(gemm=True)):
         tilings = _fused.plan_group(plans, **kwargs)
+        assert {t["scalars"]["scheme"] for t in tilings} == {int(bool(kwargs.get("waves")))}
         shapes = {(t["scalars"]["threads"], t["scalars"]["lanes_per_row"], t["scalars"]["rows_per_tile"],
                    t["scalars"]["n_slabs"], t["scalars"]["piece_cap"]) for t in tilings}
         assert len(shapes) == 1 and len(tilings) == 3
