@@ -116,16 +116,14 @@ __device__ __forceinline__ uint32_t fused_lshl3_add(uint32_t a, uint32_t b) {  /
 // boundary inside the bucket, or the 16-bit frequency field's 0 = 65536) scans to the
 // neighbouring entries before the state update, which all lanes then do together.
 struct StepFetch {
-  uint32_t bytes, ta;  // the two possible refill bytes (first << 8 | second), table address of the entry
+  uint32_t win, ta;  // the next four stream bytes, first byte highest; table address of the entry
   v2u32 e0;
 };
 
-// A lane's position in one segment: rANS state and LDS byte cursor.  The cursor is kept
-// as j = ip - 2k at step k of a 16-step group, so that a step that takes n bytes subtracts
-// 2 - n and the byte reads carry 2k in their offset field.
+// A lane's position in one segment: rANS state and LDS cursor, the cursor in bits (eight times
+// the byte address), which is the unit the refill's shift count comes in.
 struct Cursor {
-  uint32_t state, j;
-  __device__ __forceinline__ void end_group() { j += 32; }  // after 16 steps: j is ip again
+  uint32_t state, jb;
 };
 
 // `block` is the LDS offset of the column class's block (fused_block_offset).  The LDS
@@ -135,29 +133,25 @@ __device__ __forceinline__ uint32_t fused_fetch_index(uint32_t state, uint32_t b
   return lds_load_u8(block + bucket + q.table_bytes);
 }
 // Refill bytes: one read of the two aligned dwords around the cursor serves two steps (they
-// take at most four bytes), and a funnel shift brings the byte at the cursor to the bottom:
-// `window` = stream bytes [ip, ip + 4), first byte lowest.  The lanes of a wave sit at
-// scattered places of their pieces, so byte-wide reads (two per step) collide in the banks
-// about as often as random addresses would, and were the largest share of the LDS time; a
-// quarter as many reads leave the lookup and the entry read as the main LDS work.  (An
+// take at most four bytes); a funnel shift brings the byte at the cursor to the bottom and a
+// byte permute turns the four around, so that `win` = stream bytes [ip, ip + 4) with the first
+// byte highest: the order in which a refill shifts them into the state.  The lanes of a wave
+// sit at scattered places of their pieces, so byte-wide reads (two per step) collide in the
+// banks about as often as random addresses would, and were the largest share of the LDS time;
+// a quarter as many reads leave the lookup and the entry read as the main LDS work.  (An
 // unaligned 16- or 32-bit LDS read stalls the pipeline for tens of cycles on this hardware.)
 typedef __attribute__((address_space(3))) uint32_t lds_u32;
-template <int K>
 __device__ __forceinline__ void fused_fetch_window(StepFetch &s, const Cursor &c) {
-  static_assert(K % 2 == 0, "a window is read at even steps");
-  const uint32_t a = c.j & ~3u;  // 2K is a multiple of 4: it goes into the offset field
-  const uint32_t lo = *reinterpret_cast<lds_u32 *>(a + 2 * K), hi = *reinterpret_cast<lds_u32 *>(a + 2 * K + 4);
-  s.bytes = __builtin_amdgcn_alignbit(hi, lo, c.j << 3);  // the shift uses bits 0..4: (j & 3) * 8
-}
-// the window of the step after one that kept `keep` = 2 - (bytes taken)
-__device__ __forceinline__ void fused_next_window(StepFetch &s, const StepFetch &before, uint32_t keep) {
-  s.bytes = __builtin_amdgcn_alignbyte(0u, before.bytes, 2u - keep);
+  const uint32_t a = (c.jb >> 3) & ~3u;
+  const uint32_t lo = *reinterpret_cast<lds_u32 *>(a), hi = *reinterpret_cast<lds_u32 *>(a + 4);
+  // the shift uses bits 0..4 of the cursor: (ip & 3) * 8
+  s.win = __builtin_bswap32(__builtin_amdgcn_alignbit(hi, lo, c.jb));
 }
 // Keeps the window in the block that made it: left alone, the compiler sinks the funnel shift
 // past the scan branch.
 __device__ __forceinline__ void fused_pin_bytes(StepFetch &s) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("" : "+v"(s.bytes));
+  asm volatile("" : "+v"(s.win));
 #endif
 }
 __device__ __forceinline__ void fused_fetch_entry(StepFetch &s, uint32_t idx, uint32_t block) {
@@ -208,28 +202,25 @@ __device__ __forceinline__ void fused_scan(uint32_t state, StepFetch &s, uint32_
 
 // state' = freq * (state >> 16) + rel, then the refill: n = 0, 1 or 2 bytes are shifted in
 // while the state is below 2^23.  Without branches or condition registers: the state is
-// below 2^31 and at least 2^7, so c = (24 - clz(state')) >> 3 = 2 - n; the byte selector of
-// v_perm that shifts n bytes of the window in (first stream byte highest) is a window, c
-// bytes up, on the constant 01 00 04 05 06 07.  Returns c.
-__device__ __forceinline__ uint32_t fused_advance(Cursor &c, const StepFetch &s, uint32_t rel) {
+// below 2^31 and at least 2^7, so 8 n = (clz(state') - 1) & 24, and one 64-bit shift of
+// state' : window by that count moves the bytes into the state and out of the window.
+__device__ __forceinline__ void fused_advance(Cursor &c, StepFetch &s, uint32_t rel) {
   uint32_t x;
 #if defined(__HIP_DEVICE_COMPILE__)
   asm("v_mad_u32_u16 %0, %1, %2, %3 op_sel:[1,1,0,0]" : "=v"(x) : "v"(s.e0.x), "v"(c.state), "v"(rel));
 #else
   x = (s.e0.x >> 16) * (c.state >> 16) + rel;
 #endif
-  const uint32_t keep = (24u - (uint32_t)__builtin_clz(x)) >> 3;
-  const uint32_t sel = __builtin_amdgcn_alignbyte(0x00000706u, 0x05040001u, keep);
-  c.state = __builtin_amdgcn_perm(x, s.bytes, sel);
-  c.j -= keep;
-  return keep;
+  const uint32_t bits = ((uint32_t)__builtin_clz(x) - 1u) & 24u;
+  const uint64_t both = (((uint64_t)x << 32) | s.win) << bits;
+  c.state = (uint32_t)(both >> 32);
+  s.win = (uint32_t)both;
+  c.jb += bits;
 }
 
-// Two steps (numbers K and K + 1 of their group of 16, K even) of one segment, given the LDS
-// offsets of their contexts' table blocks.  Returns the images of the two symbols' bits in the
-// BF16 word (symbol << 5).
-__device__ __forceinline__ uint32_t fused_finish_step(Cursor &c, StepFetch &s, uint32_t idx, uint32_t block,
-                                                      uint32_t &keep) {
+// Two consecutive steps of one segment, given the LDS offsets of their contexts' table blocks.
+// Returns the images of the two symbols' bits in the BF16 word (symbol << 5).
+__device__ __forceinline__ uint32_t fused_finish_step(Cursor &c, StepFetch &s, uint32_t idx, uint32_t block) {
   fused_fetch_entry(s, idx, block);
   fused_pin_bytes(s);
   uint64_t miss;
@@ -238,26 +229,26 @@ __device__ __forceinline__ uint32_t fused_finish_step(Cursor &c, StepFetch &s, u
   if (__builtin_expect(miss != 0, 0)) {
     if (fused_lane_in(miss)) fused_scan(c.state, s, rel);
   }
-  keep = fused_advance(c, s, rel);
+  fused_advance(c, s, rel);
   return s.e0.y;
 }
-template <int K>
 __device__ __forceinline__ void fused_symbol_pair_in(Cursor &c, uint32_t block0, uint32_t block1, const FusedParams &q,
                                                      uint32_t &hi0, uint32_t &hi1) {
-  StepFetch s0, s1;
-  uint32_t keep;
+  StepFetch s;
   const uint32_t idx0 = fused_fetch_index(c.state, block0, q);
-  fused_fetch_window<K>(s0, c);
-  hi0 = fused_finish_step(c, s0, idx0, block0, keep);
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_sched_barrier(0);  // the lookup byte first: the LDS answers in issue order and the step waits for it
+#endif
+  fused_fetch_window(s, c);
+  hi0 = fused_finish_step(c, s, idx0, block0);
   const uint32_t idx1 = fused_fetch_index(c.state, block1, q);
-  fused_next_window(s1, s0, keep);
-  hi1 = fused_finish_step(c, s1, idx1, block1, keep);
+  hi1 = fused_finish_step(c, s, idx1, block1);
 }
 template <int K>
 __device__ __forceinline__ void fused_symbol_pair(Cursor &c, uint32_t ccw, const FusedParams &q, uint32_t &hi0,
                                                   uint32_t &hi1) {
-  fused_symbol_pair_in<K>(c, fused_block_offset<K % 4>(ccw, q.block_pitch), fused_block_offset<K % 4 + 1>(ccw, q.block_pitch),
-                          q, hi0, hi1);
+  fused_symbol_pair_in(c, fused_block_offset<K % 4>(ccw, q.block_pitch), fused_block_offset<K % 4 + 1>(ccw, q.block_pitch),
+                       q, hi0, hi1);
 }
 
 // Sixteen packed 6-bit residuals (12 bytes, MSB first) -> field k, k compile-time, sign
@@ -286,26 +277,40 @@ struct Raw6x16 {
 // ---- pieces of the tile walk shared by the GEMV and GEMM kernels ----
 
 // this row class's lookup tables -> LDS, one block per column class: table, then lookup bytes.
-// The copy is two flat loops over 16-byte and 8-byte units, unrolled so that a thread has
-// several loads in flight: copied one context after the other, load by load, the tables cost
-// a workgroup eight round trips to memory before its first step.
+// A thread issues all of its loads of a pass (four 16-byte units of the lookups, four 8-byte
+// entries) before it stores any of them: a loop whose trip count the compiler does not know
+// runs its loads one round trip after the other, which cost a workgroup seven of them (about
+// 5 us) before its first step.  Loads past the end read the last unit again; only the store
+// is conditional.
 __device__ __forceinline__ void fused_load_tables(uint8_t *lds, uint32_t blocks, uint32_t block_pitch,
                                                   const grf_bctx_fused &f, uint32_t cls, uint32_t tid,
                                                   uint32_t nthreads) {
   const uint32_t nb16 = (1u << f.lognb) / 16, entries = f.tabn + 1, tb = fused_table_bytes(f);
   const uint4 *lut = reinterpret_cast<const uint4 *>(f.lut + (size_t)cls * f.nc * (nb16 * 16));
-  const uint32_t n16 = f.nc * nb16;
-#pragma unroll 4
-  for (uint32_t i = tid; i < n16; i += nthreads) {
-    const uint32_t c = i / nb16, w = i % nb16;
-    *reinterpret_cast<uint4 *>(lds + blocks + c * block_pitch + tb + w * 16) = lut[i];
-  }
   const uint2 *tab = reinterpret_cast<const uint2 *>(f.tab) + (size_t)cls * f.nc * entries;
-  const uint32_t n8 = f.nc * entries;
-#pragma unroll 2
-  for (uint32_t i = tid; i < n8; i += nthreads) {
-    const uint32_t c = i / entries, w = i % entries;
-    *reinterpret_cast<uint2 *>(lds + blocks + c * block_pitch + w * 8) = tab[i];
+  const uint32_t n16 = f.nc * nb16, n8 = f.nc * entries;
+  constexpr int kInFlight = 4;
+  for (uint32_t base = 0; base < max(n16, n8); base += kInFlight * nthreads) {  // uniform
+    uint4 a[kInFlight];
+    uint2 e[kInFlight];
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) {
+      const uint32_t i = base + k * nthreads + tid;
+      a[k] = lut[min(i, n16 - 1)];
+      e[k] = tab[min(i, n8 - 1)];
+    }
+#if defined(__HIP_DEVICE_COMPILE__)
+    // (keeps the loads above the stores: the compiler would sink each into its store's branch)
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k)
+      asm volatile("" : "+v"(a[k].x), "+v"(a[k].y), "+v"(a[k].z), "+v"(a[k].w), "+v"(e[k].x), "+v"(e[k].y));
+#endif
+#pragma unroll
+    for (int k = 0; k < kInFlight; ++k) {
+      const uint32_t i = base + k * nthreads + tid;
+      if (i < n16) *reinterpret_cast<uint4 *>(lds + blocks + (i / nb16) * block_pitch + tb + (i % nb16) * 16) = a[k];
+      if (i < n8) *reinterpret_cast<uint2 *>(lds + blocks + (i / entries) * block_pitch + (i % entries) * 8) = e[k];
+    }
   }
 }
 
@@ -380,7 +385,7 @@ struct SegmentWalkT {
   static constexpr bool kAhead = AHEAD;
   Cursor c;
   uint32_t gofs, eofs;        // byte offsets of this segment's and the next segment's checkpoints
-  uint32_t end_state, end_j;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
+  uint32_t end_state, end_jb;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
   const uint32_t *rawp;
   const uint4 *ccp;
   uint32_t n0, n1, n2;             // !AHEAD: the next group's residual words
@@ -413,8 +418,8 @@ struct SegmentWalkT {
   }
   // the row piece was staged at piece_off from global offset a0
   __device__ __forceinline__ void start(uint32_t piece_off, uint32_t a0) {
-    c.j = piece_off + (gofs - a0);
-    end_j = c.j + (eofs - gofs);
+    c.jb = (piece_off + (gofs - a0)) << 3;
+    end_jb = c.jb + ((eofs - gofs) << 3);
   }
 
   // Start the group of symbols [t, t+16): unpack its residuals and column classes, and load
@@ -453,7 +458,6 @@ struct SegmentWalkT {
   }
     GRF_STEP2(0) GRF_STEP2(2) GRF_STEP2(4) GRF_STEP2(6)
 #undef GRF_STEP2
-    if (H == 1) c.end_group();
 #pragma unroll
     for (int k = 0; k < 4; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
   }
@@ -467,7 +471,7 @@ struct SegmentWalkT {
   // the segment must end exactly on the next checkpoint
   __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
     (void)f;
-    return c.state == end_state && c.j == end_j;
+    return c.state == end_state && c.jb == end_jb;
   }
 };
 using SegmentWalk = SegmentWalkT<false>;

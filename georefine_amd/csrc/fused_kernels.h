@@ -323,30 +323,37 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[m] = 0.f;
     if (walks) {
-      uint4 xn[M][2];  // the activations of the next group of 16 columns
-#pragma unroll
-      for (int m = 0; m < M; ++m) {
-        const uint4 *xm = reinterpret_cast<const uint4 *>(x + (size_t)m * ldx + col0);
-        xn[m][0] = xm[0];
-        xn[m][1] = xm[1];
-      }
-      for (uint32_t t = 0; t < S; t += 16) {
-        uint32_t xv[M][8];
+      // The activations of a group of 16 columns are loaded while the group before is
+      // decoded, into one of two register sets that take turns (no copies between them).
+      uint4 xa[M][2], xb[M][2];
+      auto load_x = [&](uint4 (&xs)[M][2], uint32_t t) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-          xv[m][0] = xn[m][0].x, xv[m][1] = xn[m][0].y, xv[m][2] = xn[m][0].z, xv[m][3] = xn[m][0].w;
-          xv[m][4] = xn[m][1].x, xv[m][5] = xn[m][1].y, xv[m][6] = xn[m][1].z, xv[m][7] = xn[m][1].w;
-          // the last group loads itself again rather than branch around the loads
-          const uint4 *xm = reinterpret_cast<const uint4 *>(x + (size_t)m * ldx + col0 + min(t + 16, S - 16));
-          xn[m][0] = xm[0];
-          xn[m][1] = xm[1];
+          const uint4 *xm = reinterpret_cast<const uint4 *>(x + (size_t)m * ldx + col0 + t);
+          xs[m][0] = xm[0];
+          xs[m][1] = xm[1];
         }
+      };
+      auto group = [&](uint32_t t, const uint4 (&xs)[M][2], uint4 (&xnext)[M][2]) {
+        load_x(xnext, min(t + 16, S - 16));  // the last group loads itself again rather than branch around the loads
         uint32_t pair[8];
         w.decode16(t, S, q, pair);
 #pragma unroll
-        for (int m = 0; m < M; ++m)
-#pragma unroll
-          for (int k = 0; k < 8; ++k) acc[m] = dot2_bf16(pair[k], xv[m][k], acc[m]);
+        for (int m = 0; m < M; ++m) {
+          acc[m] = dot2_bf16(pair[0], xs[m][0].x, acc[m]);
+          acc[m] = dot2_bf16(pair[1], xs[m][0].y, acc[m]);
+          acc[m] = dot2_bf16(pair[2], xs[m][0].z, acc[m]);
+          acc[m] = dot2_bf16(pair[3], xs[m][0].w, acc[m]);
+          acc[m] = dot2_bf16(pair[4], xs[m][1].x, acc[m]);
+          acc[m] = dot2_bf16(pair[5], xs[m][1].y, acc[m]);
+          acc[m] = dot2_bf16(pair[6], xs[m][1].z, acc[m]);
+          acc[m] = dot2_bf16(pair[7], xs[m][1].w, acc[m]);
+        }
+      };
+      load_x(xa, 0);
+      for (uint32_t t = 0; t < S; t += 32) {
+        group(t, xa, xb);
+        if (t + 16 < S) group(t + 16, xb, xa);
       }
       if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
     }

@@ -103,7 +103,7 @@ struct Raw5x16 {
 struct PpcxWalk {
   grf::Cursor c;
   uint32_t gofs, eofs;        // byte offsets of this segment's and the next segment's checkpoints
-  uint32_t end_state, end_j;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
+  uint32_t end_state, end_jb;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
   const uint8_t *rawp;    // the segment's first residual byte (5 * S / 8 bytes per segment)
   const uint2 *binp;      // the segment's bins, 8 bytes per 16 symbols
   uint32_t n0, n1, n2;
@@ -129,8 +129,8 @@ struct PpcxWalk {
     nb = binp[0];
   }
   __device__ __forceinline__ void start(uint32_t piece_off, uint32_t a0) {
-    c.j = piece_off + (gofs - a0);
-    end_j = c.j + (eofs - gofs);
+    c.jb = (piece_off + (gofs - a0)) << 3;
+    end_jb = c.jb + ((eofs - gofs) << 3);
   }
 
   __device__ __forceinline__ void begin16(uint32_t t, uint32_t S) {
@@ -153,13 +153,12 @@ struct PpcxWalk {
     const uint32_t bin0 = __builtin_amdgcn_ubfe(bw[H], 4 * (i), 4);                                   \
     const uint32_t bin1 = __builtin_amdgcn_ubfe(bw[H], 4 * (i) + 4, 4);                               \
     uint32_t h0, h1;                                                                                  \
-    grf::fused_symbol_pair_in<8 * H + (i)>(c, __umul24(bin0, q.block_pitch), __umul24(bin1, q.block_pitch), q, h0, h1); \
+    grf::fused_symbol_pair_in(c, __umul24(bin0, q.block_pitch), __umul24(bin1, q.block_pitch), q, h0, h1); \
     bits[i] = h0 | rr.field<8 * H + (i)>();                                                           \
     bits[(i) + 1] = h1 | rr.field<8 * H + (i) + 1>();                                                 \
   }
     GRF_STEP2(0) GRF_STEP2(2) GRF_STEP2(4) GRF_STEP2(6)
 #undef GRF_STEP2
-    if (H == 1) c.end_group();
 #pragma unroll
     for (int k = 0; k < 4; ++k) pair[k] = __builtin_amdgcn_perm(bits[2 * k + 1], bits[2 * k], 0x05040100u);
   }
@@ -171,7 +170,7 @@ struct PpcxWalk {
 
   __device__ __forceinline__ bool ended_on_checkpoint(const grf_bctx_fused &f) const {
     (void)f;
-    return c.state == end_state && c.j == end_j;
+    return c.state == end_state && c.jb == end_jb;
   }
 };
 
