@@ -12,6 +12,10 @@ Reference lines restated here (GCR = context-runtime/georefine_context_runtime):
 * ``ppcx_fit``               GCR/bitexact_predictive_codec.py:99-143
 * ``ppcx_encode/decode``     GCR/bitexact_predictive_codec.py:175-251
 * ``mix_predict``            GCR/bitexact_predictive_mix.py:60-78
+
+The container functions above are pinned by whole frames that the reference's own Python
+codecs wrote (tests/golden/frames.npz, every frame mode of both codecs, labels on ties);
+the coders below them by the reference's compiled C++ core.  No function here is unpinned.
 """
 from __future__ import annotations
 
