@@ -121,13 +121,15 @@ def reference_core():
     sz, u32, u64 = ctypes.c_size_t, ctypes.c_uint32, ctypes.c_uint64
     L.bcx_decode.argtypes = [U8P, sz, u64, u32, u32, U8P, U8P, u32, u32, u32, U16P, U32P, U16P]
     L.bcx_unpack6.argtypes = [U8P, sz, u64, U16P]
-    L.bcx_decode.restype = L.bcx_unpack6.restype = ctypes.c_int
+    L.bcx_decode_compact.argtypes = L.bcx_decode.argtypes
+    L.bcx_decode.restype = L.bcx_decode_compact.restype = L.bcx_unpack6.restype = ctypes.c_int
     return L
 
 
-def reference_decode(L, orc, frame):
-    """A frame decoded by the reference's bcx_decode / bcx_unpack6 (full 65536-slot lookup);
-    the container around them (header, inflate, digests) is read by the oracle's parser."""
+def reference_decode(L, orc, frame, compact=False):
+    """A frame decoded by the reference's bcx_decode (full 65536-slot lookup per context) or
+    bcx_decode_compact (binary search in the cumulative table), and bcx_unpack6; the container
+    around them (header, inflate, digests) is read by the oracle's parser."""
     import ctypes
     import hashlib
     s = orc.bctx_sections(frame)
@@ -142,8 +144,9 @@ def reference_decode(L, orc, frame):
         data = np.frombuffer(stream, dtype=np.uint8)
         out = np.empty(n, dtype=np.uint16)
         freq = np.ascontiguousarray(freq, dtype=np.uint32).ravel()
-        rc = L.bcx_decode(p(data, u8), len(stream), n, rows, cols, p(s["rc"], u8), p(s["cc"], u8), s["nr"], s["nc"],
-                          kind, p(main, u16) if main is not None else None, p(freq, u32), p(out, u16))
+        fn = L.bcx_decode_compact if compact else L.bcx_decode
+        rc = fn(p(data, u8), len(stream), n, rows, cols, p(s["rc"], u8), p(s["cc"], u8), s["nr"], s["nc"],
+                kind, p(main, u16) if main is not None else None, p(freq, u32), p(out, u16))
         if rc:
             raise RuntimeError(f"reference bcx_decode failed ({rc})")
         return out
@@ -162,7 +165,7 @@ def reference_decode(L, orc, frame):
     return out
 
 
-def cpu_baseline(frames, words_of, x_words, min_seconds=10.0, max_frames=12):
+def cpu_baseline(frames, words_of, x_words, min_seconds=8.0, max_frames=12):
     """CPU decode + fp32 matvec of whole frames of the workload, one thread, as the reference
     decodes a frame; frames are taken in turn until min_seconds of work are done.  Timed with
     the reference's own compiled coder where oracle/_ref holds it (kind "reference"), and
@@ -170,11 +173,11 @@ def cpu_baseline(frames, words_of, x_words, min_seconds=10.0, max_frames=12):
     from oracle import codec_oracle as orc
     names = list(frames)
 
-    def timed(decode, what):
+    def timed(decode, what, seconds=min_seconds):
         coded = produced = done = 0
         checksum = 0.0
         t0 = time.perf_counter()
-        while done < max_frames and (done == 0 or time.perf_counter() - t0 < min_seconds):
+        while done < max_frames and (done == 0 or time.perf_counter() - t0 < seconds):
             name = names[done % len(names)]
             dec = decode(frames[name])
             wf = (dec.astype(np.uint32) << 16).view(np.float32)
@@ -192,13 +195,16 @@ def cpu_baseline(frames, words_of, x_words, min_seconds=10.0, max_frames=12):
                            f"({produced / dt / 1e6:.1f} MB/s of BF16 produced)",
                     checksum=checksum)
 
-    port = dict(timed(orc.bctx_decode, "the oracle's full-LUT rANS decode of the main stream and 6-bit unpack"), kind="port")
+    port = dict(timed(orc.bctx_decode, "the oracle's full-LUT rANS decode of both streams", min_seconds / 2), kind="port")
     core = reference_core()
     if core is not None:
         result = dict(timed(lambda f: reference_decode(core, orc, f),
-                            "the reference's bcx_decode (full LUT) and bcx_unpack6, compiled from its sources"),
+                            "the reference's bcx_decode (full LUT) of both streams, compiled from its sources"),
                       kind="reference")
         result["oracle_port"] = port
+        result["compact_lookup"] = dict(timed(lambda f: reference_decode(core, orc, f, compact=True),
+                                              "the reference's bcx_decode_compact (search in the cumulative table) of both "
+                                              "streams, compiled from its sources", min_seconds / 2), kind="reference")
     else:
         result = port
     # the reference decodes one frame per thread: every host core with a frame of its own, once
@@ -313,7 +319,7 @@ def run_predictive(args):
     }), flush=True)
 
 
-def run_stack(args):
+def run_stack(args, as_dict=False):
     """Every coded linear of a 64-layer stack resident at once, one pass at batch 64.
 
     Each layer holds q, k, v, o, gate, up and down as BCTX frames.  `--distinct-layers`
@@ -435,15 +441,16 @@ def run_stack(args):
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
     dom = max(LAYER, key=lambda n_: ms[n_])
     achieved = alg[dom]["total"] / (ms[dom] * 1e-3) / 1e9
-    kernel = ("grf::fused_gemm_kernel<grf::SegmentWalkT<false>, MT>" if m > GEMV_UP_TO
-              else f"grf::fused_walk_kernel<grf::SegmentWalkT<true>, {m}, 0>")  # the stack's segments have 64 symbols
-    print(json.dumps({
+    kernel = kernel_name(False, m, False, 64)  # (of the ungrouped launch that took longest)
+    result = {
         "metric": "compressed-weight decode-GEMV GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": f"whole stack resident: {args.layers} layers x (q 5120->6144, k/v 5120->1024, o 6144->5120, "
-                               f"gate/up 5120->17408, down 17408->5120), one pass through every coded linear at batch {m}",
+                               f"gate/up 5120->17408, down 17408->5120), one pass through every coded linear at batch {m}; "
+                               f"{dense / 1e9:.1f} GB of dense BF16 held as {frame_bytes / 1e9:.1f} GB of frames "
+                               f"(no embedding or head matrix in the stack)",
                    "batch": m, "layers": args.layers, "distinct_layers": args.distinct_layers,
                    "linears": args.layers * len(LAYER), "launch": launch,
                    "launches": "q/k/v and gate/up grouped" if grouped else "one per linear"},
@@ -456,7 +463,16 @@ def run_stack(args):
                             "GBps": round(alg[n_]["total"] / (ms[n_] * 1e-3) / 1e9, 2)} for n_ in LAYER},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": f"{kernel} on {dom}"},
-    }), flush=True)
+    }
+    if as_dict:  # as a key of the headline line: the fields that line carries itself are left out
+        for key in ("metric", "unit", "n_gpus", "higher_is_better", "scaling", "vs_baseline", "dtype", "data"):
+            result.pop(key)
+        layers.clear()
+        base.clear()
+        groups = graph = None
+        torch.cuda.empty_cache()
+        return result
+    print(json.dumps(result), flush=True)
 
 
 def main():
@@ -484,6 +500,10 @@ def main():
     ap.add_argument("--no-groups", action="store_true",
                     help="one launch per linear instead of one for the matrices that take the same activations "
                          "(gate/up; in the stack also q/k/v)")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="mlp at batch 1: leave out the batch-64 step and the whole-stack pass that the default run "
+                         "adds to the line as `batch64` and `stack`")
+    ap.add_argument("--no-stack", action="store_true", help="mlp at batch 1: leave out the whole-stack pass only")
     ap.add_argument("--distinct-layers", type=int, default=1,
                     help="stack: layers encoded from their own seeds; the rest are device copies of these")
     args = ap.parse_args()
@@ -527,162 +547,245 @@ def main():
             sys.exit(f"bench.py: {name} is not eligible for the fused kernel: {tensors[name].fused_reason}")
         log(f"{name}: {rows}x{cols} mode {tensors[name].mode} frame {len(frame)} B "
             f"({8 * len(frame) / w.size:.3f} bit/weight) encode {t1 - t0:.1f}s index+upload {t2 - t1:.1f}s "
-            f"plan {tensors[name].fused_plan} tiling {(tensors[name]._tiling(args.batch) if args.batch <= GEMV_UP_TO else tensors[name]._gemm_tiling())[3]}")
+            f"resident mode {tensors[name].resident_mode} plan {tensors[name].fused_plan} "
+            f"tiling {(tensors[name]._tiling(args.batch) if args.batch <= GEMV_UP_TO else tensors[name]._gemm_tiling())[3]}")
         frames[name] = frame
         words_of[name] = w
     log(f"setup {time.perf_counter() - t_setup:.1f}s")
 
-    m = args.batch
-    rng = np.random.default_rng(7)
-    x_words = {k: bf16_words(rng.normal(0, 1, size=(max(m, 1), k))) for k in (5120, 17408)}
-    x = {k: torch.from_numpy(v).view(torch.bfloat16).cuda() for k, v in x_words.items()}
-
     # the launches of a step: gate and up take the same activations and share one launch
     from georefine_amd.bitexact_context_gpu import HipLinearGroup
-    units = []  # (label, member names, callable)
+    pair = None
     if not args.no_groups and "gate" in names and "up" in names:
         pair = HipLinearGroup([tensors["gate"], tensors["up"]])
-        units.append(("gate+up", ["gate", "up"], lambda: pair.linear(x[5120])))
-        log(f"gate+up: one launch, tiling {pair._tiling(m if m <= GEMV_UP_TO else 'gemm')[0][3]}")
-    for name in names:
-        if decode_only:
-            units.append((name, [name], lambda name=name: tensors[name].decode(check=False)))
-        elif not any(name in u[1] for u in units):
-            units.append((name, [name], lambda name=name: tensors[name].linear(x[SHAPES[name][1]])))
 
+    def measure(m):
+        """One workload at m activation rows (0: decode to dense): (result fields, x words)."""
+        rng = np.random.default_rng(7)
+        x_words = {k: bf16_words(rng.normal(0, 1, size=(max(m, 1), k))) for k in (5120, 17408)}
+        x = {k: torch.from_numpy(v).view(torch.bfloat16).cuda() for k, v in x_words.items()}
+        units = []  # (label, member names, callable)
+        if pair is not None and not decode_only:
+            units.append(("gate+up", ["gate", "up"], lambda: pair.linear(x[5120])))
+            log(f"batch {m} gate+up: one launch, tiling {pair._tiling('waves' if m <= GEMV_UP_TO else 'gemm')[0][3]}")
+        for name in names:
+            if decode_only:
+                units.append((name, [name], lambda name=name: tensors[name].decode(check=False)))
+            elif not any(name in u[1] for u in units):
+                units.append((name, [name], lambda name=name: tensors[name].linear(x[SHAPES[name][1]])))
+        ms_per_step, per_kernel_ms, launch, timing = time_launches(
+            torch, units, args.steps, args.warmup, args.graph,
+            lambda: [n_ for n_ in names if tensors[n_].error.item()] + ([] if pair is None or not pair.error.item() else ["gate+up"]))
+        if args.calibrate_copy:
+            src = torch.ones(32 * 1024 * 1024, dtype=torch.int32, device="cuda")
+            dst = torch.empty_like(src)
+            for _ in range(3):
+                torch.add(src, 1, out=dst)
+            torch.cuda.synchronize()
+        alg = {}
+        for label, members, _ in units:
+            parts = [algorithmic_bytes(tensors[n_], m) for n_ in members]
+            alg[label] = {k: sum(p_[k] for p_ in parts) for k in parts[0]}
+            if len(members) > 1:  # the members read one x
+                alg[label]["total"] -= (len(members) - 1) * m * SHAPES[members[0]][1] * 2
+            if decode_only:  # the dense matrix is written once
+                alg[label]["total"] += sum(2 * SHAPES[n_][0] * SHAPES[n_][1] for n_ in members)
+        step_bytes = sum(a_["total"] for a_ in alg.values())
+        dense_bytes = sum(2 * SHAPES[n_][0] * SHAPES[n_][1] for n_ in names)
+        value = step_bytes / (ms_per_step * 1e-3) / 1e9
+        eff_bf16 = dense_bytes / (ms_per_step * 1e-3) / 1e9
+        dom = max(per_kernel_ms, key=lambda n_: per_kernel_ms[n_])
+        kernel = kernel_name(decode_only, m, "+" in dom, tensors[names[0]].fused_plan["seg_len"])
+        traffic, traffic_source = recorded_traffic(decode_only, m, kernel)
+        achieved = alg[dom]["total"] / (per_kernel_ms[dom] * 1e-3) / 1e9
+        fields = {
+            "value": round(value, 2), "ms_per_step": round(ms_per_step, 4),
+            "config": {"workload": ("fused decode to dense BF16 (decode())" if decode_only else
+                                    "fused decode-" + ("GEMV" if m <= GEMV_UP_TO else "GEMM") + ", batch %d" % m)
+                                   + ", Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, BCTX (16,4) frames"
+                                   + (", residuals resident in packed 6-bit form"
+                                      if any(tensors[n_].resident_mode != tensors[n_].mode for n_ in names) else ""),
+                       "batch": m, "matrices": names, "launches": [u[0] for u in units],
+                       "segment": tensors[names[0]].fused_plan["seg_len"], "launch": launch, "per_kernel_timing": timing},
+            "effective_bf16_GBps": round(eff_bf16, 2),
+            "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3) if m else None,
+            "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
+            "per_kernel": {n_: {"ms": round(per_kernel_ms[n_], 4), "alg_bytes": alg[n_]["total"],
+                                "payload_bytes": alg[n_]["payload"], "index_bytes": alg[n_]["index"],
+                                "table_bytes": alg[n_]["tables"],
+                                "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2),
+                                "frac_of_hbm_peak": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+                           for n_ in per_kernel_ms},
+            "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                         "kernel": f"{kernel} on {dom}"},
+        }
+        if m > GEMV_UP_TO:
+            # the matrix cores' share: useful flops of the dominant launch against the dense BF16 peak
+            flops = sum(2.0 * m * SHAPES[n_][0] * SHAPES[n_][1] for n_ in dom.split("+"))
+            fields["mfma"] = {"achieved": round(flops / (per_kernel_ms[dom] * 1e-3) / 1e12, 2), "peak": 2500.0,
+                              "unit": "TFLOP/s", "frac": round(flops / (per_kernel_ms[dom] * 1e-3) / 2.5e15, 4)}
+        return fields, x_words
+
+    fields, x_words = measure(args.batch)
+    result = {
+        "metric": "compressed-weight decode GB/s (coded bytes read + dense BF16 written)" if decode_only
+                  else "compressed-weight decode-GEMV GB/s",
+        "value": fields.pop("value"), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": fields.pop("ms_per_step"), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u32 rANS state / bf16 weights / fp32 accumulate", "data": "synthetic",
+    }
+    result.update(fields)
+    copy_rate = measured_copy_gbps(torch)
+    result["hbm_copy_measured_GBps"] = round(copy_rate, 1)
+    result["pct_of_measured_copy"] = round(100 * result["value"] / copy_rate, 2)
+    headline = args.workload == "mlp" and args.batch == 1 and not args.only and not args.no_extras
+    if headline:
+        # the other two figures of the metric, timed in the same run: the MLP step at batch 64
+        # (fused GEMM on the matrix cores) and one pass through a whole resident stack
+        log("batch 64 ...")
+        b64, _ = measure(64)
+        b64.pop("config")
+        result["batch64"] = b64
+    if not args.no_cpu_baseline:
+        log("timing the CPU oracle on whole frames ...")
+        result["cpu_baseline"] = cpu_baseline(frames, words_of, x_words)
+        result["cpu_baseline"]["host"] = host_description()
+    if headline and not args.no_stack:
+        del tensors, pair
+        torch.cuda.empty_cache()
+        log("whole stack ...")
+        stack_args = argparse.Namespace(**vars(args))
+        stack_args.batch, stack_args.steps, stack_args.warmup = 64, max(3, args.steps // 10), max(2, args.warmup // 10)
+        result["stack"] = run_stack(stack_args, as_dict=True)
+    print(json.dumps(result), flush=True)
+
+
+def kernel_name(decode_only, m, grouped, seg_len):
+    """The kernel a launch of the workload runs (as rocprofv3 names it)."""
+    ahead = "true" if seg_len == 64 else "false"  # 64-symbol segments: the walker that reads a segment's residuals once
+    if decode_only:
+        return f"grf::fused_walk_kernel<grf::SegmentWalkT<{ahead}>, 1, 1>"
+    if m <= GEMV_UP_TO:
+        rows = min(m, 2)  # the wave-unit GEMV carries at most two rows per launch
+        return (f"grf::fused_wave_group_kernel<grf::SegmentWalkT<false>, {rows}>" if grouped
+                else f"grf::fused_wave_kernel<grf::SegmentWalkT<false>, {rows}>")
+    return ("grf::fused_gemm_group_kernel<grf::SegmentWalkT<false>, MT>" if grouped
+            else "grf::fused_gemm_kernel<grf::SegmentWalkT<false>, MT>")
+
+
+def kernel_sources_sha256():
+    """Digest of the device sources: a recorded counter figure is only quoted for these."""
+    import hashlib
+    h = hashlib.sha256()
+    for path in sorted((ROOT / "georefine_amd" / "csrc").glob("*")):
+        if path.suffix in (".h", ".hip"):
+            h.update(path.name.encode() + b"\0" + path.read_bytes())
+    return h.hexdigest()
+
+
+def recorded_traffic(decode_only, m, kernel):
+    """HBM bytes per launch of `kernel` from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE
+    record (bench.py cannot read hardware counters itself), and where the figure comes from.
+    The record names the kernels it measured and the digest of the device sources it was taken
+    with; for another kernel or other sources the figure is withheld (None) and the reason given."""
+    name = ("fused_store_decode_qwen27b_mlp_traffic.json" if decode_only else
+            "fused_gemv_m1_qwen27b_mlp_traffic.json" if m == 1 else
+            "fused_gemm_m64_qwen27b_mlp_traffic.json" if m == 64 else None)
+    if name is None or not (ROOT / "profiles" / name).exists():
+        return None, "no counter record for this workload"
+    record = json.loads((ROOT / "profiles" / name).read_text())
+    per_kernel = record.get("traffic_bytes_per_launch")
+    short = kernel.split("<")[0].split("::")[-1]
+    if not isinstance(per_kernel, dict) or short not in per_kernel:
+        return None, f"profiles/{name} holds no figure for {short}"
+    if record.get("kernel_sources_sha256") != kernel_sources_sha256():
+        return None, f"profiles/{name} was recorded with other kernel sources (its figure for {short}: {per_kernel[short]:.0f} B)"
+    return per_kernel[short], f"recorded: profiles/{name} (rocprofv3 --pmc, same kernel sources)"
+
+
+def time_launches(torch, units, steps, warmup, graph, errors):
+    """(ms per step, {label: ms per launch}, how the step was launched, how launches were timed).
+
+    After `warmup` eager steps: each launch of the step is captured ten times into a HIP graph
+    of its own and the replays are bracketed by events on the launch stream, which gives the
+    kernel's duration without the host's per-launch latency (eager events around single
+    launches where capture is not possible or --no-graph is given); then `steps` replays of
+    a graph of the whole step are timed on the host clock between synchronisations."""
     def step():
         return [run() for _, _, run in units]
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    for name in names:
-        if tensors[name].error.item():
-            sys.exit(f"bench.py: decoder error word set for {name}")
-
-    # per-launch durations with events on the stream the kernels run on
-    starts = [[torch.cuda.Event(enable_timing=True) for _ in units] for _ in range(args.steps)]
-    ends = [[torch.cuda.Event(enable_timing=True) for _ in units] for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    wall0 = time.perf_counter()
-    for s in range(args.steps):
-        for j, (_, _, run) in enumerate(units):
-            starts[s][j].record()
-            run()
-            ends[s][j].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - wall0
+    bad = errors()
+    if bad:
+        sys.exit(f"bench.py: decoder error word set for {bad}")
+    per_kernel_ms, timing = {}, "HIP events around 10 launches per graph replay"
+    if graph:
+        try:
+            for label, _, run in units:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    for _ in range(10):
+                        run()
+                g.replay()
+                torch.cuda.synchronize()
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                replays = max(2, steps // 10)
+                a.record()
+                for _ in range(replays):
+                    g.replay()
+                b.record()
+                torch.cuda.synchronize()
+                per_kernel_ms[label] = a.elapsed_time(b) / (10 * replays)
+        except Exception as exc:
+            log(f"graph capture failed ({exc}); timing eager launches")
+            per_kernel_ms = {}
+    if not per_kernel_ms:
+        timing = "HIP events around single eager launches"
+        starts = [[torch.cuda.Event(enable_timing=True) for _ in units] for _ in range(steps)]
+        ends = [[torch.cuda.Event(enable_timing=True) for _ in units] for _ in range(steps)]
+        torch.cuda.synchronize()
+        for s_ in range(steps):
+            for j, (_, _, run) in enumerate(units):
+                starts[s_][j].record()
+                run()
+                ends[s_][j].record()
+        torch.cuda.synchronize()
+        per_kernel_ms = {label: float(np.mean([starts[s_][j].elapsed_time(ends[s_][j]) for s_ in range(steps)]))
+                         for j, (label, _, _) in enumerate(units)}
     launch = "eager"
-    if args.graph:
+    wall = None
+    if graph:
         # the same step captured once and replayed: the launches of a step are submitted together,
         # which takes the host's per-launch latency out of the gaps between kernels
         try:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
                 step()
-            graph.replay()
+            g.replay()
             torch.cuda.synchronize()
         except Exception as exc:  # keep the eager figure
             log(f"graph capture failed ({exc}); reporting the eager steps")
         else:
             wall0 = time.perf_counter()
-            for _ in range(args.steps):
-                graph.replay()
+            for _ in range(steps):
+                g.replay()
             torch.cuda.synchronize()
             wall = time.perf_counter() - wall0
             launch = "hip graph replay"
-    for name in names:
-        if tensors[name].error.item():
-            sys.exit(f"bench.py: decoder error word set for {name}")
-
-    if args.calibrate_copy:
-        src = torch.ones(32 * 1024 * 1024, dtype=torch.int32, device="cuda")
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            torch.add(src, 1, out=dst)
+    if wall is None:
         torch.cuda.synchronize()
-
-    per_kernel_ms = {label: float(np.mean([starts[s][j].elapsed_time(ends[s][j]) for s in range(args.steps)]))
-                     for j, (label, _, _) in enumerate(units)}
-    alg = {}
-    for label, members, _ in units:
-        parts = [algorithmic_bytes(tensors[n_], m) for n_ in members]
-        alg[label] = {k: sum(p_[k] for p_ in parts) for k in parts[0]}
-        if len(members) > 1:  # the members read one x
-            alg[label]["total"] -= (len(members) - 1) * m * SHAPES[members[0]][1] * 2
-        if decode_only:  # the dense matrix is written once
-            alg[label]["total"] += sum(2 * SHAPES[n_][0] * SHAPES[n_][1] for n_ in members)
-    step_bytes = sum(a["total"] for a in alg.values())
-    dense_bytes = sum(2 * SHAPES[n][0] * SHAPES[n][1] for n in names)
-    ms_per_step = wall / args.steps * 1e3
-    value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    eff_bf16 = dense_bytes / (ms_per_step * 1e-3) / 1e9
-
-    # HBM bytes per launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE (scaled by a copy
-    # kernel of known size); a recorded figure, bench.py cannot read hardware counters itself
-    dom = max(per_kernel_ms, key=lambda n_: per_kernel_ms[n_])
-    grouped = "+" in dom
-    # 64-symbol segments: the walker that reads a segment's residuals once
-    ahead = "true" if tensors[names[0]].fused_plan["seg_len"] == 64 else "false"
-    if decode_only:
-        kernel = f"grf::fused_walk_kernel<grf::SegmentWalkT<{ahead}>, 1, 1>"
-    elif m <= GEMV_UP_TO:
-        kernel = (f"grf::fused_walk_group_kernel<grf::SegmentWalkT<{ahead}>, {m}>" if grouped
-                  else f"grf::fused_walk_kernel<grf::SegmentWalkT<{ahead}>, {m}, 0>")
-    else:
-        kernel = ("grf::fused_gemm_group_kernel<grf::SegmentWalkT<false>, MT>" if grouped
-                  else "grf::fused_gemm_kernel<grf::SegmentWalkT<false>, MT>")
-    traffic = None
-    recorded = ROOT / "profiles" / ("fused_store_decode_qwen27b_mlp_traffic.json" if decode_only
-                                    else "fused_gemv_m1_qwen27b_mlp_traffic.json")
-    if (m == 1 or decode_only) and recorded.exists():
-        per_kernel_traffic = json.loads(recorded.read_text()).get("traffic_bytes_per_launch")
-        if isinstance(per_kernel_traffic, dict):  # by kernel name
-            traffic = per_kernel_traffic.get(kernel.split("<")[0].split("::")[-1])
-    achieved = alg[dom]["total"] / (per_kernel_ms[dom] * 1e-3) / 1e9
-    result = {
-        "metric": "compressed-weight decode GB/s (coded bytes read + dense BF16 written)" if decode_only
-                  else "compressed-weight decode-GEMV GB/s",
-        "value": round(value, 2),
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
-        "data": "synthetic",
-        "config": {"workload": ("fused decode to dense BF16 (decode())" if decode_only else
-                                "fused decode-" + ("GEMV" if m <= GEMV_UP_TO else "GEMM") + ", batch %d" % m)
-                               + ", Qwen-27B-like MLP: gate/up 5120->17408, down 17408->5120, "
-                               "BCTX (16,4) frames, residuals resident in packed 6-bit form",
-                   "batch": m, "matrices": names, "launches": [u[0] for u in units],
-                   "segment": tensors[names[0]].fused_plan["seg_len"], "launch": launch},
-        "effective_bf16_GBps": round(eff_bf16, 2),
-        "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3) if m else None,
-        "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
-        "per_kernel": {n_: {"ms": round(per_kernel_ms[n_], 4), "alg_bytes": alg[n_]["total"],
-                            "payload_bytes": alg[n_]["payload"], "index_bytes": alg[n_]["index"],
-                            "table_bytes": alg[n_]["tables"],
-                            "GBps": round(alg[n_]["total"] / (per_kernel_ms[n_] * 1e-3) / 1e9, 2)} for n_ in per_kernel_ms},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "kernel": f"{kernel} on {dom}"},
-    }
-    if m > GEMV_UP_TO:
-        # the matrix cores' share: useful flops of the dominant launch against the dense BF16 peak
-        flops = sum(2.0 * m * SHAPES[n_][0] * SHAPES[n_][1] for n_ in dom.split("+"))
-        result["mfma"] = {"achieved": round(flops / (per_kernel_ms[dom] * 1e-3) / 1e12, 2), "peak": 2500.0,
-                          "unit": "TFLOP/s", "frac": round(flops / (per_kernel_ms[dom] * 1e-3) / 2.5e15, 4)}
-    copy_rate = measured_copy_gbps(torch)
-    result["hbm_copy_measured_GBps"] = round(copy_rate, 1)
-    result["pct_of_measured_copy"] = round(100 * value / copy_rate, 2)
-    if not args.no_cpu_baseline:
-        log("timing the CPU oracle on whole frames ...")
-        result["cpu_baseline"] = cpu_baseline(frames, words_of, x_words)
-        result["cpu_baseline"]["host"] = host_description()
-    print(json.dumps(result), flush=True)
+        wall0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - wall0
+    bad = errors()
+    if bad:
+        sys.exit(f"bench.py: decoder error word set for {bad}")
+    return wall / steps * 1e3, per_kernel_ms, launch, timing
 
 
 if __name__ == "__main__":
