@@ -47,7 +47,7 @@ class GrfPpcxFused(ctypes.Structure):
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
                   "grf_bctx_fused_decode", "grf_bctx_fused_gather", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
-                  "grf_gemm_workspace_bytes", "grf_pack_activations", "grf_bctx_gemv_group", "grf_bctx_gemm_group",
+                  "grf_gemm_workspace_bytes", "grf_bctx_gemm_noalloc", "grf_gemm_noalloc_limit_bytes", "grf_pack_activations", "grf_bctx_gemv_group", "grf_bctx_gemm_group",
                   "grf_ppcx_bins", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_last_error",
                   "grf_abi_version")
 
@@ -70,6 +70,10 @@ def declare(L):
     L.grf_bctx_gemm_lds_bytes.restype = u32
     L.grf_gemm_workspace_bytes.argtypes = [u32, u32]
     L.grf_gemm_workspace_bytes.restype = ctypes.c_size_t
+    L.grf_bctx_gemm_noalloc.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, u32, u32, vp, u32, vp, vp, vp]
+    L.grf_bctx_gemm_noalloc.restype = i
+    L.grf_gemm_noalloc_limit_bytes.argtypes = []
+    L.grf_gemm_noalloc_limit_bytes.restype = ctypes.c_size_t
     L.grf_pack_activations.argtypes = [vp, u32, u32, u32, vp, ctypes.c_size_t, vp]
     L.grf_pack_activations.restype = i
     L.grf_bctx_gemv_group.argtypes = [u32, vp, vp, vp, u32, u32, vp, vp, vp, vp, vp]

@@ -250,6 +250,20 @@ int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
                   size_t workspace_bytes, int32_t *error, void *hip_stream);
 size_t grf_gemm_workspace_bytes(uint32_t cols, uint32_t m_rows);
 
+/* grf_bctx_gemm without the workspace argument, for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid it).  No
+ * counterpart in the reference.  The packed activations go to an 8 MiB array that is part of
+ * the library's device image (every GPU the library runs on holds its copy until the process
+ * ends); the call allocates and frees nothing.  It fails with GRF_UNSUPPORTED when
+ * grf_gemm_workspace_bytes(cols, min(m_rows, 128)) exceeds grf_gemm_noalloc_limit_bytes()
+ * (128 rows: matrices up to 32 752 columns; 64 rows: twice that).  x must not be NULL.  All
+ * calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads)
+ * race; calls on one stream are ordered.  Results are those of grf_bctx_gemm, bit for bit. */
+int grf_bctx_gemm_noalloc(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, const uint16_t *x, uint32_t ldx,
+                          uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
+                          void *hip_stream);
+size_t grf_gemm_noalloc_limit_bytes(void);
+
 /* For several matrices that take the same activations (q/k/v, gate/up): writes 1..128 rows
  * of x into workspace in operand order once; grf_bctx_gemm / grf_ppcx_gemm called with
  * x == NULL, the same m_rows, a frame of this width and that workspace then multiply
