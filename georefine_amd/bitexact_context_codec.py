@@ -42,14 +42,20 @@ def _lib():
 
 
 def _input(words):
-    a = np.asarray(words)
-    if a.ndim != 2 or a.dtype.kind not in "ui" or a.dtype.itemsize != 2:
+    """The matrix as contiguous little-endian uint16 words.  Accepted: two-dimensional arrays of
+    16-bit integers (signed ones only where every value is a valid word's bit pattern read as
+    unsigned, i.e. non-negative), non-empty, at most MAX_WORDS elements
+    (GCR/bitexact_context_codec.py:172-180 accepts and rejects the same inputs)."""
+    matrix = np.asarray(words)
+    sixteen_bit_integers = matrix.dtype.kind in ("u", "i") and matrix.dtype.itemsize == 2
+    if matrix.ndim != 2 or not sixteen_bit_integers:
         raise CodecError("expected a 2D uint16 word array")
-    if not all(a.shape) or a.size > MAX_WORDS:
+    rows, cols = matrix.shape
+    if rows == 0 or cols == 0 or rows * cols > MAX_WORDS:
         raise CodecError("invalid or oversized geometry")
-    if a.dtype.kind == "i" and (np.any(a < 0) or np.any(a > 65535)):
+    if matrix.dtype.kind == "i" and matrix.min() < 0:  # (an int16 cannot exceed 65535)
         raise CodecError("word outside uint16 range")
-    return np.ascontiguousarray(a, dtype="<u2")
+    return np.ascontiguousarray(matrix, dtype="<u2")
 
 
 def _labels(a, nr, nc):

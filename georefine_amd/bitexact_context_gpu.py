@@ -4,8 +4,12 @@
 ``index_frame`` / ``CudaContextTensor`` (GCR/bitexact_context_gpu.py:66-106 and
 :109-168): the loader calls ``factory(frame, stride=..., device=...)`` and uses
 ``shape``, ``source_sha256``, ``frame_sha256``, ``frame_bytes``, ``resident_bytes``,
-``decode(check=)`` and ``gather_rows(ids, check=)``.  The frame's byte streams stay
-resident as they are; the checkpoint index is built once on the host and the
+``decode(check=)`` and ``gather_rows(ids, check=)``.  The frame's main stream stays
+resident byte for byte.  So does the residual section, with one exception: a frame that
+the fused kernels take and whose residuals are a conditional rANS stream (mode 128) has
+them decoded once on the host at load and kept as packed 6-bit fields, the form mode 0
+frames carry (``resident_mode`` 0, ``mode`` 128; ``resident_bytes`` then exceeds the
+frame's size by the difference).  The checkpoint index is built once on the host and the
 decode runs in hand-written HIP kernels through the C ABI.
 """
 from __future__ import annotations

@@ -446,9 +446,25 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         accept(name, (wrapped, own))
     host_words.clear()
 
+    def residency(context):
+        """What the device holds of a coded tensor, where the backend says so: the frame's mode,
+        the mode of the resident form (a frame whose conditional residual stream was re-packed
+        into 6-bit fields at load is resident in mode 0), and whether the fused kernels take it."""
+        native = getattr(context, "native", context)
+        if not hasattr(native, "resident_mode"):
+            return {}
+        fused = getattr(native, "fused", None) is not None
+        reason = getattr(native, "fused_reason", "")
+        return dict(frame_mode=native.mode, resident_mode=native.resident_mode,
+                    residual_repacked=native.resident_mode != native.mode, fused=fused,
+                    **({} if fused else {"fused_reason": reason}))
+
     consumed, replacements = {}, {}
     for module_name, module, weight_name in coded:
         context, resident = contexts[weight_name]
+        extra = residency(context)
+        if extra and not extra["fused"] and extra["frame_mode"] != 1:
+            log(f"{weight_name}: decoded by the general kernel and multiplied densely ({extra['fused_reason']})")
         if isinstance(module, nn.Linear):
             bias = None
             if module.bias is not None:
@@ -459,10 +475,10 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
                 bias = nn.Parameter(value, requires_grad=False)
                 consumed[bias_name] = record(bias_name, "dense_bias", runtime_dtype=str(runtime))
             replacements[module_name] = BctxLinear(context, bias, batch_invariant=batch_invariant)
-            consumed[weight_name] = record(weight_name, "compressed_linear", resident)
+            consumed[weight_name] = record(weight_name, "compressed_linear", resident, **extra)
         else:
             replacements[module_name] = BctxEmbedding(context, padding_idx=module.padding_idx)
-            consumed[weight_name] = record(weight_name, "compressed_embedding", resident)
+            consumed[weight_name] = record(weight_name, "compressed_embedding", resident, **extra)
     shared_launches = []
     for members in sibling_groups:
         modules = [replacements[m] for m in members]
@@ -507,7 +523,13 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         "resident_context_bytes": sum(consumed[n]["resident_context_bytes"] for n in compressed),
         "dense_parameter_bytes": sum(p.numel() * p.element_size() for p in model.parameters()),
         "buffer_bytes": sum(b.numel() * b.element_size() for b in model.buffers()),
-        "consumed_tensors": consumed, "restored_bf16_control": False, "transcoded": False,
+        "consumed_tensors": consumed, "restored_bf16_control": False,
+        # true when a frame's residual stream is resident in another form than the frame's own
+        # (re-packed 6-bit fields); the main stream and the decoded words are never altered
+        "transcoded": any(r.get("residual_repacked") for r in consumed.values()),
+        "residual_repacked_tensors": sorted(n for n, r in consumed.items() if r.get("residual_repacked")),
+        "general_kernel_tensors": sorted(n for n, r in consumed.items()
+                                         if r.get("fused") is False and r.get("frame_mode") != 1),
         "shared_launches": shared_launches,
     }
     return model, receipt

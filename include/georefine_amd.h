@@ -162,14 +162,13 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  *   lut         u8  [nr][nc << lognb]        lognb = 16 - shift; sparse index of a
  *                                            symbol with slots in the bucket (best: the
  *                                            one owning most of them)
- *   tab         u32 [nr][nc][tabn+1][4]      entry(cc, sparse): start | (freq & 0xFFFF)<<16
- *                                            (0 stands for 65536); symbol<<5; then (freq<<16 |
- *                                            symbol<<5) of the previous and of the next live
- *                                            symbol of the context (0: none); unused entries: 0
+ *   tab         u64 [nr][nc][tabn+1]         entry(cc, sparse): low32 = start |
+ *                                            (freq & 0xFFFF)<<16 (0 stands for 65536),
+ *                                            high32 = symbol<<5; unused entries: 0
  *   col_class   u8  [cols]
- * main_bytes must be readable for 16 bytes past main_n_bytes.  raw6 is 4-byte aligned;
- * with seg_len 64 and 16-byte alignment the GEMV reads a segment's 48 residual bytes
- * once, as it starts, instead of 12 at a time. */
+ * main_bytes must be readable for 16 bytes past main_n_bytes (the kernels copy it in
+ * 16-byte units).  raw6 is 4-byte aligned; with seg_len 64 and 16-byte alignment the slab
+ * kernels read a segment's 48 residual bytes once, as it starts, instead of 12 at a time. */
 typedef struct grf_bctx_fused {
   const uint8_t *main_bytes;
   const uint8_t *raw6;
@@ -189,7 +188,9 @@ typedef struct grf_bctx_fused {
  * one row class; threads is a multiple of 64, at most 1024.
  *   tile_rows   u32 [n_tiles*rows_per_tile]  row of each slot, 0xFFFFFFFF = empty
  *   tile_class  u8  [n_tiles]                row class shared by the tile's rows
- *   piece_cap   LDS bytes reserved per row piece of one slab (multiple of 16)
+ *   piece_cap   LDS bytes reserved per row piece of one slab (multiple of 16): at least the
+ *               longest span from the 16-byte aligned start of a piece's first segment to
+ *               the end of its last one, plus 8 (the refill reads an aligned 8-byte window)
  *   scheme      GRF_TILE_SLABS: lane (r, p) of the workgroup walks segment b*lanes_per_row + p
  *               of the tile's row r in slab b, the whole workgroup slab by slab
  *               (threads >= rows_per_tile*lanes_per_row).
@@ -215,7 +216,10 @@ typedef struct grf_fused_tiling {
  * decode() + F.linear of BctxLinear.forward, :365-376).  y[m][n] = bf16(sum_k x[m][k] *
  * W[n][k] + bias[n]) for 1 <= m_rows <= 8, fp32 accumulation in an order that does not
  * depend on m_rows (the M-invariance contract of GS/miv_gemv.py:10-29).
- * x: BF16 [m_rows][ldx], y: BF16 [m_rows][ldy], bias: BF16 [rows] or NULL. */
+ * x: BF16 [m_rows][ldx], y: BF16 [m_rows][ldy], bias: BF16 [rows] or NULL.  With a
+ * GRF_TILE_WAVES tiling x must be 16-byte aligned with ldx a multiple of 8 (the kernel reads
+ * it in 16-byte vectors, two rows per launch: more rows run as further launches with the same
+ * arithmetic per row); with a GRF_TILE_SLABS tiling 4-byte aligned with an even ldx. */
 int grf_bctx_gemv(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, const uint16_t *x, uint32_t ldx,
                   uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
                   void *hip_stream);
@@ -237,7 +241,7 @@ int grf_bctx_fused_gather(const grf_bctx_fused *frame, const grf_fused_tiling *t
 /* Fused decode-GEMM on the matrix cores for any number of activation rows; same operand
  * meaning as grf_bctx_gemv.  Batch-invariant in the sense of GS/bi_csrc/bi_gemm.cuh:1-17:
  * with one tiling, row m of y is a function of row m of x and of W only.  x must be
- * 8-byte aligned with ldx a multiple of 4.  More than 64 rows run as several launches.
+ * 8-byte aligned with ldx a multiple of 4.  More than 128 rows run as several launches.
  *
  * A tiling for this function has threads = 64 * ceil(rows_per_tile / 16) *
  * ceil(lanes_per_row / 4): a wave walks four lane-segments of 16 rows and feeds the words
