@@ -133,14 +133,8 @@ def verify(package, decoder=codec.decode):
         decode_tensor(package, row, decoder)
         source += row["source_bytes"]
         coded += row["frame_bytes"]
-    for name, pin in (manifest.get("metadata_assets") or {}).items():
-        rel = PurePosixPath(name)
-        if rel.is_absolute() or ".." in rel.parts or not rel.parts or rel.parts[0] != "sidecars":
-            raise PackageError(f"unsafe metadata asset name: {name!r}")
-        payload = Path(package).joinpath(*rel.parts).read_bytes()
-        if len(payload) != pin.get("bytes") or hashlib.sha256(payload).hexdigest() != pin.get("sha256"):
-            raise PackageError(f"sidecar integrity mismatch: {name}")
-    return {"tensors": len(entries), "source_bytes": source, "frame_bytes": coded}
+    sidecars = read_metadata(package, manifest) if ("metadata_assets" in manifest or "files" in manifest) else {}
+    return {"tensors": len(entries), "source_bytes": source, "frame_bytes": coded, "metadata_assets": len(sidecars)}
 
 
 def _words(tensor):
@@ -189,6 +183,104 @@ def write_package(package, tensors, *, row_classes=16, col_classes=4, sidecars=N
                 "tensors": rows, "metadata_assets": assets}
     (package / "manifest.json").write_text(json.dumps(manifest, indent=1), encoding="utf-8")
     return manifest
+
+
+# ------------------------------------------------------------------ metadata sidecars
+
+def _asset_name(name):
+    if not isinstance(name, str):
+        raise PackageError("metadata asset name must be a string")
+    rel = PurePosixPath(name)
+    if (rel.is_absolute() or not rel.parts or rel.parts[0] != "sidecars" or ".." in rel.parts or "." in rel.parts
+            or rel.as_posix() != name):
+        raise PackageError(f"unsafe metadata asset name: {name!r}")
+    return name
+
+
+def read_metadata(package, manifest):
+    """The package's metadata sidecars (configuration files of the model), every byte checked
+    against the manifest: name -> bytes.
+
+    A package pins them twice (GCR/bitexact_context_serving.py:131-236): ``metadata_assets``
+    gives size and SHA-256 per sidecar, and ``files`` pins the archive ``model-assets.tar.xz``
+    that holds them; ``source.index_sha256``, where present, pins the archived safetensors
+    index once more.  A package may also carry the sidecars as plain files under
+    ``sidecars/``: they must then be exactly the pinned set.  Packages written by
+    ``write_package`` have plain files only.  Nothing is extracted to disk here."""
+    import io
+    import lzma
+    import tarfile
+    package = Path(package)
+    assets = manifest.get("metadata_assets")
+    if not isinstance(assets, dict):
+        raise PackageError("manifest metadata_assets must be an object")
+    pins = {}
+    for name, pin in assets.items():
+        name = _asset_name(name)
+        if (not isinstance(pin, dict) or type(pin.get("bytes")) is not int or pin["bytes"] < 0
+                or not _is_digest(pin.get("sha256"))):
+            raise PackageError(f"invalid metadata asset pin: {name}")
+        pins[name] = pin
+
+    def check(found, what):
+        if set(found) != set(pins):
+            raise PackageError(f"{what} differ from manifest metadata_assets")
+        for name, payload in found.items():
+            if len(payload) != pins[name]["bytes"] or hashlib.sha256(payload).hexdigest() != pins[name]["sha256"]:
+                raise PackageError(f"{what}: integrity mismatch: {name}")
+
+    members = None
+    files = manifest.get("files")
+    if files is not None:
+        if not isinstance(files, list):
+            raise PackageError("manifest files must be a list")
+        by_path = {}
+        for item in files:
+            if not isinstance(item, dict) or not isinstance(item.get("path"), str) or item["path"] in by_path:
+                raise PackageError("malformed or duplicate package file inventory")
+            by_path[item["path"]] = item
+        pin = by_path.get("model-assets.tar.xz")
+        if pin is not None:
+            if type(pin.get("bytes")) is not int or not _is_digest(pin.get("sha256")):
+                raise PackageError("manifest lacks model-assets.tar.xz byte/SHA pin")
+            path = package / "model-assets.tar.xz"
+            if path.is_symlink() or not path.is_file():
+                raise PackageError("metadata archive must be a regular file")
+            archive = path.read_bytes()
+            if len(archive) != pin["bytes"] or hashlib.sha256(archive).hexdigest() != pin["sha256"]:
+                raise PackageError("metadata archive size/SHA mismatch")
+            members = {}
+            try:
+                with tarfile.open(fileobj=io.BytesIO(archive), mode="r:xz") as tf:
+                    for member in tf.getmembers():
+                        name = _asset_name(member.name)
+                        if name in members or not member.isfile():
+                            raise PackageError(f"duplicate or irregular metadata archive member: {name}")
+                        members[name] = tf.extractfile(member).read()
+            except (tarfile.TarError, lzma.LZMAError) as exc:
+                raise PackageError("invalid xz metadata archive") from exc
+            check(members, "metadata archive members")
+            index_sha = (manifest.get("source") or {}).get("index_sha256")
+            index = members.get("sidecars/model.safetensors.index.json")
+            if index_sha is not None and (index is None or hashlib.sha256(index).hexdigest() != index_sha):
+                raise PackageError("archived safetensors index differs from manifest source pin")
+    physical = None
+    source = package / "sidecars"
+    if source.exists():
+        if source.is_symlink() or not source.is_dir():
+            raise PackageError("physical sidecars must be a regular directory")
+        physical = {}
+        for path in sorted(source.rglob("*")):
+            if path.is_symlink():
+                raise PackageError("physical sidecars contain a symlink")
+            if path.is_file():
+                physical[path.relative_to(package).as_posix()] = path.read_bytes()
+        check(physical, "physical sidecars")
+    if members is None and physical is None:
+        if pins:
+            raise PackageError("package holds neither a metadata archive nor sidecar files")
+        return {}
+    return members if members is not None else physical
 
 
 # ------------------------------------------------------------------ predictive candidates

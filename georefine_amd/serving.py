@@ -37,22 +37,48 @@ def hip_predictive_factory(frame, reference_uint16_numpy, stride=1024, device="c
 class SharedProducts:
     """Sibling linears that are applied to the same tensor one after the other (q/k/v
     projections, gate and up) as one launch: the first member called with a tensor runs the
-    whole group and keeps the outputs, the others pick theirs up.  A call with another tensor
-    (identity, version counter, address or shape) runs the group again."""
+    whole group and keeps the outputs, the others pick theirs up.  Every output is handed out
+    once: when the last member has taken its own, or a member asks again, or the tensor differs
+    (identity, version counter, address, shape), the next call runs the group anew.  Within
+    one pass the kept outputs assume that the activations were not rewritten behind the
+    version counter (a kernel writing through a raw pointer, a graph replay): callers that do
+    that between the members' calls must not share launches."""
 
     def __init__(self, group, biases, batch_invariant=False):
         self.group, self.biases, self.batch_invariant = group, list(biases), batch_invariant
         self.launches = 0
         self._key = self._x = self._outs = None
+        self._taken = set()
 
     def output(self, index, x):
         key = (id(x), x._version, x.data_ptr(), tuple(x.shape), tuple(x.stride()))
-        if key != self._key or self._x is None or self._x() is not x:
+        if key != self._key or self._outs is None or self._x() is not x or index in self._taken:
             import weakref
-            self._outs = self.group.linear(x, self.biases, batch_invariant=self.batch_invariant)
-            self._key, self._x = key, weakref.ref(x)
+            self._outs = list(self.group.linear(x, self.biases, batch_invariant=self.batch_invariant))
+            self._key, self._x, self._taken = key, weakref.ref(x), set()
             self.launches += 1
-        return self._outs[index]
+        out, self._outs[index] = self._outs[index], None
+        self._taken.add(index)
+        if len(self._taken) == len(self._outs):  # the pass is over: nothing is kept beyond it
+            self._key = self._x = self._outs = None
+            self._taken = set()
+        return out
+
+
+def decode_errors(model):
+    """Names of the coded modules of ``model`` whose device error word is set (a segment did
+    not end on its checkpoint in some launch since the word was last cleared).  The fused
+    kernels never trap and ``linear`` does not read the word back on every call; a server calls
+    this between steps, or every so many steps: one small device-to-host read per module."""
+    bad = []
+    for name, module in model.named_modules():
+        weight = getattr(module, "context_weight", None)
+        words = [getattr(getattr(weight, "native", weight), "error", None)]
+        if getattr(module, "shared", None) is not None:
+            words.append(getattr(module.shared[0].group, "error", None))
+        if any(w is not None and int(w.item()) != 0 for w in words):
+            bad.append(name)
+    return bad
 
 
 class BctxLinear(nn.Module):
@@ -231,6 +257,8 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
     package = Path(package)
     try:
         manifest, entries = pkg.read_manifest(package)
+        # the model's configuration sidecars are checked against their pins before any weight is read
+        sidecars = pkg.read_metadata(package, manifest) if ("metadata_assets" in manifest or "files" in manifest) else {}
     except pkg.PackageError as exc:
         raise ContextServingError(str(exc)) from exc
     if tensor_factory is None:
@@ -516,7 +544,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
     receipt = {
         "schema": "georefine.bctx_serving_load.v1", "status": "ok", "format": "BCTX v1",
         "device": str(device), "dtype_default": str(dtype),
-        "package_manifest": str(package / "manifest.json"),
+        "package_manifest": str(package / "manifest.json"), "verified_metadata_assets": sorted(sidecars),
         "tensor_count": len(entries), "consumed_count": len(consumed),
         "unused_package_tensors": sorted(set(entries) - set(consumed)),
         "compressed_tensor_count": len(compressed),

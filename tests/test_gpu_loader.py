@@ -175,3 +175,14 @@ def test_sibling_projections_share_a_launch(tmp_path):
     assert torch.equal(alone.view(torch.uint16), plain.blocks[0].k_proj(x).view(torch.uint16))
     x.add_(1)  # the same tensor object with new contents: not served from the kept outputs
     assert torch.equal(first.k_proj(x).view(torch.uint16), plain.blocks[0].k_proj(x).view(torch.uint16))
+    # an output is handed out once: the same member asking again with the same tensor runs the group again
+    before = first.k_proj.shared[0].launches
+    again = first.k_proj(x)
+    assert first.k_proj.shared[0].launches == before + 1
+    assert torch.equal(again.view(torch.uint16), plain.blocks[0].k_proj(x).view(torch.uint16))
+    # the receipt says what is resident, and no launch of all these reported a decode error
+    for name, row in receipt["consumed_tensors"].items():
+        if row["kind"].startswith("compressed"):
+            assert row["fused"] == (row["frame_mode"] != 1) and row["residual_repacked"] == (row["frame_mode"] == 128)
+    assert receipt["transcoded"] == bool(receipt["residual_repacked_tensors"])
+    assert serving.decode_errors(shared) == [] and serving.decode_errors(plain) == []

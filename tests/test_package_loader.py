@@ -105,7 +105,7 @@ def test_reader_rejects_tampering(tmp_path):
         pkg.verify(path)
     (path / "sidecars" / "config.json").write_bytes(b"{}")
     frame.write_bytes(bytes(data[:-1]) + bytes([data[-1] ^ 1]))
-    with pytest.raises(pkg.PackageError, match="sidecar integrity"):
+    with pytest.raises(pkg.PackageError, match="physical sidecars: integrity mismatch"):
         pkg.verify(path)
 
 
@@ -150,6 +150,102 @@ def test_loader_fills_model_and_matches_dense(tmp_path, workers):
     assert receipt["consumed_tensors"]["lin.bias"]["kind"] == "dense_bias"
     assert receipt["consumed_tensors"]["fp32_exception"]["runtime_dtype"] == "torch.float32"
     assert receipt["transcoded"] is False and seen and seen[-1][:2] == (2, 2)
+
+
+def _reference_shaped_package(tmp_path, *, bad_archive=False, bad_asset_pin=False, bad_index_pin=False,
+                              physical_sidecars=False):
+    """A package whose manifest has the fields, names and nesting of the one the reference's
+    own loader test assembles (tests/test_bitexact_context_serving.py:50-118 of the reference):
+    thirteen sidecars pinned under ``metadata_assets`` and archived as model-assets.tar.xz,
+    that archive pinned under ``files``, the safetensors index pinned again under
+    ``source.index_sha256``, tensor receipts with name / dtype / shape / source_bytes / frame /
+    frame_bytes / frame_sha256 / source_sha256 / complete, frames named frames/<i>.bctx.  The
+    frames here are real BCTX frames (the reference's test stores placeholders and decodes them
+    with a stand-in)."""
+    import io
+    import tarfile
+    package = tmp_path / "package"
+    (package / "frames").mkdir(parents=True)
+    sidecars = {
+        "sidecars/config.json": b'{"eos_token_id":248044,"pad_token_id":null}',
+        "sidecars/generation_config.json": b'{"eos_token_id":[248046,248044],"pad_token_id":248044}',
+        "sidecars/model.safetensors.index.json": b'{"weight_map":{}}',
+    }
+    for i in range(10):
+        sidecars[f"sidecars/asset-{i:02d}.json"] = f'{{"asset":{i}}}'.encode()
+    assets = {name: {"bytes": len(data), "sha256": hashlib.sha256(data).hexdigest()} for name, data in sidecars.items()}
+    if bad_asset_pin:
+        assets["sidecars/config.json"]["sha256"] = "0" * 64
+    buffer = io.BytesIO()
+    with tarfile.open(fileobj=buffer, mode="w:xz") as tf:
+        for name, payload in sidecars.items():
+            member = tarfile.TarInfo(name)
+            member.size = len(payload)
+            tf.addfile(member, io.BytesIO(payload))
+    archive = buffer.getvalue()
+    archive_sha = hashlib.sha256(archive).hexdigest()
+    if bad_archive:
+        archive = archive[:12] + bytes([archive[12] ^ 1]) + archive[13:]
+    (package / "model-assets.tar.xz").write_bytes(archive)
+    if physical_sidecars:
+        for name, payload in sidecars.items():
+            (package / name).parent.mkdir(parents=True, exist_ok=True)
+            (package / name).write_bytes(payload)
+    tensors = _tensors()
+    tensors["mtp.layers.0.weight"] = torch.ones(2, 2, dtype=torch.bfloat16)
+    rows = []
+    for i, (name, tensor) in enumerate(tensors.items()):
+        words = tensor.contiguous().view(torch.uint16).numpy()
+        frame = codec.encode(words.reshape(pkg.frame_shape(list(tensor.shape))))
+        rel = f"frames/{i}.bctx"
+        (package / rel).write_bytes(frame)
+        rows.append({"name": name, "dtype": "BF16", "shape": list(tensor.shape), "source_bytes": tensor.numel() * 2,
+                     "frame": rel, "frame_bytes": len(frame), "frame_sha256": hashlib.sha256(frame).hexdigest(),
+                     "source_sha256": hashlib.sha256(words.tobytes()).hexdigest(), "complete": True})
+    index_sha = hashlib.sha256(sidecars["sidecars/model.safetensors.index.json"]).hexdigest()
+    (package / "manifest.json").write_text(json.dumps({
+        "schema": "bitexact-context-package-v1", "complete": True, "tensors": rows, "metadata_assets": assets,
+        "source": {"index_sha256": "0" * 64 if bad_index_pin else index_sha},
+        "files": [{"path": "model-assets.tar.xz", "bytes": len(archive), "sha256": archive_sha}],
+    }))
+    return package, tensors, sidecars
+
+
+@pytest.mark.parametrize("physical", [False, True])
+def test_loader_reads_a_manifest_of_the_reference_shape(tmp_path, physical):
+    package, tensors, sidecars = _reference_shaped_package(tmp_path, physical_sidecars=physical)
+    manifest, entries = pkg.read_manifest(package)
+    assert set(entries) == set(tensors) and pkg.read_metadata(package, manifest) == sidecars
+    totals = pkg.verify(package)
+    model, receipt = _load(package)
+    assert receipt["status"] == "ok" and receipt["verified_metadata_assets"] == sorted(sidecars)
+    assert receipt["compressed_tensor_count"] == 2 and len(receipt["verified_metadata_assets"]) == 13
+    assert sorted(receipt["unused_package_tensors"]) == ["mtp.layers.0.weight"]
+    dense = TinyModel()
+    with torch.no_grad():
+        for name, p in dense.named_parameters():
+            p.copy_(tensors[name].float())
+    ids = torch.tensor([[0, 3, 7]])
+    assert torch.allclose(model(ids).float(), dense(ids).float(), atol=2e-2, rtol=2e-2)
+    assert totals
+
+
+@pytest.mark.parametrize("fault,message", [
+    (dict(bad_archive=True), "metadata archive size/SHA mismatch"),
+    (dict(bad_asset_pin=True), "integrity mismatch: sidecars/config.json"),
+    (dict(bad_index_pin=True), "safetensors index differs"),
+])
+def test_loader_rejects_metadata_that_misses_its_pins(tmp_path, fault, message):
+    package, _, _ = _reference_shaped_package(tmp_path, **fault)
+    with pytest.raises(serving.ContextServingError, match=message):
+        _load(package)
+
+
+def test_loader_rejects_stray_physical_sidecars(tmp_path):
+    package, _, _ = _reference_shaped_package(tmp_path, physical_sidecars=True)
+    (package / "sidecars" / "extra.json").write_bytes(b"{}")
+    with pytest.raises(serving.ContextServingError, match="physical sidecars differ"):
+        _load(package)
 
 
 def test_loader_errors(tmp_path):
