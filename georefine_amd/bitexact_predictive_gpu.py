@@ -141,7 +141,7 @@ class HipPredictiveTensor:
     DENSE_ABOVE = 128  # activation rows above which linear() decodes to a dense transient
 
     def __init__(self, frame, reference_uint16_numpy, stride=1024, device="cuda:0", *, fused=True,
-                 fused_segment=None):
+                 fused_segment=None, resident_contexts=True):
         if not isinstance(stride, int) or not 1 <= stride <= 65536:
             raise codec.CodecError("invalid checkpoint stride")
         ix = _read_frame(frame, reference_uint16_numpy, stride, fused=fused, fused_segment=fused_segment)
@@ -197,6 +197,24 @@ class HipPredictiveTensor:
                 self._prepare_fused()
             except _fused.FusedUnsupported as exc:
                 self.fused, self.fused_reason = None, str(exc)
+        # What the tile walker needs of the reference is the 4-bit bin of every word (the
+        # decoded word itself comes from the frame's symbols alone), and the reference is given
+        # here, once.  Keeping that plane, half a byte per weight, takes the reference out of
+        # every later call: a product is then one launch over the frame's bytes and the plane,
+        # with no dense reference anywhere.  (The reference's kernels form the bin from the
+        # reference word inside the decode loop, GCR/bitexact_predictive_gpu_kernels.py:36-42,
+        # which needs the dense reference resident.)
+        self.has_contexts = False
+        if self.fused is not None and resident_contexts:
+            words = np.ascontiguousarray(reference_uint16_numpy, dtype=np.uint16).reshape(self.shape)
+            ref = torch.from_numpy(words).to(self.device)  # transient
+            with torch.cuda.device(self.device):
+                bins, status = self._bins(ref)
+                torch.cuda.synchronize(self.device)
+            self._status(status, False)
+            self.buffers["context_bins"] = bins
+            self.has_contexts = True
+            del ref
 
     @property
     def resident_bytes(self):
@@ -250,8 +268,18 @@ class HipPredictiveTensor:
                                          torch.cuda.current_stream(self.device).cuda_stream)
         return bins, status
 
+    def _contexts(self, reference_bf16_device):
+        """(bins plane, status): the resident plane, or one made from the reference given."""
+        if self.has_contexts:
+            return self.buffers["context_bins"], 0
+        if reference_bf16_device is None:
+            raise ValueError("this tensor keeps no context plane: the reference must be given")
+        return self._bins(self._reference(reference_bf16_device))
+
     def _reference(self, reference_bf16_device):
         import torch
+        if reference_bf16_device is None:
+            raise ValueError("the one-lane-per-checkpoint kernel decodes against the reference: it must be given")
         ref = reference_bf16_device.to(device=self.device).contiguous()
         if tuple(ref.shape) != tuple(self.shape) or ref.dtype != torch.bfloat16:
             raise ValueError("reference device tensor shape/dtype mismatch")
@@ -289,7 +317,6 @@ class HipPredictiveTensor:
             raise codec.CodecError("frame is not eligible for the fused kernels: " + str(self.fused_reason))
         from .bitexact_context_gpu import PackedActivations
         packed = x if isinstance(x, PackedActivations) else None
-        ref = self._reference(reference_bf16_device)
         if packed is not None:
             if not use_gemm or packed.cols != self.shape[1] or packed.buffer.device != self.device:
                 raise ValueError("packed activations go to the GEMM of a weight of their width on their device")
@@ -311,7 +338,7 @@ class HipPredictiveTensor:
             if check:  # between checks the word keeps what earlier launches reported
                 self.error.zero_()
             with torch.cuda.device(self.device):
-                bins, status = self._bins(ref)
+                bins, status = self._contexts(reference_bf16_device)
                 if not status:
                     extra = ()
                     if use_gemm:
@@ -346,13 +373,12 @@ class HipPredictiveTensor:
         import torch
         if self.mode == 2:
             return self.buffers["raw"].view(torch.bfloat16).reshape(self.shape)
-        ref = self._reference(reference_bf16_device)
         if self.fused is not None and not general:
             out = torch.empty(self.shape, device=self.device, dtype=torch.uint16)
             if check:  # between checks the word keeps what earlier launches reported
                 self.error.zero_()
             with torch.cuda.device(self.device):
-                bins, status = self._bins(ref)
+                bins, status = self._contexts(reference_bf16_device)
                 if not status:
                     status = self._lib.grf_ppcx_fused_decode(ctypes.byref(self.fused),
                                                              ctypes.byref(self._tiling_for(0)[0]), bins.data_ptr(),
@@ -360,6 +386,7 @@ class HipPredictiveTensor:
                                                              torch.cuda.current_stream(self.device).cuda_stream)
             self._status(status, check)
             return out.view(torch.bfloat16)
+        ref = self._reference(reference_bf16_device)
         count = (self.n + self.stride - 1) // self.stride
         out = torch.empty(count * self.stride, device=self.device, dtype=torch.uint16)
         if check:  # between checks the word keeps what earlier launches reported

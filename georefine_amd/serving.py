@@ -163,9 +163,14 @@ class PredictiveContextTensor:
         self.resident_bytes = resident_bytes
         self._decode_lock = threading.RLock()
 
+    def _needs_reference(self):
+        """False when the native tensor keeps the contexts of its reference and takes the tile
+        walker: nothing of the references is then read after load."""
+        return not (getattr(self.native, "has_contexts", False) and getattr(self.native, "fused", None) is not None)
+
     def decode(self, *, check=True):
         with self._decode_lock:
-            value = self.native.decode(self._reference(check), check=check)
+            value = self.native.decode(self._reference(check) if self._needs_reference() else None, check=check)
             if self.transform == "target transpose":
                 value = value.transpose(-2, -1).contiguous()
             return value
@@ -184,13 +189,16 @@ class PredictiveContextTensor:
 
     def linear(self, x, bias=None, *, check=False, batch_invariant=False):
         """x W^T + bias.  A frame stored untransposed goes through the native tensor's fused
-        product (reference decoded, then decode and dot in one kernel); a transposed frame holds
-        W^T row by row, so it is decoded and multiplied densely."""
+        product: one launch that decodes and contracts, with the contexts of the reference read
+        from the plane kept at load (a native tensor without that plane gets the reference
+        decoded first); a transposed frame holds W^T row by row, so it is decoded and multiplied
+        densely."""
         fused = getattr(self.native, "linear", None)
         if fused is None or self.transform == "target transpose":
             return torch.nn.functional.linear(x, self.decode(check=check), bias)
         with self._decode_lock:
-            return fused(self._reference(check), x, bias, check=check, batch_invariant=batch_invariant)
+            return fused(self._reference(check) if self._needs_reference() else None, x, bias, check=check,
+                         batch_invariant=batch_invariant)
 
 
 # ----------------------------------------------------------------------------- loader

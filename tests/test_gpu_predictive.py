@@ -95,15 +95,28 @@ def test_ppcx_wrong_reference_on_device_sets_error(oracle):
     from georefine_amd import bitexact_predictive_codec as codec
     from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
     _, target, ref = next(_pairs())
-    t = HipPredictiveTensor(_frame_for_mode(codec, target, ref, 0), ref, stride=64)
+    frame = _frame_for_mode(codec, target, ref, 0)
+    t = HipPredictiveTensor(frame, ref, stride=64, resident_contexts=False)  # contexts from the reference of each call
     other = torch.from_numpy(np.roll(ref, 3, axis=1).copy()).view(torch.bfloat16).cuda()
-    assert t.fused is not None
+    assert t.fused is not None and not t.has_contexts
     with pytest.raises(codec.CodecError):  # contexts differ: segments miss their checkpoints
         t.decode(other)
     with pytest.raises(codec.CodecError):
         t.decode(other, general=True)
     with pytest.raises(ValueError):
         t.decode(other[:, :8])
+    with pytest.raises(ValueError):
+        t.decode(None)
+    # a tensor that keeps its context plane (the default) needs no reference after construction
+    kept = HipPredictiveTensor(frame, ref, stride=64)
+    assert kept.has_contexts and kept.resident_bytes == t.resident_bytes + target.size // 2
+    assert np.array_equal(kept.decode(None).view(torch.uint16).cpu().numpy(), target)
+    x = torch.from_numpy(bf16_words(np.random.default_rng(5).normal(0, 1, size=(3, target.shape[1])))).view(torch.bfloat16).cuda()
+    ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
+    for rows in (1, 3):
+        assert torch.equal(kept.linear(None, x[:rows]).view(torch.uint16), t.linear(ref_dev, x[:rows]).view(torch.uint16))
+    with pytest.raises(ValueError):  # the one-lane-per-checkpoint kernel reads the reference words themselves
+        kept.decode(None, general=True)
 
 
 def test_mix_predict_device_matches_host_bits(oracle):
@@ -166,7 +179,8 @@ def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle,
     target = weight_like(rng, 200, 1280)
     tf = (target.astype(np.uint32) << 16).view(np.float32)
     ref = bf16_words(tf + rng.normal(0, 0.003, target.shape).astype(np.float32))
-    t = HipPredictiveTensor(_frame_for_mode(codec, target, ref, mode), ref, stride=1024, device="cuda:0")
+    t_frame = _frame_for_mode(codec, target, ref, mode)
+    t = HipPredictiveTensor(t_frame, ref, stride=1024, device="cuda:0")
     assert t.fused is not None, t.fused_reason
     ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
     dense_w = torch.from_numpy(target).view(torch.bfloat16).cuda().float()
@@ -194,9 +208,14 @@ def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle,
     for m in (1, 8, 17, 32):
         ym = t.linear(ref_dev, x[:m], bias, batch_invariant=True)
         assert torch.equal(ym.view(torch.uint16), y40[:m].view(torch.uint16)), m
+    # the tensor keeps the contexts of the reference it was built with: the argument is not read
+    assert t.has_contexts
+    assert torch.equal(t.linear(None, x, bias, check=True).view(torch.uint16), y40.view(torch.uint16))
     wrong = torch.from_numpy(np.roll(ref, 5, axis=1).copy()).view(torch.bfloat16).cuda()
-    with pytest.raises(codec.CodecError):
-        t.linear(wrong, x[:2], check=True)
+    per_call = HipPredictiveTensor(t_frame, ref, stride=1024, device="cuda:0", resident_contexts=False)
+    assert torch.equal(per_call.linear(ref_dev, x, bias, check=True).view(torch.uint16), y40.view(torch.uint16))
+    with pytest.raises(codec.CodecError):  # contexts of another reference: segments miss their checkpoints
+        per_call.linear(wrong, x[:2], check=True)
 
 
 # ---------------------------------------------------------------- seeded sweep over predictive frames
