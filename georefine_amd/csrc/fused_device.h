@@ -349,13 +349,14 @@ __device__ __forceinline__ uint32_t fused_stage_piece(uint8_t *lds, uint32_t pie
 // vector-memory counter says so; lanes of the same wave read them afterwards.
 __device__ __forceinline__ uint32_t fused_stage_piece_dma(uint8_t *lds, uint32_t region0, uint32_t cap,
                                                           const grf_bctx_fused &f, uint32_t g0, uint32_t g1, uint32_t rl,
-                                                          uint32_t p, uint32_t P, uint32_t rows_per_wave) {
+                                                          uint32_t p, uint32_t logp, uint32_t rows_per_wave) {
   typedef __attribute__((address_space(3))) void lds_void;
+  const uint32_t P = 1u << logp;
   const uint32_t a0 = g0 & ~15u;
   // rounds the longest piece of the wave needs (uniform: every lane takes part in the ballots)
   uint32_t longest = g1 > a0 ? g1 - a0 : 0;
   for (uint32_t d = P; d < 64; d <<= 1) longest = max(longest, (uint32_t)__shfl_xor((int)longest, (int)d, 64));
-  const uint32_t rounds = (longest + P * 16 - 1) / (P * 16);
+  const uint32_t rounds = (longest + P * 16 - 1) >> (logp + 4);
   for (uint32_t i = 0; i < rounds; ++i) {
     const uint32_t o = a0 + (i * P + p) * 16;
     for (uint32_t r = 0; r < rows_per_wave; ++r) {  // uniform

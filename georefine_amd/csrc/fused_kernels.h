@@ -251,40 +251,84 @@ struct WaveLdsLayout {
   }
 };
 
+// Sum over the P = 2^logp lanes of a row group, delivered in the group's first lane (other
+// lanes end with partial sums).  Pairwise, neighbours first: ((l0 + l1) + (l2 + l3)) + ...; the
+// first four levels stay inside a row of sixteen lanes and are lane-permuting adds (no LDS
+// round trip), wider groups finish with wave shuffles.
+__device__ __forceinline__ float group_sum_to_first_lane(float v, uint32_t logp) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  auto moved = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value, 0xF,
+                                                                  0xF, false));
+  };
+  v += moved(v, std::integral_constant<int, 0xB1>{});                 // lanes i ^ 1 (quad permute 1,0,3,2)
+  v += moved(v, std::integral_constant<int, 0x4E>{});                 // lanes i ^ 2 (quad permute 2,3,0,1)
+  if (logp >= 3) v += moved(v, std::integral_constant<int, 0x141>{});  // mirror within 8: lane 0 takes lane 7's quad sum
+  if (logp >= 4) v += moved(v, std::integral_constant<int, 0x140>{});  // mirror within 16: lane 0 takes lane 15's half sum
+  if (logp >= 5) v += __shfl_xor(v, 16, 64);
+  if (logp >= 6) v += __shfl_xor(v, 32, 64);
+#else
+  (void)logp;
+#endif
+  return v;
+}
+
 template <class Walk, int M>
 __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fused &f, const grf_fused_tiling &g,
                                                 const uint16_t *x, uint32_t ldx, uint16_t *y, uint32_t ldy,
                                                 const uint16_t *bias, int32_t *error, uint32_t tile) {
   const WaveLdsLayout L(f, g, M);
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
-  const uint32_t wave = tid / 64, lane = tid % 64, nwaves = nthreads / 64;
+  const uint32_t lane = tid % 64, nwaves = nthreads / 64;
+#if defined(__HIP_DEVICE_COMPILE__)
+  // the wave's number, told to the compiler as the scalar it is: the unit loop's counters
+  // and branches then live in scalar registers
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);
+#else
+  const uint32_t wave = tid / 64;
+#endif
   const uint32_t P = g.lanes_per_row, rpw = 64 / P, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
-  const uint32_t rl = lane / P, p = lane % P;
+  // P is a power of two: lane coordinates by shift and mask.  A unit u = (row group grp, slab b)
+  // with u = grp * n_slabs + b; a wave steps through its units u = wave, wave + nwaves, ... by
+  // adding (nwaves / n_slabs, nwaves % n_slabs) with a carry, in scalar registers: divisions by
+  // values only known at run time cost some twenty vector instructions each, and there were
+  // six of them per unit.
+  const uint32_t logp = 31 - __builtin_clz(P);
+  const uint32_t rl = lane >> logp, p = lane & (P - 1);
   float *sub = reinterpret_cast<float *>(lds + L.sub);
   uint32_t *rows = reinterpret_cast<uint32_t *>(lds + L.rows);
   const uint32_t piece_off = L.stream + (wave * rpw + rl) * g.piece_cap;
   const uint32_t groups = (R + rpw - 1) / rpw, units = groups * g.n_slabs;
+  const uint32_t step_grp = nwaves / g.n_slabs, step_b = nwaves % g.n_slabs;
   uint32_t bad = 0;
 
   // The byte range [g0, g1) of a unit's row piece is the first of two dependent reads before
   // the piece can be copied, so it is read one unit ahead (and the first one before the
   // tables are copied).
-  auto span_of = [&](uint32_t u, uint32_t row, uint32_t &g0, uint32_t &g1) {
-    g0 = g1 = 0;
-    if (row == grf::kNoRow) return;
-    const uint32_t first_seg = (u % g.n_slabs) * P;
-    const uint32_t seg_base = row * f.segs_per_row + first_seg;
+  // (Loads in a branch that only some lanes take make the compiler wait for every load in
+  // flight where the branch ends, so lanes without a row read the matrix's first entries and
+  // discard them.)
+  auto span_of = [&](uint32_t b, uint32_t row, uint32_t &g0, uint32_t &g1) {
+    const uint32_t first_seg = b << logp;
+    const uint32_t seg_base = row == grf::kNoRow ? 0 : row * f.segs_per_row + first_seg;
+    const uint32_t past = row == grf::kNoRow ? 0 : min(P, f.segs_per_row - first_seg);
     g0 = f.seg_offset[seg_base];
-    g1 = f.seg_offset[seg_base + min(P, f.segs_per_row - first_seg)];
+    g1 = f.seg_offset[seg_base + past];  // (no row: an empty range)
   };
+  auto advance = [&](uint32_t &grp, uint32_t &b) {  // the unit nwaves further on
+    grp += step_grp;
+    b += step_b;
+    if (b >= g.n_slabs) b -= g.n_slabs, ++grp;
+  };
+  uint32_t grp = wave / g.n_slabs, b = wave % g.n_slabs;  // this wave's first unit
   uint32_t row, g0, g1;
   {
-    const uint32_t slot0 = (wave / g.n_slabs) * rpw + rl;
+    const uint32_t slot0 = grp * rpw + rl;
     row = (wave < units && slot0 < R) ? g.tile_rows[tile * R + slot0] : grf::kNoRow;
     if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
-    span_of(wave, row, g0, g1);
+    span_of(b, row, g0, g1);
   }
   for (uint32_t i = tid; i < R; i += nthreads) {
     const uint32_t rw = g.tile_rows[tile * R + i];
@@ -292,85 +336,88 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
   }
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   __syncthreads();
-  for (uint32_t u = wave; u < units; u += nwaves) {  // wave-uniform
+  const uint32_t later_half = blockIdx.x >= gridDim.x / 2 ? 1u : 0u;
+  uint32_t left = wave < units ? (units - 1 - wave) / nwaves : 0;  // units after the current one
+  for (uint32_t u = wave; u < units; u += nwaves, --left) {  // wave-uniform
 #if defined(__HIP_DEVICE_COMPILE__)
     // Waves with more units still to do go first.  Left alone the arbiter prefers the older
     // of the two workgroups that share a compute unit, which then finishes long before the
     // other and leaves it the unit at half occupancy.
-    switch (min(3u, (units - 1 - u) / nwaves + (blockIdx.x >= gridDim.x / 2 ? 1u : 0u))) {  // + the later-started half
+    switch (min(3u, left + later_half)) {  // + the later-started half
       case 0: __builtin_amdgcn_s_setprio(0); break;
       case 1: __builtin_amdgcn_s_setprio(1); break;
       case 2: __builtin_amdgcn_s_setprio(2); break;
       default: __builtin_amdgcn_s_setprio(3); break;
     }
 #endif
-    const uint32_t slot = (u / g.n_slabs) * rpw + rl, b = u % g.n_slabs;
-    const uint32_t first_seg = b * P;
+    const uint32_t slot = grp * rpw + rl;
+    const uint32_t first_seg = b << logp;
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
     if (u != wave) row = slot < R ? rows[slot] : grf::kNoRow;  // (read again: cheaper than a register over the walk)
     const bool walks = row != grf::kNoRow && p < nseg;
     const uint32_t col0 = (first_seg + p) * S;
     Walk w;
-    if (walks) w.prefetch(f, row * f.segs_per_row + first_seg + p, (uint64_t)row * K + col0, col0);
-    const uint32_t a0 = grf::fused_stage_piece_dma(lds, L.stream + wave * rpw * g.piece_cap, g.piece_cap, f, g0, g1, rl, p, P, rpw);
+    {  // every lane loads (see span_of); lanes that do not walk read segment 0's entries
+      const uint32_t seg = walks ? row * f.segs_per_row + first_seg + p : 0;
+      w.prefetch(f, seg, walks ? (uint64_t)row * K + col0 : 0, walks ? col0 : 0);
+    }
+    const uint32_t a0 = grf::fused_stage_piece_dma(lds, L.stream + wave * rpw * g.piece_cap, g.piece_cap, f, g0, g1, rl, p, logp, rpw);
     if (walks) w.start(piece_off, a0);
+    const uint32_t slot_base = grp * rpw, slab = b;  // this unit's, kept while the counters move on
     {  // the next unit's byte range, on its way during this unit's walk
-      const uint32_t un = u + nwaves, sn = (un / g.n_slabs) * rpw + rl;
-      span_of(un, (un < units && sn < R) ? rows[sn] : grf::kNoRow, g0, g1);
+      advance(grp, b);
+      const uint32_t sn = grp * rpw + rl;
+      span_of(b, (u + nwaves < units && sn < R) ? rows[sn] : grf::kNoRow, g0, g1);
     }
     __builtin_amdgcn_wave_barrier();
     float acc[M];
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[m] = 0.f;
     if (walks) {
-      // The activations of a group of 16 columns are loaded while the group before is
-      // decoded, into one of two register sets that take turns (no copies between them).
-      uint4 xa[M][2], xb[M][2];
-      auto load_x = [&](uint4 (&xs)[M][2], uint32_t t) {
+      // The activations are read eight columns (16 bytes per row) at a time, each load issued
+      // while the eight symbols before it are decoded: two register sets, one for the first and
+      // one for the second half of a group of 16, so nothing is copied between them.
+      uint4 xa[M], xb[M];
+      auto load_x = [&](uint4 (&xs)[M], uint32_t t) {
 #pragma unroll
-        for (int m = 0; m < M; ++m) {
-          const uint4 *xm = reinterpret_cast<const uint4 *>(x + (size_t)m * ldx + col0 + t);
-          xs[m][0] = xm[0];
-          xs[m][1] = xm[1];
-        }
+        for (int m = 0; m < M; ++m) xs[m] = *reinterpret_cast<const uint4 *>(x + (size_t)m * ldx + col0 + t);
       };
-      auto group = [&](uint32_t t, const uint4 (&xs)[M][2], uint4 (&xnext)[M][2]) {
-        load_x(xnext, min(t + 16, S - 16));  // the last group loads itself again rather than branch around the loads
-        uint32_t pair[8];
-        w.decode16(t, S, q, pair);
+      auto contract = [&](const uint32_t (&pair)[4], const uint4 (&xs)[M]) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-          acc[m] = dot2_bf16(pair[0], xs[m][0].x, acc[m]);
-          acc[m] = dot2_bf16(pair[1], xs[m][0].y, acc[m]);
-          acc[m] = dot2_bf16(pair[2], xs[m][0].z, acc[m]);
-          acc[m] = dot2_bf16(pair[3], xs[m][0].w, acc[m]);
-          acc[m] = dot2_bf16(pair[4], xs[m][1].x, acc[m]);
-          acc[m] = dot2_bf16(pair[5], xs[m][1].y, acc[m]);
-          acc[m] = dot2_bf16(pair[6], xs[m][1].z, acc[m]);
-          acc[m] = dot2_bf16(pair[7], xs[m][1].w, acc[m]);
+          acc[m] = dot2_bf16(pair[0], xs[m].x, acc[m]);
+          acc[m] = dot2_bf16(pair[1], xs[m].y, acc[m]);
+          acc[m] = dot2_bf16(pair[2], xs[m].z, acc[m]);
+          acc[m] = dot2_bf16(pair[3], xs[m].w, acc[m]);
         }
       };
       load_x(xa, 0);
-      for (uint32_t t = 0; t < S; t += 32) {
-        group(t, xa, xb);
-        if (t + 16 < S) group(t + 16, xb, xa);
+      for (uint32_t t = 0; t < S; t += 16) {
+        uint32_t pair[4];
+        load_x(xb, t + 8);
+        w.begin16(t, S);
+        w.template half<0>(q, pair);
+        contract(pair, xa);
+        load_x(xa, min(t + 16, S - 8));  // the last group loads a half again rather than branch around the load
+        w.template half<1>(q, pair);
+        contract(pair, xb);
       }
       if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
     }
     // The unit's sum of a row: its P segment partials (0 for lanes without a segment) added
-    // pairwise, neighbours first -- lane distances 1, 2, 4, ... -- in every lane at once.
+    // pairwise, neighbours first -- lane distances 1, 2, 4, ...
     {
       // (the lane's coordinates are worked out again rather than kept in registers over the walk)
       uint32_t ln = __lane_id();
 #if defined(__HIP_DEVICE_COMPILE__)
       asm volatile("" : "+v"(ln));
 #endif
-      const uint32_t p2 = ln % P, slot2 = (u / g.n_slabs) * rpw + ln / P;
+      const uint32_t p2 = ln & (P - 1), rl2 = ln >> logp;
+      const uint32_t slot2 = slot_base + rl2;
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        float sum = acc[m];
-        for (uint32_t d = 1; d < P; d <<= 1) sum += __shfl_xor(sum, d, 64);
-        if (p2 == 0 && slot2 < R) sub[(slot2 * g.n_slabs + u % g.n_slabs) * M + m] = sum;
+        const float sum = group_sum_to_first_lane(acc[m], logp);
+        if (p2 == 0 && slot2 < R) sub[(slot2 * g.n_slabs + slab) * M + m] = sum;
       }
     }
   }
