@@ -342,31 +342,31 @@ __device__ __forceinline__ uint32_t fused_stage_piece(uint8_t *lds, uint32_t pie
 
 // The same copy made by one wave for itself (wave-unit tiling), without vector registers: the
 // loads write the LDS directly.  Such a load puts the 16 bytes of lane l at (base + 16 * l) of
-// a wave-uniform base, whatever address the lane read, so one instruction can fill 256
-// contiguous bytes of one row's piece from that row's 16-lane group (P lanes in general): the
-// rows take turns, each with the base that makes its lanes land on its own piece.  Round i
-// moves chunks [i * P, (i + 1) * P) of every row.  The bytes are in the LDS when the wave's
-// vector-memory counter says so; lanes of the same wave read them afterwards.
+// a wave-uniform base, whatever address the lane read, so one instruction moves up to 1 KiB of
+// consecutive bytes: the rows of the unit take turns, all 64 lanes copying one row's piece
+// (its byte range, which the row's own lanes hold, is handed to the others through scalar
+// registers).  A piece longer than 1 KiB takes further rounds.  The bytes are in the LDS when
+// the wave's vector-memory counter says so; lanes of the same wave read them afterwards.
+// (Sixteen lanes per instruction, each row served by its own lanes, took four times as many
+// instructions, and a wave spent 2 us per unit issuing them.)
 __device__ __forceinline__ uint32_t fused_stage_piece_dma(uint8_t *lds, uint32_t region0, uint32_t cap,
-                                                          const grf_bctx_fused &f, uint32_t g0, uint32_t g1, uint32_t rl,
-                                                          uint32_t p, uint32_t logp, uint32_t rows_per_wave) {
+                                                          const grf_bctx_fused &f, uint32_t g0, uint32_t g1, uint32_t lane,
+                                                          uint32_t logp, uint32_t rows_per_wave) {
   typedef __attribute__((address_space(3))) void lds_void;
-  const uint32_t P = 1u << logp;
-  const uint32_t a0 = g0 & ~15u;
-  // rounds the longest piece of the wave needs (uniform: every lane takes part in the ballots)
-  uint32_t longest = g1 > a0 ? g1 - a0 : 0;
-  for (uint32_t d = P; d < 64; d <<= 1) longest = max(longest, (uint32_t)__shfl_xor((int)longest, (int)d, 64));
-  const uint32_t rounds = (longest + P * 16 - 1) >> (logp + 4);
-  for (uint32_t i = 0; i < rounds; ++i) {
-    const uint32_t o = a0 + (i * P + p) * 16;
-    for (uint32_t r = 0; r < rows_per_wave; ++r) {  // uniform
-      // lane l = r * P + p of row r must land on region(r) + (i * P + p) * 16
-      const uint32_t base = region0 + r * cap + i * P * 16 - r * P * 16;
-      if (rl == r && o < g1)
-        __builtin_amdgcn_global_load_lds(f.main_bytes + o, (lds_void *)(lds + base), 16, 0, 0);
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t rounds = (cap + 1023) >> 10;  // uniform: a figure of the tiling
+  for (uint32_t r = 0; r < rows_per_wave; ++r) {  // uniform
+    const uint32_t s0 = __builtin_amdgcn_readlane(g0, r << logp) & ~15u, s1 = __builtin_amdgcn_readlane(g1, r << logp);
+    for (uint32_t i = 0; i < rounds; ++i) {
+      const uint32_t o = s0 + (i * 64 + lane) * 16;
+      if (o < s1)
+        __builtin_amdgcn_global_load_lds(f.main_bytes + o, (lds_void *)(lds + (region0 + r * cap + i * 1024)), 16, 0, 0);
     }
   }
-  return a0;
+#else
+  (void)lds, (void)region0, (void)cap, (void)f, (void)g1, (void)lane, (void)logp, (void)rows_per_wave;
+#endif
+  return g0 & ~15u;
 }
 
 // BF16 word in bits 0..15 (bits above are unspecified): symbol bits | mantissa low 5 bits

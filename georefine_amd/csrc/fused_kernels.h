@@ -343,12 +343,11 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     // Waves with more units still to do go first.  Left alone the arbiter prefers the older
     // of the two workgroups that share a compute unit, which then finishes long before the
     // other and leaves it the unit at half occupancy.
-    switch (min(3u, left + later_half)) {  // + the later-started half
-      case 0: __builtin_amdgcn_s_setprio(0); break;
-      case 1: __builtin_amdgcn_s_setprio(1); break;
-      case 2: __builtin_amdgcn_s_setprio(2); break;
-      default: __builtin_amdgcn_s_setprio(3); break;
-    }
+    // Between walks a wave has a hundred-odd instructions to issue (row sums, addresses, the
+    // loads of the next unit), each waiting on the one before; at the walking waves' priority
+    // it got a turn so rarely that this took 3 us per unit.  It goes first, and back to its
+    // walking priority when the walk starts.
+    __builtin_amdgcn_s_setprio(3);
 #endif
     const uint32_t slot = grp * rpw + rl;
     const uint32_t first_seg = b << logp;
@@ -356,12 +355,14 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     if (u != wave) row = slot < R ? rows[slot] : grf::kNoRow;  // (read again: cheaper than a register over the walk)
     const bool walks = row != grf::kNoRow && p < nseg;
     const uint32_t col0 = (first_seg + p) * S;
+    // The copy of the pieces goes first: its byte ranges arrived during the walk before, while
+    // a wait for them placed after this unit's other loads would wait for those as well.
+    const uint32_t a0 = grf::fused_stage_piece_dma(lds, L.stream + wave * rpw * g.piece_cap, g.piece_cap, f, g0, g1, lane, logp, rpw);
     Walk w;
     {  // every lane loads (see span_of); lanes that do not walk read segment 0's entries
       const uint32_t seg = walks ? row * f.segs_per_row + first_seg + p : 0;
       w.prefetch(f, seg, walks ? (uint64_t)row * K + col0 : 0, walks ? col0 : 0);
     }
-    const uint32_t a0 = grf::fused_stage_piece_dma(lds, L.stream + wave * rpw * g.piece_cap, g.piece_cap, f, g0, g1, rl, p, logp, rpw);
     if (walks) w.start(piece_off, a0);
     const uint32_t slot_base = grp * rpw, slab = b;  // this unit's, kept while the counters move on
     {  // the next unit's byte range, on its way during this unit's walk
@@ -370,9 +371,18 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
       span_of(b, (u + nwaves < units && sn < R) ? rows[sn] : grf::kNoRow, g0, g1);
     }
     __builtin_amdgcn_wave_barrier();
+#if defined(__HIP_DEVICE_COMPILE__)
+    switch (min(3u, left + later_half)) {  // + the later-started half
+      case 0: __builtin_amdgcn_s_setprio(0); break;
+      case 1: __builtin_amdgcn_s_setprio(1); break;
+      case 2: __builtin_amdgcn_s_setprio(2); break;
+      default: __builtin_amdgcn_s_setprio(3); break;
+    }
+#endif
     float acc[M];
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[m] = 0.f;
+    uint32_t warm = 0;
     if (walks) {
       // The activations are read eight columns (16 bytes per row) at a time, each load issued
       // while the eight symbols before it are decoded: two register sets, one for the first and
@@ -401,9 +411,21 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
         load_x(xa, min(t + 16, S - 8));  // the last group loads a half again rather than branch around the load
         w.template half<1>(q, pair);
         contract(pair, xb);
+        if (t == 0) {
+          // The next unit's stream bytes come from HBM, and its copy to LDS can only start when
+          // this walk is over: a wave then waited some 3 us per unit for them.  One word of
+          // every 128-byte line of the next piece is read now (its range has arrived by the end
+          // of the first group), which brings the lines into the L2 for that copy to find.
+          for (uint32_t o = (g0 & ~127u) + p * 128; o < g1; o += P * 128)
+            warm ^= *reinterpret_cast<const uint32_t *>(f.main_bytes + o);
+        }
       }
       if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
     }
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" ::"v"(warm));  // (the words read ahead are wanted for their side effect only)
+    __builtin_amdgcn_s_setprio(3);
+#endif
     // The unit's sum of a row: its P segment partials (0 for lanes without a segment) added
     // pairwise, neighbours first -- lane distances 1, 2, 4, ...
     {
