@@ -387,8 +387,8 @@ struct SegmentWalkT {
   Cursor c;
   uint32_t gofs, eofs;        // byte offsets of this segment's and the next segment's checkpoints
   uint32_t end_state, end_jb;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
-  const uint32_t *rawp;
-  const uint4 *ccp;
+  const uint8_t *raw_base, *cc_base;  // the frame's residual and class arrays (uniform)
+  uint32_t raw_off, cc_off;           // byte offsets of this segment's first group in them
   uint32_t n0, n1, n2;             // !AHEAD: the next group's residual words
   uint32_t rw[AHEAD ? 12 : 1];     // AHEAD: the segment's residual words
   uint4 nc4;
@@ -402,20 +402,25 @@ struct SegmentWalkT {
     eofs = f.seg_offset[seg_ + 1];
     c.state = f.seg_state[seg_];
     end_state = f.seg_state[seg_ + 1];
-    rawp = reinterpret_cast<const uint32_t *>(f.raw6 + elem0 / 4 * 3);
-    ccp = reinterpret_cast<const uint4 *>(f.col_class + col0);
+    // a uniform base plus a 32-bit lane offset: the loads then take their address from a scalar
+    // pair and one vector register, and no 64-bit address is worked out per group
+    raw_base = f.raw6;
+    cc_base = f.col_class;
+    raw_off = (uint32_t)(elem0 / 4 * 3);
+    cc_off = col0;
     if constexpr (AHEAD) {
-      const uint4 *r4 = reinterpret_cast<const uint4 *>(rawp);  // 48-byte groups: 16-byte aligned
+      const uint4 *r4 = reinterpret_cast<const uint4 *>(raw_base + raw_off);  // 48-byte groups: 16-byte aligned
       const uint4 a = r4[0], b = r4[1], d = r4[2];
       rw[0] = a.x, rw[1] = a.y, rw[2] = a.z, rw[3] = a.w;
       rw[4] = b.x, rw[5] = b.y, rw[6] = b.z, rw[7] = b.w;
       rw[8] = d.x, rw[9] = d.y, rw[10] = d.z, rw[11] = d.w;
     } else {
-      n0 = rawp[0];
-      n1 = rawp[1];
-      n2 = rawp[2];
+      const uint32_t *r = reinterpret_cast<const uint32_t *>(raw_base + raw_off);
+      n0 = r[0];
+      n1 = r[1];
+      n2 = r[2];
     }
-    nc4 = ccp[0];
+    nc4 = *reinterpret_cast<const uint4 *>(cc_base + cc_off);
   }
   // the row piece was staged at piece_off from global offset a0
   __device__ __forceinline__ void start(uint32_t piece_off, uint32_t a0) {
@@ -432,14 +437,14 @@ struct SegmentWalkT {
     cw[3] = nc4.w;
     // the last group loads itself again rather than branch around the loads
     const uint32_t next = min(t / 16 + 1, S / 16 - 1);
-    nc4 = ccp[next];
+    nc4 = *reinterpret_cast<const uint4 *>(cc_base + (cc_off + next * 16));
     if constexpr (AHEAD) {  // the words of the groups still to come move down one group
       rr.set(rw[0], rw[1], rw[2]);
 #pragma unroll
       for (int i = 0; i < 9; ++i) rw[i] = rw[i + 3];
     } else {
       rr.set(n0, n1, n2);
-      const uint32_t *nx = rawp + next * 3;
+      const uint32_t *nx = reinterpret_cast<const uint32_t *>(raw_base + (raw_off + next * 12));
       n0 = nx[0];
       n1 = nx[1];
       n2 = nx[2];

@@ -388,9 +388,10 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
       // while the eight symbols before it are decoded: two register sets, one for the first and
       // one for the second half of a group of 16, so nothing is copied between them.
       uint4 xa[M], xb[M];
-      auto load_x = [&](uint4 (&xs)[M], uint32_t t) {
+      auto load_x = [&](uint4 (&xs)[M], uint32_t t) {  // (uniform base, 32-bit lane offset in bytes)
 #pragma unroll
-        for (int m = 0; m < M; ++m) xs[m] = *reinterpret_cast<const uint4 *>(x + (size_t)m * ldx + col0 + t);
+        for (int m = 0; m < M; ++m)
+          xs[m] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint8_t *>(x) + ((uint32_t)m * ldx + col0 + t) * 2u);
       };
       auto contract = [&](const uint32_t (&pair)[4], const uint4 (&xs)[M]) {
 #pragma unroll
@@ -485,6 +486,8 @@ int launch_wave(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16
 constexpr uint32_t kWaveRowsPerPass = 2;
 
 inline int check_wave_operands(const char *who, const grf_bctx_fused &f, const uint16_t *x, uint32_t ldx) {
+  if (ldx > (1u << 29))  // the kernel addresses x with 32-bit byte offsets
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": leading dimension of x too large");
   if ((ldx & 7) || ((uintptr_t)x & 15))
     return grf::set_error(GRF_BAD_ARGUMENT,
                           std::string(who) + ": wave units read x in 16-byte vectors (aligned, ldx a multiple of 8)");
