@@ -126,10 +126,12 @@ def gemm_shape(p, r):
 
 
 def lds_bytes_gemm(nc, lognb, tabn, p, r, piece_cap):
+    """Tables, then sixteen row pieces of four segments per wave; later every wave's partial sums."""
     a16 = lambda v: (v + 15) // 16 * 16
+    waves = gemm_shape(p, r)[2] // 64
     total = a16(nc * (a16((tabn + 1) * 8) + (1 << lognb)))
-    total = a16(total + r * piece_cap)
-    return max(total, gemm_shape(p, r)[2] // 64 * GEMM_MAX_TILES * 1024)  # later: every wave's partial sums
+    total = a16(total + waves * 16 * piece_cap)
+    return max(total, waves * GEMM_MAX_TILES * 1024)
 
 
 WINDOW = 8  # bytes the refill reads from the 4-byte aligned cursor on
@@ -146,6 +148,17 @@ def piece_capacity(offsets, rows, spr, p):
         g0 = off[:, b]
         g1 = off[:, b + p] if b + p < spr else end_of_row
         longest = max(longest, int((g1 - (g0 & ~15)).max()))
+    return (longest + WINDOW + 15) // 16 * 16
+
+
+def quad_piece_capacity(offsets, rows, spr):
+    """LDS bytes of a GEMM wave's row piece: four consecutive segments of a row from any first
+    segment (fewer at the row's end), from the 16-byte aligned start, plus the refill's window."""
+    off = offsets[:-1].reshape(rows, spr).astype(np.int64)
+    end_of_row = np.concatenate((off[1:, 0], [int(offsets[-1])]))
+    ends = np.concatenate((off, end_of_row[:, None]), axis=1)  # ends[:, s] = start of segment s, [:, spr] = row end
+    last = np.minimum(np.arange(spr) + 4, spr)
+    longest = int((ends[:, last] - (off & ~15)).max())
     return (longest + WINDOW + 15) // 16 * 16
 
 
@@ -371,6 +384,12 @@ class FramePlan:
         return dict(rows=self.rows, cols=self.cols, nr=self.nr, nc=self.nc, seg_len=self.seg_len,
                     segs_per_row=self.spr, shift=self.shift, lognb=self.lognb, tabn=self.tabn)
 
+    def quad_cap(self):
+        """Capacity of the row pieces of the GEMM's waves (four segments)."""
+        if "quad" not in self._caps:
+            self._caps["quad"] = quad_piece_capacity(self.seg_offset, self.rows, self.spr)
+        return self._caps["quad"]
+
     def _cap(self, p):
         if p not in self._caps:
             self._caps[p] = piece_capacity(self.seg_offset, self.rows, self.spr, p)
@@ -414,14 +433,14 @@ class FramePlan:
         """The one tiling every fused GEMM launch uses, whatever its row count: the order in
         which an output element accumulates follows the tiling, so it must not change with M."""
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_gemm_tiling(
-            self.spr, self.class_rows, self._cap,
+            self.spr, self.class_rows, lambda lanes: self.quad_cap(),
             lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, p_, r_, cap_),
             seg_len=self.seg_len, table_bytes=self.table_bytes())
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                 n_tiles=n_tiles, piece_cap=cap, scheme=SCHEME_SLABS), lds=lds)
+                                 n_tiles=n_tiles, piece_cap=cap, scheme=SCHEME_WAVES), lds=lds)
 
 
 def plan_group(plans, m=None, gemm=False, waves=False):
@@ -437,8 +456,10 @@ def plan_group(plans, m=None, gemm=False, waves=False):
     table = max(pl.table_bytes() for pl in plans)
     scheme = SCHEME_SLABS
     if gemm:
+        scheme = SCHEME_WAVES
         lds_fn = lambda p_, r_, cap_: max(lds_bytes_gemm(pl.nc, pl.lognb, pl.tabn, p_, r_, cap_) for pl in plans)
-        threads, p, r, n_slabs, _, cap, lds = choose_gemm_tiling(first.spr, class_rows, cap_fn, lds_fn,
+        quad_cap = max(pl.quad_cap() for pl in plans)
+        threads, p, r, n_slabs, _, cap, lds = choose_gemm_tiling(first.spr, class_rows, lambda lanes: quad_cap, lds_fn,
                                                                  seg_len=first.seg_len, table_bytes=table)
     elif waves:
         scheme = SCHEME_WAVES

@@ -53,7 +53,7 @@ int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
                   size_t workspace_bytes, int32_t *error, void *hip_stream) {
   if (!frame || !tiling || !y || !error)  // x may be null: rows packed by grf_pack_activations
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemm: null argument");
-  if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemm")) return rc;
+  if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemm", grf::kGemmTiling)) return rc;
   return grf::launch_gemm<grf::SegmentWalk>("grf_bctx_gemm", *frame, *tiling, x, ldx, m_rows, y, ldy, bias, workspace,
                                             workspace_bytes, error, (hipStream_t)hip_stream);
 }
@@ -70,7 +70,7 @@ int grf_bctx_gemm_noalloc(const grf_bctx_fused *frame, const grf_fused_tiling *t
                           "grf_bctx_gemm_noalloc: the packed activations of one launch exceed the 8 MiB scratch "
                           "(grf_gemm_workspace_bytes(cols, m_rows) > grf_gemm_noalloc_limit_bytes()); use grf_bctx_gemm "
                           "with a workspace");
-  if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemm_noalloc")) return rc;
+  if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemm_noalloc", grf::kGemmTiling)) return rc;
   void *ptr = nullptr;
   if (int rc = scratch_address(&ptr)) return rc;
   // every launch writes all it reads of the scratch (its rows, zero rows up to the tile, the

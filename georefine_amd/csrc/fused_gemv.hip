@@ -3,7 +3,7 @@
 #include "fused_kernels.h"
 
 namespace grf {
-int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who, bool wave_units) {
+int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who, TilingUse use) {
   auto bad = [&](const char *why) { return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": " + why); };
   if (!f.main_bytes || !f.raw6 || !f.seg_state || !f.seg_offset || !g.tile_rows || !g.tile_class || !f.lut ||
       !f.tab || !f.col_class)
@@ -12,8 +12,11 @@ int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const 
   if (f.seg_len == 0 || f.seg_len % 16 || (uint64_t)f.seg_len * f.segs_per_row != f.cols)
     return bad("segment length must be a multiple of 16 that divides the row length");
   if (!g.threads || g.threads % 64 || g.threads > (uint32_t)grf::kFusedMaxThreads) return bad("thread count");
-  if (g.scheme == GRF_TILE_WAVES) {
-    if (!wave_units) return bad("this entry point takes slab tilings only");
+  if (use == kGemmTiling) {  // waves of 16 rows x 4 segments with their own stream pieces
+    if (g.scheme != GRF_TILE_WAVES) return bad("the GEMM takes a wave tiling (piece_cap for pieces of four segments)");
+    if (!g.lanes_per_row || !g.rows_per_tile) return bad("empty tile");
+  } else if (g.scheme == GRF_TILE_WAVES) {
+    if (use != kGemvTiling) return bad("this entry point takes slab tilings only");
     const uint32_t lanes = g.lanes_per_row;
     if (lanes < 4 || lanes > 64 || (lanes & (lanes - 1))) return bad("a wave unit has 4, 8, 16, 32 or 64 lanes per row");
     if (!g.rows_per_tile) return bad("empty tile");
@@ -46,7 +49,7 @@ int grf_bctx_gemv(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
                   void *hip_stream) {
   if (!frame || !tiling || !x || !y || !error)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemv: null argument");
-  if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemv", true)) return rc;
+  if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemv", grf::kGemvTiling)) return rc;
   return grf::launch_gemv<grf::SegmentWalk>("grf_bctx_gemv", *frame, *tiling, x, ldx, m_rows, y, ldy, bias, error,
                                             (hipStream_t)hip_stream);
 }

@@ -35,7 +35,8 @@
 namespace grf {
 int set_error(int code, const std::string &what);                                          // decode_general.hip
 // fused_gemv.hip; wave_units: the entry point takes GRF_TILE_WAVES tilings
-int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who, bool wave_units = false);
+enum TilingUse { kSlabTiling, kGemvTiling, kGemmTiling };  // what an entry point does with the tiling it is given
+int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who, TilingUse use = kSlabTiling);
 
 // A kernel may ask for more than 64 KiB of dynamic LDS only after its limit has been raised;
 // done once per kernel and device (not per launch: it is a driver call, and a launch that
@@ -635,16 +636,18 @@ struct GemmShape {
   }
 };
 
-// Tables and stream pieces as in the GEMV kernel; the same memory later holds the partial
-// sums of every wave (1 KiB per wave and activation tile).
+// Tables, then for every wave the pieces of its sixteen rows (piece_cap: the capacity of a
+// piece of four segments); the same memory later holds the partial sums of every wave (1 KiB
+// per wave and activation tile).
 struct GemmLdsLayout {
   uint32_t blocks, block_pitch, stream, total;
   __host__ __device__ GemmLdsLayout(const grf_bctx_fused &f, const grf_fused_tiling &g) {
     blocks = 0;
     block_pitch = grf::fused_table_bytes(f) + (1u << f.lognb);
     stream = grf::align_up(f.nc * block_pitch, 16);
-    total = grf::align_up(stream + g.rows_per_tile * g.piece_cap, 16);
-    const uint32_t sums = GemmShape(g).threads / 64 * kSumTiles * 1024;
+    const uint32_t waves = GemmShape(g).threads / 64;
+    total = grf::align_up(stream + waves * 16 * g.piece_cap, 16);
+    const uint32_t sums = waves * kSumTiles * 1024;
     if (total < sums) total = sums;
   }
 };
@@ -713,44 +716,72 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
   constexpr uint32_t m_pad = MT * 16;
 
-  const uint32_t wave = tid / 64, lane = tid % 64;
+  const uint32_t lane = tid % 64;
+#if defined(__HIP_DEVICE_COMPILE__)
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid / 64);  // (a scalar: the loop below branches on it)
+#else
+  const uint32_t wave = tid / 64;
+#endif
   const uint32_t rb = wave % shape.row_blocks, quad = wave / shape.row_blocks;
-  const uint32_t r = rb * 16 + lane % 16, p = quad * 4 + lane / 16;
-  uint32_t row = (r < R && p < P) ? g.tile_rows[tile * R + r] : grf::kNoRow;
+  const uint32_t r = rb * 16 + lane % 16, p4 = lane / 16;
+  uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
   if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
-  grf::PieceSpan span{0, 0};  // started before the table copy so that the latencies overlap
-  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
+
+  // A wave keeps its sixteen rows and its quad of lane-segments for the whole launch and goes
+  // through the slabs on its own: in slab b it walks segments b * P + 4 * quad .. + 3 of every
+  // row.  It copies the rows' pieces of those four segments to its own part of the LDS (the
+  // loads write the LDS directly, one row per instruction), so the waves of a workgroup share
+  // the tables and nothing else until their partial sums meet at the end.
+  const uint32_t region = L.stream + wave * 16 * g.piece_cap;
+  const uint32_t piece_off = region + (lane % 16) * g.piece_cap;
+  // byte range of the lane's row piece in a slab; lanes without a row, and slabs past the row's
+  // end, read the matrix's first entry and get an empty range (no load sits in a branch)
+  auto span_of = [&](uint32_t b, uint32_t &g0, uint32_t &g1) {
+    const uint32_t first = b * P + quad * 4;
+    const bool any = row != grf::kNoRow && first < f.segs_per_row && quad * 4 < P;
+    const uint32_t base = any ? row * f.segs_per_row + first : 0;
+    g0 = f.seg_offset[base];
+    g1 = f.seg_offset[base + (any ? min(4u, min(P - quad * 4, f.segs_per_row - first)) : 0)];
+  };
+  uint32_t g0, g1;
+  span_of(0, g0, g1);  // started before the table copy so that the latencies overlap
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
 
   float4v acc[MT];
 #pragma unroll
   for (int j = 0; j < MT; ++j) acc[j] = (float4v){0.f, 0.f, 0.f, 0.f};
   uint32_t bad = 0;
+  __syncthreads();  // the tables are in place
 
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
-    if (b) __syncthreads();  // everyone is done with the previous slab's stream bytes
-    const uint32_t first_seg = b * P;
-    const uint32_t nseg = min(P, f.segs_per_row - first_seg);
-    const uint32_t piece_off = L.stream + r * g.piece_cap;
-    const bool active = row != grf::kNoRow && p < nseg;
-    const uint32_t seg_base = row != grf::kNoRow ? row * f.segs_per_row + first_seg : 0;
-    const uint32_t col0 = (first_seg + p) * S;
+    const uint32_t first_seg = b * P + quad * 4;
+    if (first_seg >= f.segs_per_row || quad * 4 >= P) break;  // uniform: this wave's quad has no segment from here on
+    const uint32_t nseg = min(4u, min(P - quad * 4, f.segs_per_row - first_seg));
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_s_setprio(3);  // between walks a wave's few instructions go first
+#endif
+    const bool active = row != grf::kNoRow && p4 < nseg;
+    const uint32_t col0 = (first_seg + p4) * S;
+    // the pieces first: their ranges arrived during the walk before
+    const uint32_t a0 = grf::fused_stage_piece_dma(lds, region, g.piece_cap, f, g0, g1, lane, 0, 16);
     Walk w;
-    uint32_t a0 = 0;
-    if (active) w.prefetch(f, seg_base + p, (uint64_t)row * K + col0, col0);
-    if (row != grf::kNoRow) {
-      a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
-      if (b + 1 < g.n_slabs)  // the next slab's byte range, while this one is walked
-        span.fetch(f, seg_base + P, min(P, f.segs_per_row - first_seg - P));
+    {
+      const uint32_t seg = active ? row * f.segs_per_row + first_seg + p4 : 0;
+      w.prefetch(f, seg, active ? (uint64_t)row * K + col0 : 0, active ? col0 : 0);
     }
-    __syncthreads();
+    if (active) w.start(piece_off, a0);  // (a0: of the lane's own row, which its four lanes share)
+    span_of(b + 1, g0, g1);  // the next slab's byte range, on its way during this walk
+    __builtin_amdgcn_wave_barrier();
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (b + 1 < g.n_slabs) __builtin_amdgcn_s_setprio(1);
+    else __builtin_amdgcn_s_setprio(0);
+#endif
     if (__ballot(active) == 0) continue;  // nothing to walk in this wave (the branch is per wave)
-    if (active) w.start(piece_off, a0);
     // A lane's k-slots are real columns when its segment exists, whether or not its own
     // row does; other lanes feed zeros (their weights are zero too, but 0 * NaN is not):
     // they read the chunk of zeros that ends the packed copy and never move on.  The load
     // after a segment's last half group reads the chunk that follows it, at most that one.
-    const bool feeds = p < nseg;
+    const bool feeds = p4 < nseg;
     const uint32_t x_step = feeds ? m_pad : 0;
     const uint4 *xl = xp + (size_t)(feeds ? col0 / 8 : K / 8) * m_pad + lane % 16;
     uint4 xa[MT];
@@ -771,6 +802,9 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     }
     if (active && !w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
   }
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_s_setprio(0);
+#endif
 
   // partial sums of every wave -> LDS, then each output element adds its quads in order;
   // four activation tiles at a time, which is what the LDS allocation is sized for
@@ -935,7 +969,7 @@ inline int build_group(const char *who, const GroupSpec &spec, bool gemm, FusedG
     if (!spec.frames[i] || !spec.tilings[i] || !spec.y[i]) return bad("null member");
     const grf_bctx_fused &f = *spec.frames[i];
     const grf_fused_tiling &g = *spec.tilings[i];
-    if (int rc = grf::check_fused_frame(f, g, who, !gemm)) return rc;
+    if (int rc = grf::check_fused_frame(f, g, who, gemm ? kGemmTiling : kGemvTiling)) return rc;
     if (f.cols != spec.frames[0]->cols) return bad("members must have one width");
     if (g.threads != spec.tilings[0]->threads) return bad("member tilings must share one thread count");
     if (g.scheme != spec.tilings[0]->scheme) return bad("member tilings must share one scheme");

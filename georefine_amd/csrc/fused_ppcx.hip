@@ -177,7 +177,7 @@ struct PpcxWalk {
 // The PPCX frame in the walker's frame structure: raw6 = packed 5-bit residuals,
 // col_class = the bins plane, nr = labels, nc = 16 bins.
 int walker_frame(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins, const char *who,
-                 grf_bctx_fused &f) {
+                 grf_bctx_fused &f, grf::TilingUse use = grf::kSlabTiling) {
   if (!frame || !tiling || !bins) return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": null argument");
   f = grf_bctx_fused{};
   f.main_bytes = frame->main_bytes;
@@ -197,7 +197,7 @@ int walker_frame(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, co
   f.shift = frame->shift;
   f.lognb = frame->lognb;
   f.tabn = frame->tabn;
-  if (int rc = grf::check_fused_frame(f, *tiling, who)) return rc;
+  if (int rc = grf::check_fused_frame(f, *tiling, who, use)) return rc;
   if (f.seg_len % 32)  // a segment's residual bytes must start on a dword
     return grf::set_error(GRF_UNSUPPORTED, std::string(who) + ": segment length must be a multiple of 32");
   return GRF_OK;
@@ -249,7 +249,7 @@ int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, c
                   size_t workspace_bytes, int32_t *error, void *hip_stream) {
   if (!y || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemm: null argument");  // x may be null: packed rows
   grf_bctx_fused f;
-  if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_gemm", f)) return rc;
+  if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_gemm", f, grf::kGemmTiling)) return rc;
   return grf::launch_gemm<PpcxWalk>("grf_ppcx_gemm", f, *tiling, x, ldx, m_rows, y, ldy, bias, workspace,
                                     workspace_bytes, error, (hipStream_t)hip_stream);
 }

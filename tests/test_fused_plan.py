@@ -71,7 +71,14 @@ def test_tilings_cover_each_row_once_with_one_class_per_tile(shape):
             members = tile[tile != 0xFFFFFFFF]
             assert members.size and np.all(ix["rows"][members] == cls)
         assert s["threads"] % 64 == 0 and s["threads"] <= 1024
-        if s["scheme"] == _fused.SCHEME_WAVES:  # a wave walks 64 / P rows of P segments at a time
+        piece = s["lanes_per_row"]  # segments of one row piece
+        if t is tilings[-1]:  # the GEMM: waves of 16 rows x 4 segments, each with its own pieces
+            assert s["scheme"] == _fused.SCHEME_WAVES
+            assert s["threads"] == 64 * -(-s["rows_per_tile"] // 16) * -(-s["lanes_per_row"] // 4)
+            assert t["lds"] == _fused.lds_bytes_gemm(plan.nc, plan.lognb, plan.tabn, s["lanes_per_row"],
+                                                     s["rows_per_tile"], s["piece_cap"])
+            piece = 4
+        elif s["scheme"] == _fused.SCHEME_WAVES:  # a wave walks 64 / P rows of P segments at a time
             assert s["lanes_per_row"] in (4, 8, 16, 32, 64) and 1 <= s["rows_per_tile"]
             assert t is tilings[3] and t["lds"] == _fused.lds_bytes_waves(
                 plan.nc, plan.lognb, plan.tabn, 2, s["threads"], s["lanes_per_row"], s["rows_per_tile"], s["n_slabs"],
@@ -80,11 +87,13 @@ def test_tilings_cover_each_row_once_with_one_class_per_tile(shape):
             assert s["lanes_per_row"] * s["rows_per_tile"] <= s["threads"]
         assert s["n_slabs"] == -(-plan.spr // s["lanes_per_row"])
         assert t["lds"] <= _fused.MAX_LDS
-        # a row piece of any slab fits its LDS slot together with the window the refill reads
+        # a row piece fits its LDS slot together with the window the refill reads (the GEMM's
+        # pieces start at any segment: a slab's first segment need not be a multiple of four)
         off = plan.seg_offset.astype(np.int64)
-        for b in range(s["n_slabs"]):
-            first = np.arange(shape[0]) * plan.spr + b * s["lanes_per_row"]
-            last = first + min(s["lanes_per_row"], plan.spr - b * s["lanes_per_row"])
+        starts = range(plan.spr) if t is tilings[-1] else range(0, plan.spr, piece)
+        for b in starts:
+            first = np.arange(shape[0]) * plan.spr + b
+            last = first + min(piece, plan.spr - b)
             assert np.max(off[last] - (off[first] & ~15)) + 8 <= s["piece_cap"]
     g = tilings[-1]["scalars"]
     waves, blocks = g["threads"] // 64, -(-g["rows_per_tile"] // 16)
@@ -200,7 +209,7 @@ def test_group_plans_share_one_tile_shape_and_keep_every_member_complete():
         frames.append(ix)
     for kwargs in (dict(m=1), dict(m=8), dict(m=2, waves=True), dict(gemm=True)):
         tilings = _fused.plan_group(plans, **kwargs)
-        assert {t["scalars"]["scheme"] for t in tilings} == {int(bool(kwargs.get("waves")))}
+        assert {t["scalars"]["scheme"] for t in tilings} == {int(bool(kwargs.get("waves") or kwargs.get("gemm")))}
         shapes = {(t["scalars"]["threads"], t["scalars"]["lanes_per_row"], t["scalars"]["rows_per_tile"],
                    t["scalars"]["n_slabs"], t["scalars"]["piece_cap"]) for t in tilings}
         assert len(shapes) == 1 and len(tilings) == 3
