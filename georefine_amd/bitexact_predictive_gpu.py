@@ -245,10 +245,12 @@ class HipPredictiveTensor:
         self.fused_plan = dict(sc, **store[3])
 
     def _tiling_for(self, key):
-        """Device copy of a tiling: key 0 = store sink, 1/2/4/8 = GEMV row buckets, "gemm"."""
+        """Device copy of a tiling: key 0 = store sink, "waves" = the GEMV (wave units, one tiling
+        for every row count), 1/2/4/8 = GEMV row buckets of the slab kernels, "gemm"."""
         import torch
         if key not in self._tilings:
-            host = self._plan.gemm_tiling() if key == "gemm" else self._plan.tiling(key)
+            host = (self._plan.gemm_tiling() if key == "gemm" else
+                    self._plan.tiling(_fused.WAVE_ROWS_PER_PASS, waves=True) if key == "waves" else self._plan.tiling(key))
             rows = torch.from_numpy(host["tile_rows"].view(np.int32)).to(self.device)
             classes = torch.from_numpy(host["tile_class"]).to(self.device)
             g = _hip_abi.GrfFusedTiling()
@@ -328,9 +330,9 @@ class HipPredictiveTensor:
             x2 = x.reshape(-1, x.shape[-1]).to(self.device)
             if x2.shape[-1] != self.shape[1]:
                 raise ValueError("activation width does not match the weight")
-            align = 4 if use_gemm else 2  # elements: the GEMM reads 8 bytes at a time, the GEMV 4
+            align = 4 if use_gemm else 8  # elements: the GEMM reads 8 bytes at a time, the GEMV 16
             if x2.stride(-1) != 1 or x2.stride(0) % align or x2.data_ptr() % (2 * align):
-                x2 = x2.contiguous()
+                x2 = x2.clone(memory_format=torch.contiguous_format)
         if bias is not None:
             bias = bias.to(device=self.device, dtype=torch.bfloat16).contiguous()
         y = torch.empty((m, self.shape[0]), device=self.device, dtype=torch.bfloat16)
@@ -351,7 +353,7 @@ class HipPredictiveTensor:
                         extra = (space.data_ptr(), space.numel())
                     else:
                         fn = self._lib.grf_ppcx_gemv
-                        tiling = self._tiling_for(next(v for v in (1, 2, 4, 8) if v >= m))[0]
+                        tiling = self._tiling_for("waves")[0]
                     status = fn(ctypes.byref(self.fused), ctypes.byref(tiling), bins.data_ptr(),
                                 x2.data_ptr() if x2 is not None else None, x2.stride(0) if x2 is not None else 0,
                                 m, y.data_ptr(), y.stride(0),

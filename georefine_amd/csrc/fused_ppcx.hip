@@ -239,7 +239,7 @@ int grf_ppcx_gemv(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, c
                   void *hip_stream) {
   if (!x || !y || !error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemv: null argument");
   grf_bctx_fused f;
-  if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_gemv", f)) return rc;
+  if (int rc = walker_frame(frame, tiling, bins, "grf_ppcx_gemv", f, grf::kGemvTiling)) return rc;
   return grf::launch_gemv<PpcxWalk>("grf_ppcx_gemv", f, *tiling, x, ldx, m_rows, y, ldy, bias, error,
                                     (hipStream_t)hip_stream);
 }
