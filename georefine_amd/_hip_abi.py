@@ -15,7 +15,8 @@ class GrfStream(ctypes.Structure):
 class GrfBctxFrame(ctypes.Structure):
     _fields_ = [("main", GrfStream), ("residual", GrfStream), ("row_class", ctypes.c_void_p),
                 ("col_class", ctypes.c_void_p), ("rows", ctypes.c_uint32), ("cols", ctypes.c_uint32),
-                ("nc", ctypes.c_uint32), ("mode", ctypes.c_uint32), ("stride", ctypes.c_uint32)]
+                ("nc", ctypes.c_uint32), ("mode", ctypes.c_uint32), ("stride", ctypes.c_uint32),
+                ("raw6_segment", ctypes.c_uint32)]
 
 
 class GrfPpcxFrame(ctypes.Structure):
@@ -29,7 +30,8 @@ class GrfBctxFused(ctypes.Structure):
                 ("seg_offset", ctypes.c_void_p), ("lut", ctypes.c_void_p), ("tab", ctypes.c_void_p),
                 ("col_class", ctypes.c_void_p)] + [
         (name, ctypes.c_uint32) for name in (
-            "main_n_bytes", "rows", "cols", "nr", "nc", "seg_len", "segs_per_row", "shift", "lognb", "tabn")]
+            "main_n_bytes", "rows", "cols", "nr", "nc", "seg_len", "segs_per_row", "shift", "lognb", "tabn",
+            "raw_interleaved")]
 
 
 class GrfFusedTiling(ctypes.Structure):

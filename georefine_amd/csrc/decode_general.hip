@@ -25,6 +25,16 @@ int fail(int code, const std::string &what) { return grf::set_error(code, what);
 constexpr int kThreads = 256;
 
 // MODE128: residual is a second rANS stream whose context is the main symbol.
+// Index of element (row, col) among the packed 6-bit fields: the frame's own order, or, for
+// a tensor that keeps them for the fused kernels, groups of 16 ordered by their position in
+// the segment before the segment's number.
+__device__ __forceinline__ uint64_t raw6_index(const grf_bctx_frame &f, uint32_t row, uint32_t col) {
+  if (!f.raw6_segment) return (uint64_t)row * f.cols + col;
+  const uint32_t S = f.raw6_segment, spr = f.cols / S;
+  const uint64_t group = ((uint64_t)row * (S / 16) + (col % S) / 16) * spr + col / S;
+  return group * 16 + col % 16;
+}
+
 template <bool MODE128>
 __global__ __launch_bounds__(kThreads) void bctx_decode_kernel(grf_bctx_frame f, const int64_t *block_ids,
                                                                 uint32_t count, uint16_t *out, int32_t *error) {
@@ -57,7 +67,7 @@ __global__ __launch_bounds__(kThreads) void bctx_decode_kernel(grf_bctx_frame f,
       r = grf::rans_step_global(rstate, rip, f.residual.bytes, f.residual.n_bytes,
                                 f.residual.cum + (size_t)m * 65, f.residual.bucket + (size_t)m * 256, bad);
     else
-      r = grf::packed_field<6>(f.residual.bytes, f.residual.n_bytes, start + t);
+      r = grf::packed_field<6>(f.residual.bytes, f.residual.n_bytes, raw6_index(f, row, col));
     dst[t] = (uint16_t)grf::bctx_word(m, r);
     if (++col == f.cols) {
       col = 0;

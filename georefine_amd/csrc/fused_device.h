@@ -389,6 +389,7 @@ struct SegmentWalkT {
   uint32_t end_state, end_jb;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
   const uint8_t *raw_base, *cc_base;  // the frame's residual and class arrays (uniform)
   uint32_t raw_off, cc_off;           // byte offsets of this segment's first group in them
+  uint32_t raw_stride;                // bytes from a group's residuals to the next group's
   uint32_t n0, n1, n2;             // !AHEAD: the next group's residual words
   uint32_t rw[AHEAD ? 12 : 1];     // AHEAD: the segment's residual words
   uint4 nc4;
@@ -406,7 +407,13 @@ struct SegmentWalkT {
     // pair and one vector register, and no 64-bit address is worked out per group
     raw_base = f.raw6;
     cc_base = f.col_class;
-    raw_off = (uint32_t)(elem0 / 4 * 3);
+    if (f.raw_interleaved) {  // a row's groups ordered by position in the segment, then by segment
+      raw_off = (uint32_t)(((elem0 - col0) / 16 + col0 / f.seg_len) * 12);
+      raw_stride = f.segs_per_row * 12;
+    } else {
+      raw_off = (uint32_t)(elem0 / 4 * 3);
+      raw_stride = 12;
+    }
     cc_off = col0;
     if constexpr (AHEAD) {
       const uint4 *r4 = reinterpret_cast<const uint4 *>(raw_base + raw_off);  // 48-byte groups: 16-byte aligned
@@ -444,7 +451,7 @@ struct SegmentWalkT {
       for (int i = 0; i < 9; ++i) rw[i] = rw[i + 3];
     } else {
       rr.set(n0, n1, n2);
-      const uint32_t *nx = reinterpret_cast<const uint32_t *>(raw_base + (raw_off + next * 12));
+      const uint32_t *nx = reinterpret_cast<const uint32_t *>(raw_base + (raw_off + next * raw_stride));
       n0 = nx[0];
       n1 = nx[1];
       n2 = nx[2];

@@ -86,7 +86,8 @@ template <>
 struct ahead_of<grf::SegmentWalk> { using type = grf::SegmentWalkAhead; };
 constexpr uint32_t kAheadMaxRows = 4;
 // a segment's residuals are 48 bytes, read as three 16-byte vectors
-inline bool reads_ahead(const grf_bctx_fused &f) { return f.seg_len == 64 && !((uintptr_t)f.raw6 & 15); }
+// (a segment's 48 residual bytes are contiguous only in the frame's own order)
+inline bool reads_ahead(const grf_bctx_fused &f) { return f.seg_len == 64 && !f.raw_interleaved && !((uintptr_t)f.raw6 & 15); }
 
 // One workgroup's walk over tile `tile` of a frame.
 template <class Walk, int M, int SINK>

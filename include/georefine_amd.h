@@ -109,7 +109,10 @@ typedef struct grf_stream {
 
 /* A BCTX frame as the decode kernels see it (the buffers CudaContextTensor keeps,
  * GCR/bitexact_context_gpu.py:96-125). mode 0: residual.bytes is the packed 6-bit
- * stream and the other residual fields are unused; mode 128: residual is a full stream. */
+ * stream and the other residual fields are unused; mode 128: residual is a full stream.
+ * raw6_segment (mode 0): 0 when the 6-bit fields are in the frame's own order (element e at
+ * bit 6 e); S > 0 when the 12-byte groups of 16 fields are kept in the order the fused
+ * kernels read them (see grf_bctx_fused.raw_interleaved) for segments of S symbols. */
 typedef struct grf_bctx_frame {
   grf_stream main;
   grf_stream residual;
@@ -119,6 +122,7 @@ typedef struct grf_bctx_frame {
   uint32_t nc;
   uint32_t mode;
   uint32_t stride;
+  uint32_t raw6_segment;
 } grf_bctx_frame;
 
 /* Replaces the Triton launch of decode_words (GCR/bitexact_context_gpu.py:149-150,
@@ -166,6 +170,11 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  *                                            (freq & 0xFFFF)<<16 (0 stands for 65536),
  *                                            high32 = symbol<<5; unused entries: 0
  *   col_class   u8  [cols]
+ * raw_interleaved: 0 = raw6 in the frame's order (the 12-byte group g of row r at
+ * (r * cols / 16 + g) * 12); 1 = a row's groups ordered by position in the segment first:
+ * group t of segment s of row r at ((r * seg_len / 16 + t) * segs_per_row + s) * 12, so that
+ * the lanes of a row, which are at the same position of neighbouring segments, read
+ * neighbouring bytes and every 128-byte line is used in one visit.
  * main_bytes must be readable for 16 bytes past main_n_bytes (the kernels copy it in
  * 16-byte units).  raw6 is 4-byte aligned; with seg_len 64 and 16-byte alignment the slab
  * kernels read a segment's 48 residual bytes once, as it starts, instead of 12 at a time. */
@@ -182,6 +191,7 @@ typedef struct grf_bctx_fused {
   uint32_t nr, nc;
   uint32_t seg_len, segs_per_row;
   uint32_t shift, lognb, tabn;
+  uint32_t raw_interleaved;
 } grf_bctx_fused;
 
 /* How a launch cuts the frame into workgroups.  A tile is up to rows_per_tile rows of
