@@ -405,7 +405,7 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
         }
       };
       load_x(xa, 0);
-      for (uint32_t t = 0; t < S; t += 16) {
+      auto group = [&](uint32_t t) {
         uint32_t pair[4];
         load_x(xb, t + 8);
         w.begin16(t, S);
@@ -414,6 +414,11 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
         load_x(xa, min(t + 16, S - 8));  // the last group loads a half again rather than branch around the load
         w.template half<1>(q, pair);
         contract(pair, xb);
+      };
+      // two groups per trip: the registers that carry the next group's residuals, classes and
+      // activations then change roles twice and end where they began, without copies
+      for (uint32_t t = 0; t < S; t += 32) {
+        group(t);
         if (t == 0) {
           // The next unit's stream bytes come from HBM, and its copy to LDS can only start when
           // this walk is over: a wave then waited some 3 us per unit for them.  One word of
@@ -422,6 +427,7 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
           for (uint32_t o = (g0 & ~127u) + p * 128; o < g1; o += P * 128)
             warm ^= *reinterpret_cast<const uint32_t *>(f.main_bytes + o);
         }
+        if (t + 16 < S) group(t + 16);
       }
       if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
     }
