@@ -370,6 +370,9 @@ class FramePlan:
         self.shift = choose_shift(nc, lut_budget or LUT_BUDGET)
         self.lognb = 16 - self.shift
         self.lut, self.tab, self.tabn = sparse_tables(main_freq, nr, nc, self.shift, image)
+        # a context that is one symbol of frequency 65536 (entry field 0): the kernels then keep the
+        # scan that knows such entries
+        self.whole_range = int((np.asarray(main_freq) >= 65536).any())
         self.seg_state = np.concatenate((seg_states, [1 << 23])).astype(np.uint32)
         self.seg_offset = np.concatenate((seg_offsets, [main_bytes])).astype(np.uint32)
         self.row_class = np.asarray(row_class)
@@ -382,7 +385,8 @@ class FramePlan:
 
     def scalars(self):
         return dict(rows=self.rows, cols=self.cols, nr=self.nr, nc=self.nc, seg_len=self.seg_len,
-                    segs_per_row=self.spr, shift=self.shift, lognb=self.lognb, tabn=self.tabn)
+                    segs_per_row=self.spr, shift=self.shift, lognb=self.lognb, tabn=self.tabn,
+                    whole_range=self.whole_range)
 
     def quad_cap(self):
         """Capacity of the row pieces of the GEMM's waves (four segments)."""

@@ -31,7 +31,7 @@ class GrfBctxFused(ctypes.Structure):
                 ("col_class", ctypes.c_void_p)] + [
         (name, ctypes.c_uint32) for name in (
             "main_n_bytes", "rows", "cols", "nr", "nc", "seg_len", "segs_per_row", "shift", "lognb", "tabn",
-            "raw_interleaved")]
+            "raw_interleaved", "whole_range")]
 
 
 class GrfFusedTiling(ctypes.Structure):
@@ -44,7 +44,8 @@ class GrfPpcxFused(ctypes.Structure):
     _fields_ = [(name, ctypes.c_void_p) for name in (
         "main_bytes", "raw5", "seg_state", "seg_offset", "lut", "tab")] + [
         (name, ctypes.c_uint32) for name in (
-            "main_n_bytes", "rows", "cols", "n_labels", "seg_len", "segs_per_row", "shift", "lognb", "tabn")]
+            "main_n_bytes", "rows", "cols", "n_labels", "seg_len", "segs_per_row", "shift", "lognb", "tabn",
+            "whole_range")]
 
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",

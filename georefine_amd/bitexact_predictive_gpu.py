@@ -240,6 +240,7 @@ class HipPredictiveTensor:
         sc = plan.scalars()
         f.seg_len, f.segs_per_row, f.shift, f.lognb, f.tabn = (sc["seg_len"], sc["segs_per_row"], sc["shift"],
                                                                 sc["lognb"], sc["tabn"])
+        f.whole_range = sc["whole_range"]
         self.fused = f
         store = self._tiling_for(0)
         self.fused_plan = dict(sc, **store[3])

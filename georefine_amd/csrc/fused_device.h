@@ -76,7 +76,11 @@ __device__ __forceinline__ uint8_t lds_load_u8(uint32_t off) { return *reinterpr
 
 struct FusedParams {  // uniform values the step needs, kept in scalar registers
   uint32_t shift, block_pitch, table_bytes;
+  uint32_t whole_range;  // some context is one symbol of frequency 65536 (grf_bctx_fused.whole_range)
 };
+// Which scan the step carries for lanes that miss: the one that knows whole-range entries, or
+// the shorter one for frames that promise to have none.
+enum ScanKind : int { kScanAny = 0, kScanNoWholeRange = 1 };
 
 // cc * pitch with cc = byte BYTE of `ccw`: one multiply whose operand select does the extraction
 template <int BYTE>
@@ -182,10 +186,27 @@ __device__ __forceinline__ bool fused_lane_in(uint64_t mask) {
 #endif
 }
 
-// For the lanes that missed: scan from the entry at `s.ta`, backward or forward, to the one
-// that holds the slot.  An entry with frequency 65536 (field 0, start 0) returns rel = state,
-// so that the update freq16 * (state >> 16) + rel leaves the state as it is.
+// For the lanes that missed: from the entry at `s.ta`, whose `rel` (slot - start, as a signed
+// number) says which way to go, step to the entry that holds the slot; the entry in hand is
+// known not to hold it, so the step comes first and the test after.  The tables cover every
+// slot (the host checks that the frequencies of a context add up to 65536), so the scan ends;
+// the trip limit only keeps a wave from spinning on tables that were overwritten.
 __device__ __forceinline__ void fused_scan(uint32_t state, StepFetch &s, uint32_t &rel) {
+  const uint32_t slot = state & 0xFFFFu;
+  uint32_t ta = s.ta;
+  v2u32 e = s.e0;
+  uint32_t left = 256;
+  do {
+    ta += (int32_t)rel < 0 ? -8 : 8;
+    e = *reinterpret_cast<lds_v2u32 *>(ta);
+    rel = slot - (e.x & 0xFFFFu);
+  } while (rel >= (e.x >> 16) && --left);
+  s.e0 = e;
+}
+// The same for frames in which a context may be a single symbol of frequency 65536 (field 0,
+// start 0): such an entry always reports a miss and is not left; it returns rel = state, so
+// that the update freq16 * (state >> 16) + rel leaves the state as it is.
+__device__ __forceinline__ void fused_scan_whole(uint32_t state, StepFetch &s, uint32_t &rel) {
   const uint32_t slot = state & 0xFFFFu;
   uint32_t ta = s.ta;
   v2u32 e = s.e0;
@@ -220,6 +241,7 @@ __device__ __forceinline__ void fused_advance(Cursor &c, StepFetch &s, uint32_t 
 
 // Two consecutive steps of one segment, given the LDS offsets of their contexts' table blocks.
 // Returns the images of the two symbols' bits in the BF16 word (symbol << 5).
+template <int SCAN>
 __device__ __forceinline__ uint32_t fused_finish_step(Cursor &c, StepFetch &s, uint32_t idx, uint32_t block) {
   fused_fetch_entry(s, idx, block);
   fused_pin_bytes(s);
@@ -227,11 +249,17 @@ __device__ __forceinline__ uint32_t fused_finish_step(Cursor &c, StepFetch &s, u
   uint32_t rel = fused_locate(c.state, s.e0.x, miss);
   // a branch on the whole mask first: the common path then leaves EXEC alone
   if (__builtin_expect(miss != 0, 0)) {
-    if (fused_lane_in(miss)) fused_scan(c.state, s, rel);
+    if (fused_lane_in(miss)) {
+      if constexpr (SCAN == kScanNoWholeRange)
+        fused_scan(c.state, s, rel);
+      else
+        fused_scan_whole(c.state, s, rel);
+    }
   }
   fused_advance(c, s, rel);
   return s.e0.y;
 }
+template <int SCAN = kScanAny>
 __device__ __forceinline__ void fused_symbol_pair_in(Cursor &c, uint32_t block0, uint32_t block1, const FusedParams &q,
                                                      uint32_t &hi0, uint32_t &hi1) {
   StepFetch s;
@@ -240,14 +268,14 @@ __device__ __forceinline__ void fused_symbol_pair_in(Cursor &c, uint32_t block0,
   __builtin_amdgcn_sched_barrier(0);  // the lookup byte first: the LDS answers in issue order and the step waits for it
 #endif
   fused_fetch_window(s, c);
-  hi0 = fused_finish_step(c, s, idx0, block0);
+  hi0 = fused_finish_step<SCAN>(c, s, idx0, block0);
   const uint32_t idx1 = fused_fetch_index(c.state, block1, q);
-  hi1 = fused_finish_step(c, s, idx1, block1);
+  hi1 = fused_finish_step<SCAN>(c, s, idx1, block1);
 }
-template <int K>
+template <int K, int SCAN = kScanAny>
 __device__ __forceinline__ void fused_symbol_pair(Cursor &c, uint32_t ccw, const FusedParams &q, uint32_t &hi0,
                                                   uint32_t &hi1) {
-  fused_symbol_pair_in(c, fused_block_offset<K % 4>(ccw, q.block_pitch), fused_block_offset<K % 4 + 1>(ccw, q.block_pitch),
+  fused_symbol_pair_in<SCAN>(c, fused_block_offset<K % 4>(ccw, q.block_pitch), fused_block_offset<K % 4 + 1>(ccw, q.block_pitch),
                        q, hi0, hi1);
 }
 
@@ -396,9 +424,11 @@ struct SegmentWalkT {
   Raw6x16 rr;      // the group being decoded
   uint32_t cw[4];
 
-  // Global reads for segment `seg_` (elem0 / col0: its first element / column), issued
-  // before the workgroup waits for the slab's stream bytes so that their latency overlaps it.
-  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t col0) {
+  // Global reads for segment `seg_` (elem0 / col0: its first element / column; seg_in_row =
+  // col0 / seg_len, which the caller has without dividing), issued before the wait for the
+  // stream bytes so that their latency overlaps it.
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t col0,
+                                           uint32_t seg_in_row) {
     gofs = f.seg_offset[seg_];
     eofs = f.seg_offset[seg_ + 1];
     c.state = f.seg_state[seg_];
@@ -408,7 +438,7 @@ struct SegmentWalkT {
     raw_base = f.raw6;
     cc_base = f.col_class;
     if (f.raw_interleaved) {  // a row's groups ordered by position in the segment, then by segment
-      raw_off = (uint32_t)(((elem0 - col0) / 16 + col0 / f.seg_len) * 12);
+      raw_off = ((uint32_t)((elem0 - col0) / 16) + seg_in_row) * 12;
       raw_stride = f.segs_per_row * 12;
     } else {
       raw_off = (uint32_t)(elem0 / 4 * 3);
@@ -459,13 +489,13 @@ struct SegmentWalkT {
   }
   // Half H (0 or 1) of the group: eight symbols into four BF16 pairs (word k in the low
   // half, k+1 in the high half).
-  template <int H>
+  template <int H, int SCAN = kScanAny>
   __device__ __forceinline__ void half(const FusedParams &q, uint32_t (&pair)[4]) {
     uint32_t bits[8];
 #define GRF_STEP2(i)                                                                   \
   {                                                                                    \
     uint32_t h0, h1;                                                                   \
-    fused_symbol_pair<8 * H + (i)>(c, cw[(8 * H + (i)) / 4], q, h0, h1);               \
+    fused_symbol_pair<8 * H + (i), SCAN>(c, cw[(8 * H + (i)) / 4], q, h0, h1);         \
     bits[i] = fused_word_bits(h0, rr.field<8 * H + (i)>());                            \
     bits[(i) + 1] = fused_word_bits(h1, rr.field<8 * H + (i) + 1>());                  \
   }

@@ -99,7 +99,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
-  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
+  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f), f.whole_range};
 
   const uint32_t r = tid / P, p = tid % P;
   uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
@@ -137,7 +137,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
     const uint64_t elem0 = (uint64_t)row * K + col0;
     Walk w;
     uint32_t a0 = 0;
-    if (walks) w.prefetch(f, seg_base + p, elem0, col0);
+    if (walks) w.prefetch(f, seg_base + p, elem0, col0, first_seg + p);
     if (row != grf::kNoRow) {
       a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
       if (b + 1 < g.n_slabs)  // the next slab's byte range, while this one is walked
@@ -275,7 +275,7 @@ __device__ __forceinline__ float group_sum_to_first_lane(float v, uint32_t logp)
   return v;
 }
 
-template <class Walk, int M>
+template <class Walk, int M, int SCAN>
 __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fused &f, const grf_fused_tiling &g,
                                                 const uint16_t *x, uint32_t ldx, uint16_t *y, uint32_t ldy,
                                                 const uint16_t *bias, int32_t *error, uint32_t tile) {
@@ -291,7 +291,7 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
 #endif
   const uint32_t P = g.lanes_per_row, rpw = 64 / P, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
-  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
+  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f), f.whole_range};
   // P is a power of two: lane coordinates by shift and mask.  A unit u = (row group grp, slab b)
   // with u = grp * n_slabs + b; a wave steps through its units u = wave, wave + nwaves, ... by
   // adding (nwaves / n_slabs, nwaves % n_slabs) with a carry, in scalar registers: divisions by
@@ -363,7 +363,7 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     Walk w;
     {  // every lane loads (see span_of); lanes that do not walk read segment 0's entries
       const uint32_t seg = walks ? row * f.segs_per_row + first_seg + p : 0;
-      w.prefetch(f, seg, walks ? (uint64_t)row * K + col0 : 0, walks ? col0 : 0);
+      w.prefetch(f, seg, walks ? (uint64_t)row * K + col0 : 0, walks ? col0 : 0, walks ? first_seg + p : 0);
     }
     if (walks) w.start(piece_off, a0);
     const uint32_t slot_base = grp * rpw, slab = b;  // this unit's, kept while the counters move on
@@ -409,10 +409,10 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
         uint32_t pair[4];
         load_x(xb, t + 8);
         w.begin16(t, S);
-        w.template half<0>(q, pair);
+        w.template half<0, SCAN>(q, pair);
         contract(pair, xa);
         load_x(xa, min(t + 16, S - 8));  // the last group loads a half again rather than branch around the load
-        w.template half<1>(q, pair);
+        w.template half<1, SCAN>(q, pair);
         contract(pair, xb);
       };
       // two groups per trip: the registers that carry the next group's residuals, classes and
@@ -466,26 +466,37 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
   if (bad) atomicOr(error, (int)bad);
 }
 
-template <class Walk, int M>
+// SCAN: the scan the step carries for lanes whose lookup byte names a neighbour of their symbol
+// (grf::ScanKind); the launch picks the short one for frames without whole-range contexts.  (A
+// choice inside the kernel was tried: after every symbol the two scans' registers have to be
+// brought together again, which cost more than the short scan saves.)
+template <class Walk, int M, int SCAN>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_wave_kernel(
     grf_bctx_fused f, grf_fused_tiling g, const uint16_t *x, uint32_t ldx, uint16_t *y, uint32_t ldy,
     const uint16_t *bias, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  fused_wave_body<Walk, M>(lds, f, g, x, ldx, y, ldy, bias, error, blockIdx.x);
+  fused_wave_body<Walk, M, SCAN>(lds, f, g, x, ldx, y, ldy, bias, error, blockIdx.x);
 }
 
-template <class Walk, int M>
-int launch_wave(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint16_t *y,
-                uint32_t ldy, const uint16_t *bias, int32_t *error, hipStream_t s) {
+template <class Walk, int M, int SCAN>
+int launch_wave_scan(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint16_t *y,
+                     uint32_t ldy, const uint16_t *bias, int32_t *error, hipStream_t s) {
   const WaveLdsLayout L(f, g, M);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
-  constexpr auto kernel = &fused_wave_kernel<Walk, M>;
+  constexpr auto kernel = &fused_wave_kernel<Walk, M, SCAN>;
   if (L.total > 64 * 1024)
     if (int rc = allow_full_lds<kernel>()) return rc;
   hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, x, ldx, y, ldy, bias, error);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
   return GRF_OK;
+}
+
+template <class Walk, int M>
+int launch_wave(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint16_t *y,
+                uint32_t ldy, const uint16_t *bias, int32_t *error, hipStream_t s) {
+  return f.whole_range ? launch_wave_scan<Walk, M, grf::kScanAny>(f, g, x, ldx, y, ldy, bias, error, s)
+                       : launch_wave_scan<Walk, M, grf::kScanNoWholeRange>(f, g, x, ldx, y, ldy, bias, error, s);
 }
 
 // The wave-unit GEMV keeps the activations of a group of columns in registers: two rows per
@@ -562,12 +573,13 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_walk_group_kernel
                                  blockIdx.x - a.first_tile[i]);
 }
 
-template <class Walk, int M>
+template <class Walk, int M, int SCAN>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_wave_group_kernel(
     FusedGroup a, const uint16_t *x, uint32_t ldx, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t i = group_member(a, blockIdx.x);
-  fused_wave_body<Walk, M>(lds, a.f[i], a.g[i], x, ldx, a.y[i], a.ldy[i], a.bias[i], error, blockIdx.x - a.first_tile[i]);
+  fused_wave_body<Walk, M, SCAN>(lds, a.f[i], a.g[i], x, ldx, a.y[i], a.ldy[i], a.bias[i], error,
+                                 blockIdx.x - a.first_tile[i]);
 }
 
 template <class Walk, int M, int SINK>
@@ -711,7 +723,7 @@ __device__ __forceinline__ void gemm_contract(float4v (&acc)[MT], const uint4 (&
 }
 
 // MT: 16-row activation tiles of this launch (m_rows <= 16 * MT, xp packed with m_pad = 16 * MT)
-template <class Walk, int MT>
+template <class Walk, int MT, int SCAN>
 __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fused &f, const grf_fused_tiling &g,
                                                 const uint4 *xp, uint32_t m_rows, uint16_t *y, uint32_t ldy,
                                                 const uint16_t *bias, int32_t *error, uint32_t tile) {
@@ -720,7 +732,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
-  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f)};
+  const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f), f.whole_range};
   constexpr uint32_t m_pad = MT * 16;
 
   const uint32_t lane = tid % 64;
@@ -774,7 +786,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     Walk w;
     {
       const uint32_t seg = active ? row * f.segs_per_row + first_seg + p4 : 0;
-      w.prefetch(f, seg, active ? (uint64_t)row * K + col0 : 0, active ? col0 : 0);
+      w.prefetch(f, seg, active ? (uint64_t)row * K + col0 : 0, active ? col0 : 0, active ? first_seg + p4 : 0);
     }
     if (active) w.start(piece_off, a0);  // (a0: of the lane's own row, which its four lanes share)
     span_of(b + 1, g0, g1);  // the next slab's byte range, on its way during this walk
@@ -797,12 +809,12 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
       uint32_t lo[4] = {0u, 0u, 0u, 0u}, hi[4] = {0u, 0u, 0u, 0u};
       if (active) {
         w.begin16(t, S);
-        w.template half<0>(q, lo);
+        w.template half<0, SCAN>(q, lo);
       }
       gemm_contract<MT>(acc, xa, lo);
       xl += x_step;
       gemm_load_x<MT>(xa, xl);
-      if (active) w.template half<1>(q, hi);
+      if (active) w.template half<1, SCAN>(q, hi);
       gemm_contract<MT>(acc, xa, hi);
       xl += x_step;
       gemm_load_x<MT>(xa, xl);
@@ -843,40 +855,40 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
 }
 
 // Up to four activation tiles: 80 vector registers, six waves per SIMD.
-template <class Walk, int MT>
+template <class Walk, int MT, int SCAN>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_gemm_kernel(
     grf_bctx_fused f, grf_fused_tiling g, const uint4 *xp, uint32_t m_rows, uint16_t *y, uint32_t ldy,
     const uint16_t *bias, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  fused_gemm_body<Walk, MT>(lds, f, g, xp, m_rows, y, ldy, bias, error, blockIdx.x);
+  fused_gemm_body<Walk, MT, SCAN>(lds, f, g, xp, m_rows, y, ldy, bias, error, blockIdx.x);
 }
 
 // Eight activation tiles: the accumulators and operands alone take 64 registers, so fewer
 // waves are resident; still cheaper than decoding the matrix twice.
-template <class Walk, int MT>
+template <class Walk, int MT, int SCAN>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_wide_kernel(grf_bctx_fused f, grf_fused_tiling g,
                                                                                  const uint4 *xp, uint32_t m_rows,
                                                                                  uint16_t *y, uint32_t ldy,
                                                                                  const uint16_t *bias, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  fused_gemm_body<Walk, MT>(lds, f, g, xp, m_rows, y, ldy, bias, error, blockIdx.x);
+  fused_gemm_body<Walk, MT, SCAN>(lds, f, g, xp, m_rows, y, ldy, bias, error, blockIdx.x);
 }
 
-template <class Walk, int MT>
+template <class Walk, int MT, int SCAN>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_gemm_group_kernel(
     FusedGroup a, const uint4 *xp, uint32_t m_rows, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t i = group_member(a, blockIdx.x);
-  fused_gemm_body<Walk, MT>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], error,
+  fused_gemm_body<Walk, MT, SCAN>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], error,
                             blockIdx.x - a.first_tile[i]);
 }
 
-template <class Walk, int MT>
+template <class Walk, int MT, int SCAN>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_wide_group_kernel(FusedGroup a, const uint4 *xp,
                                                                                        uint32_t m_rows, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t i = group_member(a, blockIdx.x);
-  fused_gemm_body<Walk, MT>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], error,
+  fused_gemm_body<Walk, MT, SCAN>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], error,
                             blockIdx.x - a.first_tile[i]);
 }
 
@@ -886,13 +898,20 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
   const GemmLdsLayout L(f, g);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused GEMM: LDS demand exceeds 160 KiB");
   if (x) launch_pack(x, ldx, m_rows, f.cols, MT * 16, xp, s);  // else the caller packed these rows already
-  constexpr auto kernel = [] {
-    if constexpr (MT <= 4) return &fused_gemm_kernel<Walk, MT>;
-    else return &fused_gemm_wide_kernel<Walk, MT>;
-  }();
-  if (L.total > 64 * 1024)
-    if (int rc = allow_full_lds<kernel>()) return rc;
-  hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, xp, m_rows, y, ldy, bias, error);
+  auto launch = [&](auto scan) -> int {
+    constexpr int SCAN = decltype(scan)::value;
+    constexpr auto kernel = [] {
+      if constexpr (MT <= 4) return &fused_gemm_kernel<Walk, MT, SCAN>;
+      else return &fused_gemm_wide_kernel<Walk, MT, SCAN>;
+    }();
+    if (L.total > 64 * 1024)
+      if (int rc = allow_full_lds<kernel>()) return rc;
+    hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, xp, m_rows, y, ldy, bias, error);
+    return GRF_OK;
+  };
+  if (int rc = f.whole_range ? launch(std::integral_constant<int, grf::kScanAny>{})
+                             : launch(std::integral_constant<int, grf::kScanNoWholeRange>{}))
+    return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused GEMM: ") + hipGetErrorString(e));
   return GRF_OK;
@@ -1024,17 +1043,30 @@ int launch_gemv_group(const char *who, const GroupSpec &spec, const uint16_t *x,
       lds = std::max(lds, WaveLdsLayout(a.f[i], a.g[i], kWaveRowsPerPass).total);
     }
     if (lds > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused kernel: LDS demand exceeds 160 KiB");
+    bool whole = false;  // one member with a whole-range context: the scan that knows them, for all
+    for (uint32_t i = 0; i < a.n; ++i) whole = whole || a.f[i].whole_range;
     for (uint32_t m0 = 0; m0 < m_rows; m0 += kWaveRowsPerPass) {
       FusedGroup part = a;
       for (uint32_t i = 0; i < a.n; ++i) part.y[i] = a.y[i] + (size_t)m0 * a.ldy[i];
       const uint16_t *xs = x + (size_t)m0 * ldx;
       const bool one = m_rows - m0 == 1;
-      constexpr auto k1 = &fused_wave_group_kernel<Walk, 1>;
-      constexpr auto k2 = &fused_wave_group_kernel<Walk, 2>;
-      if (lds > 64 * 1024)
-        if (int rc = one ? allow_full_lds<k1>() : allow_full_lds<k2>()) return rc;
-      if (one) hipLaunchKernelGGL(k1, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, part, xs, ldx, error);
-      else hipLaunchKernelGGL(k2, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, part, xs, ldx, error);
+      auto launch = [&](auto kernel_tag) -> int {
+        constexpr auto kernel = decltype(kernel_tag)::value;
+        if (lds > 64 * 1024)
+          if (int rc = allow_full_lds<kernel>()) return rc;
+        hipLaunchKernelGGL(kernel, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, part, xs, ldx, error);
+        return GRF_OK;
+      };
+      using K1 = std::integral_constant<decltype(&fused_wave_group_kernel<Walk, 1, grf::kScanAny>),
+                                        &fused_wave_group_kernel<Walk, 1, grf::kScanAny>>;
+      using K2 = std::integral_constant<decltype(&fused_wave_group_kernel<Walk, 2, grf::kScanAny>),
+                                        &fused_wave_group_kernel<Walk, 2, grf::kScanAny>>;
+      using S1 = std::integral_constant<decltype(&fused_wave_group_kernel<Walk, 1, grf::kScanNoWholeRange>),
+                                        &fused_wave_group_kernel<Walk, 1, grf::kScanNoWholeRange>>;
+      using S2 = std::integral_constant<decltype(&fused_wave_group_kernel<Walk, 2, grf::kScanNoWholeRange>),
+                                        &fused_wave_group_kernel<Walk, 2, grf::kScanNoWholeRange>>;
+      const int rc = whole ? (one ? launch(K1{}) : launch(K2{})) : (one ? launch(S1{}) : launch(S2{}));
+      if (rc) return rc;
       hipError_t e = hipGetLastError();
       if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused kernel: ") + hipGetErrorString(e));
     }
@@ -1066,13 +1098,22 @@ int launch_gemm_group_rows(const FusedGroup &a, uint32_t m_rows, const uint4 *xp
   uint32_t lds = 0;
   for (uint32_t i = 0; i < a.n; ++i) lds = std::max(lds, GemmLdsLayout(a.f[i], a.g[i]).total);
   if (lds > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused GEMM: LDS demand exceeds 160 KiB");
-  constexpr auto kernel = [] {
-    if constexpr (MT <= 4) return &fused_gemm_group_kernel<Walk, MT>;
-    else return &fused_gemm_wide_group_kernel<Walk, MT>;
-  }();
-  if (lds > 64 * 1024)
-    if (int rc = allow_full_lds<kernel>()) return rc;
-  hipLaunchKernelGGL(kernel, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, a, xp, m_rows, error);
+  bool whole = false;  // one member with a whole-range context: the scan that knows them, for all
+  for (uint32_t i = 0; i < a.n; ++i) whole = whole || a.f[i].whole_range;
+  auto launch = [&](auto scan) -> int {
+    constexpr int SCAN = decltype(scan)::value;
+    constexpr auto kernel = [] {
+      if constexpr (MT <= 4) return &fused_gemm_group_kernel<Walk, MT, SCAN>;
+      else return &fused_gemm_wide_group_kernel<Walk, MT, SCAN>;
+    }();
+    if (lds > 64 * 1024)
+      if (int rc = allow_full_lds<kernel>()) return rc;
+    hipLaunchKernelGGL(kernel, dim3(a.first_tile[a.n]), dim3(a.g[0].threads), lds, s, a, xp, m_rows, error);
+    return GRF_OK;
+  };
+  if (int rc = whole ? launch(std::integral_constant<int, grf::kScanAny>{})
+                     : launch(std::integral_constant<int, grf::kScanNoWholeRange>{}))
+    return rc;
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused GEMM: ") + hipGetErrorString(e));
   return GRF_OK;

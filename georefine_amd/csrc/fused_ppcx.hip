@@ -115,7 +115,7 @@ struct PpcxWalk {
     return reinterpret_cast<const uint32_t *>(rawp + ((10 * g) & ~3u));
   }
   // global reads of the segment, issued before the wait for the slab's stream bytes
-  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t) {
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t, uint32_t) {
     gofs = f.seg_offset[seg_];
     eofs = f.seg_offset[seg_ + 1];
     c.state = f.seg_state[seg_];
@@ -145,7 +145,7 @@ struct PpcxWalk {
     n2 = d[2];
     nb = binp[next];
   }
-  template <int H>
+  template <int H, int SCAN = grf::kScanAny>
   __device__ __forceinline__ void half(const grf::FusedParams &q, uint32_t (&pair)[4]) {
     uint32_t bits[8];
 #define GRF_STEP2(i)                                                                                  \
@@ -153,7 +153,7 @@ struct PpcxWalk {
     const uint32_t bin0 = __builtin_amdgcn_ubfe(bw[H], 4 * (i), 4);                                   \
     const uint32_t bin1 = __builtin_amdgcn_ubfe(bw[H], 4 * (i) + 4, 4);                               \
     uint32_t h0, h1;                                                                                  \
-    grf::fused_symbol_pair_in(c, __umul24(bin0, q.block_pitch), __umul24(bin1, q.block_pitch), q, h0, h1); \
+    grf::fused_symbol_pair_in<SCAN>(c, __umul24(bin0, q.block_pitch), __umul24(bin1, q.block_pitch), q, h0, h1); \
     bits[i] = h0 | rr.field<8 * H + (i)>();                                                           \
     bits[(i) + 1] = h1 | rr.field<8 * H + (i) + 1>();                                                 \
   }
@@ -197,6 +197,7 @@ int walker_frame(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, co
   f.shift = frame->shift;
   f.lognb = frame->lognb;
   f.tabn = frame->tabn;
+  f.whole_range = frame->whole_range;
   if (int rc = grf::check_fused_frame(f, *tiling, who, use)) return rc;
   if (f.seg_len % 32)  // a segment's residual bytes must start on a dword
     return grf::set_error(GRF_UNSUPPORTED, std::string(who) + ": segment length must be a multiple of 32");

@@ -175,6 +175,9 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  * group t of segment s of row r at ((r * seg_len / 16 + t) * segs_per_row + s) * 12, so that
  * the lanes of a row, which are at the same position of neighbouring segments, read
  * neighbouring bytes and every 128-byte line is used in one visit.
+ * whole_range: nonzero if some context is a single symbol of frequency 65536 (entry field 0,
+ * the state does not change there); 0 promises there is none, and the scan for lanes whose
+ * lookup byte names a neighbour of their symbol then leaves that case out.
  * main_bytes must be readable for 16 bytes past main_n_bytes (the kernels copy it in
  * 16-byte units).  raw6 is 4-byte aligned; with seg_len 64 and 16-byte alignment the slab
  * kernels read a segment's 48 residual bytes once, as it starts, instead of 12 at a time. */
@@ -192,6 +195,7 @@ typedef struct grf_bctx_fused {
   uint32_t seg_len, segs_per_row;
   uint32_t shift, lognb, tabn;
   uint32_t raw_interleaved;
+  uint32_t whole_range;
 } grf_bctx_fused;
 
 /* How a launch cuts the frame into workgroups.  A tile is up to rows_per_tile rows of
@@ -325,6 +329,7 @@ typedef struct grf_ppcx_fused {
   uint32_t n_labels;
   uint32_t seg_len, segs_per_row;
   uint32_t shift, lognb, tabn;
+  uint32_t whole_range; /* as in grf_bctx_fused */
 } grf_ppcx_fused;
 
 /* The bin of every reference word (GCR/bitexact_predictive_codec.py:106-110, device form
