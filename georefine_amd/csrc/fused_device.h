@@ -304,6 +304,14 @@ struct Raw6x16 {
 
 // ---- pieces of the tile walk shared by the GEMV and GEMM kernels ----
 
+// Entry `i` of the segment index (states or offsets).  The arrays have at most 2^28 + 1 entries
+// (a segment is at least 16 symbols), so the byte offset fits 32 bits: the load then takes the
+// array's base from a scalar pair and the offset from one register, with no 64-bit address
+// arithmetic per lane.
+__device__ __forceinline__ uint32_t fused_index_entry(const uint32_t *index, uint32_t i) {
+  return *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint8_t *>(index) + (i << 2));
+}
+
 // this row class's lookup tables -> LDS, one block per column class: table, then lookup bytes.
 // A thread issues all of its loads of a pass (four 16-byte units of the lookups, four 8-byte
 // entries) before it stores any of them: a loop whose trip count the compiler does not know
@@ -427,21 +435,23 @@ struct SegmentWalkT {
   // Global reads for segment `seg_` (elem0 / col0: its first element / column; seg_in_row =
   // col0 / seg_len, which the caller has without dividing), issued before the wait for the
   // stream bytes so that their latency overlaps it.
-  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint64_t elem0, uint32_t col0,
+  // (A matrix has fewer than 2^32 elements, so element and byte offsets are 32-bit numbers.)
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t col0,
                                            uint32_t seg_in_row) {
-    gofs = f.seg_offset[seg_];
-    eofs = f.seg_offset[seg_ + 1];
-    c.state = f.seg_state[seg_];
-    end_state = f.seg_state[seg_ + 1];
+    gofs = fused_index_entry(f.seg_offset, seg_);
+    eofs = fused_index_entry(f.seg_offset, seg_ + 1);
+    c.state = fused_index_entry(f.seg_state, seg_);
+    end_state = fused_index_entry(f.seg_state, seg_ + 1);
     // a uniform base plus a 32-bit lane offset: the loads then take their address from a scalar
     // pair and one vector register, and no 64-bit address is worked out per group
     raw_base = f.raw6;
     cc_base = f.col_class;
     if (f.raw_interleaved) {  // a row's groups ordered by position in the segment, then by segment
-      raw_off = ((uint32_t)((elem0 - col0) / 16) + seg_in_row) * 12;
+      const uint32_t group = (elem0 - col0) / 16 + seg_in_row;
+      raw_off = ((group << 1) + group) << 2;  // * 12 without the quarter-rate 32-bit multiply
       raw_stride = f.segs_per_row * 12;
     } else {
-      raw_off = (uint32_t)(elem0 / 4 * 3);
+      raw_off = elem0 / 4 * 3;
       raw_stride = 12;
     }
     cc_off = col0;

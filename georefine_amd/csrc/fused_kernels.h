@@ -137,7 +137,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
     const uint64_t elem0 = (uint64_t)row * K + col0;
     Walk w;
     uint32_t a0 = 0;
-    if (walks) w.prefetch(f, seg_base + p, elem0, col0, first_seg + p);
+    if (walks) w.prefetch(f, seg_base + p, (uint32_t)elem0, col0, first_seg + p);
     if (row != grf::kNoRow) {
       a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
       if (b + 1 < g.n_slabs)  // the next slab's byte range, while this one is walked
@@ -253,6 +253,17 @@ struct WaveLdsLayout {
   }
 };
 
+// Product of two numbers below 2^24 whose product is below 2^32 (row and segment indices of a
+// wave tiling: check_fused_frame holds rows and columns to that): the 24-bit multiply issues
+// at full rate, the 32-bit one at a quarter of it.
+__device__ __forceinline__ uint32_t mul24(uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __umul24(a, b);
+#else
+  return a * b;
+#endif
+}
+
 // Sum over the P = 2^logp lanes of a row group, delivered in the group's first lane (other
 // lanes end with partial sums).  Pairwise, neighbours first: ((l0 + l1) + (l2 + l3)) + ...; the
 // first four levels stay inside a row of sixteen lanes and are lane-permuting adds (no LDS
@@ -314,10 +325,10 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
   // discard them.)
   auto span_of = [&](uint32_t b, uint32_t row, uint32_t &g0, uint32_t &g1) {
     const uint32_t first_seg = b << logp;
-    const uint32_t seg_base = row == grf::kNoRow ? 0 : row * f.segs_per_row + first_seg;
+    const uint32_t seg_base = row == grf::kNoRow ? 0 : mul24(row, f.segs_per_row) + first_seg;
     const uint32_t past = row == grf::kNoRow ? 0 : min(P, f.segs_per_row - first_seg);
-    g0 = f.seg_offset[seg_base];
-    g1 = f.seg_offset[seg_base + past];  // (no row: an empty range)
+    g0 = grf::fused_index_entry(f.seg_offset, seg_base);
+    g1 = grf::fused_index_entry(f.seg_offset, seg_base + past);  // (no row: an empty range)
   };
   auto advance = [&](uint32_t &grp, uint32_t &b) {  // the unit nwaves further on
     grp += step_grp;
@@ -356,14 +367,14 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
     if (u != wave) row = slot < R ? rows[slot] : grf::kNoRow;  // (read again: cheaper than a register over the walk)
     const bool walks = row != grf::kNoRow && p < nseg;
-    const uint32_t col0 = (first_seg + p) * S;
+    const uint32_t col0 = mul24(first_seg + p, S);
     // The copy of the pieces goes first: its byte ranges arrived during the walk before, while
     // a wait for them placed after this unit's other loads would wait for those as well.
     const uint32_t a0 = grf::fused_stage_piece_dma(lds, L.stream + wave * rpw * g.piece_cap, g.piece_cap, f, g0, g1, lane, logp, rpw);
     Walk w;
     {  // every lane loads (see span_of); lanes that do not walk read segment 0's entries
-      const uint32_t seg = walks ? row * f.segs_per_row + first_seg + p : 0;
-      w.prefetch(f, seg, walks ? (uint64_t)row * K + col0 : 0, walks ? col0 : 0, walks ? first_seg + p : 0);
+      const uint32_t seg = walks ? mul24(row, f.segs_per_row) + first_seg + p : 0;
+      w.prefetch(f, seg, walks ? mul24(row, K) + col0 : 0, walks ? col0 : 0, walks ? first_seg + p : 0);
     }
     if (walks) w.start(piece_off, a0);
     const uint32_t slot_base = grp * rpw, slab = b;  // this unit's, kept while the counters move on
@@ -758,9 +769,9 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   auto span_of = [&](uint32_t b, uint32_t &g0, uint32_t &g1) {
     const uint32_t first = b * P + quad * 4;
     const bool any = row != grf::kNoRow && first < f.segs_per_row && quad * 4 < P;
-    const uint32_t base = any ? row * f.segs_per_row + first : 0;
-    g0 = f.seg_offset[base];
-    g1 = f.seg_offset[base + (any ? min(4u, min(P - quad * 4, f.segs_per_row - first)) : 0)];
+    const uint32_t base = any ? mul24(row, f.segs_per_row) + first : 0;
+    g0 = grf::fused_index_entry(f.seg_offset, base);
+    g1 = grf::fused_index_entry(f.seg_offset, base + (any ? min(4u, min(P - quad * 4, f.segs_per_row - first)) : 0));
   };
   uint32_t g0, g1;
   span_of(0, g0, g1);  // started before the table copy so that the latencies overlap
@@ -780,13 +791,13 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     __builtin_amdgcn_s_setprio(3);  // between walks a wave's few instructions go first
 #endif
     const bool active = row != grf::kNoRow && p4 < nseg;
-    const uint32_t col0 = (first_seg + p4) * S;
+    const uint32_t col0 = mul24(first_seg + p4, S);
     // the pieces first: their ranges arrived during the walk before
     const uint32_t a0 = grf::fused_stage_piece_dma(lds, region, g.piece_cap, f, g0, g1, lane, 0, 16);
     Walk w;
     {
-      const uint32_t seg = active ? row * f.segs_per_row + first_seg + p4 : 0;
-      w.prefetch(f, seg, active ? (uint64_t)row * K + col0 : 0, active ? col0 : 0, active ? first_seg + p4 : 0);
+      const uint32_t seg = active ? mul24(row, f.segs_per_row) + first_seg + p4 : 0;
+      w.prefetch(f, seg, active ? mul24(row, K) + col0 : 0, active ? col0 : 0, active ? first_seg + p4 : 0);
     }
     if (active) w.start(piece_off, a0);  // (a0: of the lane's own row, which its four lanes share)
     span_of(b + 1, g0, g1);  // the next slab's byte range, on its way during this walk
