@@ -668,12 +668,13 @@ def kernel_name(decode_only, m, grouped, seg_len):
     ahead = "true" if seg_len == 64 else "false"  # 64-symbol segments: the walker that reads a segment's residuals once
     if decode_only:
         return f"grf::fused_walk_kernel<grf::SegmentWalkT<{ahead}>, 1, 1>"
+    # (last template argument 1: the scan for frames without whole-range contexts, which these are)
     if m <= GEMV_UP_TO:
         rows = min(m, 2)  # the wave-unit GEMV carries at most two rows per launch
-        return (f"grf::fused_wave_group_kernel<grf::SegmentWalkT<false>, {rows}>" if grouped
-                else f"grf::fused_wave_kernel<grf::SegmentWalkT<false>, {rows}>")
-    return ("grf::fused_gemm_group_kernel<grf::SegmentWalkT<false>, MT>" if grouped
-            else "grf::fused_gemm_kernel<grf::SegmentWalkT<false>, MT>")
+        return (f"grf::fused_wave_group_kernel<grf::SegmentWalkT<false>, {rows}, 1>" if grouped
+                else f"grf::fused_wave_kernel<grf::SegmentWalkT<false>, {rows}, 1>")
+    return ("grf::fused_gemm_group_kernel<grf::SegmentWalkT<false>, MT, 1>" if grouped
+            else "grf::fused_gemm_kernel<grf::SegmentWalkT<false>, MT, 1>")
 
 
 def kernel_sources_sha256():
