@@ -395,7 +395,6 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     float acc[M];
 #pragma unroll
     for (int m = 0; m < M; ++m) acc[m] = 0.f;
-    uint32_t warm = 0;
     if (walks) {
       // The activations are read eight columns (16 bytes per row) at a time, each load issued
       // while the eight symbols before it are decoded: two register sets, one for the first and
@@ -430,20 +429,11 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
       // activations then change roles twice and end where they began, without copies
       for (uint32_t t = 0; t < S; t += 32) {
         group(t);
-        if (t == 0) {
-          // The next unit's stream bytes come from HBM, and its copy to LDS can only start when
-          // this walk is over: a wave then waited some 3 us per unit for them.  One word of
-          // every 128-byte line of the next piece is read now (its range has arrived by the end
-          // of the first group), which brings the lines into the L2 for that copy to find.
-          for (uint32_t o = (g0 & ~127u) + p * 128; o < g1; o += P * 128)
-            warm ^= *reinterpret_cast<const uint32_t *>(f.main_bytes + o);
-        }
         if (t + 16 < S) group(t + 16);
       }
       if (!w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
     }
 #if defined(__HIP_DEVICE_COMPILE__)
-    asm volatile("" ::"v"(warm));  // (the words read ahead are wanted for their side effect only)
     __builtin_amdgcn_s_setprio(3);
 #endif
     // The unit's sum of a row: its P segment partials (0 for lanes without a segment) added
