@@ -772,6 +772,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   for (int j = 0; j < MT; ++j) acc[j] = (float4v){0.f, 0.f, 0.f, 0.f};
   uint32_t bad = 0;
   __syncthreads();  // the tables are in place
+  const uint32_t later_half = blockIdx.x >= gridDim.x / 2 ? 1u : 0u;
 
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
     const uint32_t first_seg = b * P + quad * 4;
@@ -793,8 +794,15 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     span_of(b + 1, g0, g1);  // the next slab's byte range, on its way during this walk
     __builtin_amdgcn_wave_barrier();
 #if defined(__HIP_DEVICE_COMPILE__)
-    if (b + 1 < g.n_slabs) __builtin_amdgcn_s_setprio(1);
-    else __builtin_amdgcn_s_setprio(0);
+    // walking priority as in the GEMV: the slabs still to do, + 1 for the later-started half of
+    // the grid (left alone, the older of the two workgroups on a compute unit runs ahead and
+    // leaves the other the unit at half occupancy)
+    switch (min(3u, (g.n_slabs - 1 - b) + later_half)) {
+      case 0: __builtin_amdgcn_s_setprio(0); break;
+      case 1: __builtin_amdgcn_s_setprio(1); break;
+      case 2: __builtin_amdgcn_s_setprio(2); break;
+      default: __builtin_amdgcn_s_setprio(3); break;
+    }
 #endif
     if (__ballot(active) == 0) continue;  // nothing to walk in this wave (the branch is per wave)
     // A lane's k-slots are real columns when its segment exists, whether or not its own
