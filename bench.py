@@ -32,6 +32,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0
+LAST_LEVEL_CACHE_BYTES = 256 << 20  # MI355X: 256 MB behind the L2s
 MODEL_BF16_BYTES = 55_586_113_293  # dense BF16 bytes of the 27B model one token has to read at batch 1
 SHAPES = {"gate": (17408, 5120), "up": (17408, 5120), "down": (5120, 17408)}
 # one layer of the whole-stack workload: attention projections, then the MLP
@@ -312,12 +313,17 @@ def run_predictive(args):
         "config": {"workload": f"PPCX target 5120x17408 coded against a reference (target + N(0, 0.002)), product with "
                                f"{m} activation rows as served: contexts of the reference resident as a 4-bit plane, no "
                                f"dense reference; three targets in rotation", "batch": m, "launch": launch},
-        "ms_per_product": round(ms_product, 4), "frame_bytes": len(frame), "resident_bytes": coded,
+        "ms_per_product": round(ms_per_step / len(copies), 4), "ms_per_product_eager_events": round(ms_product, 4),
+        "frame_bytes": len(frame), "resident_bytes": coded,
         "context_plane_bytes": target.size // 2,
         "algorithmic_bytes_per_product": alg, "tok_s_equiv_rows_per_s": round(m * len(copies) / (ms_per_step * 1e-3), 1),
-        "roofline": {"bound": "hbm", "achieved": round(alg / (ms_product * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(alg / (ms_product * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "pack_activations_kernel + grf::fused_gemm_kernel<PpcxWalk, MT> (one product, HIP events)"},
+        # per product: the step's wall time over its products (under a graph the launches follow one
+        # another without host gaps; events around single eager launches, kept beside it, include them)
+        "roofline": {"bound": "hbm", "achieved": round(value, 2), "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": round(value / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": ("grf::fused_wave_kernel<PpcxWalk, 1, SCAN>" if m == 1 else
+                                "pack_activations_kernel + grf::fused_gemm_kernel / fused_gemm_wide_kernel<PpcxWalk, MT, SCAN>")
+                               + " (a product's share of the step)"},
     }), flush=True)
 
 
@@ -561,23 +567,41 @@ def main():
     if not args.no_groups and "gate" in names and "up" in names:
         pair = HipLinearGroup([tensors["gate"], tensors["up"]])
 
+    # Device copies of the layer's matrices, taken in turn by the timed steps and launches, enough
+    # that any one matrix's copies are twice the last-level cache: repeated passes over one 128 MB
+    # matrix would find it in that cache, which a model of 64 layers never does.
+    n_layers = max(1, -(-2 * LAST_LEVEL_CACHE_BYTES // min(tensors[n_].resident_bytes for n_ in names)))
+    layers = [(tensors, pair)]
+    for _ in range(n_layers - 1):
+        copy_ = {n_: tensors[n_].clone() for n_ in names}
+        layers.append((copy_, HipLinearGroup([copy_["gate"], copy_["up"]]) if pair is not None else None))
+    log(f"{n_layers} device copies of the layer, taken in turn")
+
     def measure(m):
         """One workload at m activation rows (0: decode to dense): (result fields, x words)."""
         rng = np.random.default_rng(7)
         x_words = {k: bf16_words(rng.normal(0, 1, size=(max(m, 1), k))) for k in (5120, 17408)}
         x = {k: torch.from_numpy(v).view(torch.bfloat16).cuda() for k, v in x_words.items()}
-        units = []  # (label, member names, callable)
+
+        def units_of(tensors, pair):  # the launches of a step: (label, member names, callable)
+            units = []
+            if pair is not None and not decode_only:
+                units.append(("gate+up", ["gate", "up"], lambda: pair.linear(x[5120])))
+            for name in names:
+                if decode_only:
+                    units.append((name, [name], lambda name=name: tensors[name].decode(check=False)))
+                elif not any(name in u[1] for u in units):
+                    units.append((name, [name], lambda name=name: tensors[name].linear(x[SHAPES[name][1]])))
+            return units
+
+        per_layer = [units_of(*layer) for layer in layers]
+        units = per_layer[0]
         if pair is not None and not decode_only:
-            units.append(("gate+up", ["gate", "up"], lambda: pair.linear(x[5120])))
             log(f"batch {m} gate+up: one launch, tiling {pair._tiling('waves' if m <= GEMV_UP_TO else 'gemm')[0][3]}")
-        for name in names:
-            if decode_only:
-                units.append((name, [name], lambda name=name: tensors[name].decode(check=False)))
-            elif not any(name in u[1] for u in units):
-                units.append((name, [name], lambda name=name: tensors[name].linear(x[SHAPES[name][1]])))
         ms_per_step, per_kernel_ms, launch, timing = time_launches(
-            torch, units, args.steps, args.warmup, args.graph,
-            lambda: [n_ for n_ in names if tensors[n_].error.item()] + ([] if pair is None or not pair.error.item() else ["gate+up"]))
+            torch, per_layer, args.steps, args.warmup, args.graph,
+            lambda: sorted({n_ for ts, pr in layers for n_ in names if ts[n_].error.item()}
+                           | {"gate+up" for ts, pr in layers if pr is not None and pr.error.item()}))
         if args.calibrate_copy:
             src = torch.ones(32 * 1024 * 1024, dtype=torch.int32, device="cuda")
             dst = torch.empty_like(src)
@@ -608,7 +632,8 @@ def main():
                                    + (", residuals resident in packed 6-bit form"
                                       if any(tensors[n_].resident_mode != tensors[n_].mode for n_ in names) else ""),
                        "batch": m, "matrices": names, "launches": [u[0] for u in units],
-                       "segment": tensors[names[0]].fused_plan["seg_len"], "launch": launch, "per_kernel_timing": timing},
+                       "segment": tensors[names[0]].fused_plan["seg_len"], "launch": launch, "per_kernel_timing": timing,
+                       "layer_copies": n_layers},
             "effective_bf16_GBps": round(eff_bf16, 2),
             "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3) if m else None,
             "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
@@ -654,7 +679,7 @@ def main():
         result["cpu_baseline"] = cpu_baseline(frames, words_of, x_words)
         result["cpu_baseline"]["host"] = host_description()
     if headline and not args.no_stack:
-        del tensors, pair
+        del tensors, pair, layers
         torch.cuda.empty_cache()
         log("whole stack ...")
         stack_args = argparse.Namespace(**vars(args))
@@ -707,31 +732,37 @@ def recorded_traffic(decode_only, m, kernel):
     return per_kernel[short], f"recorded: profiles/{name} (rocprofv3 --pmc, same kernel sources)"
 
 
-def time_launches(torch, units, steps, warmup, graph, errors):
+def time_launches(torch, per_layer, steps, warmup, graph, errors):
     """(ms per step, {label: ms per launch}, how the step was launched, how launches were timed).
 
-    After `warmup` eager steps: each launch of the step is captured ten times into a HIP graph
-    of its own and the replays are bracketed by events on the launch stream, which gives the
-    kernel's duration without the host's per-launch latency (eager events around single
-    launches where capture is not possible or --no-graph is given); then `steps` replays of
-    a graph of the whole step are timed on the host clock between synchronisations."""
-    def step():
-        return [run() for _, _, run in units]
+    `per_layer[c]` holds the launches of a step on copy c of the layer's matrices; step i runs
+    on copy i mod len(per_layer), so no step finds its matrices in the caches.  After `warmup`
+    eager steps: each launch is captured twelve times into a HIP graph of its own, over the
+    copies in turn, and the replays are bracketed by events on the launch stream, which gives
+    the kernel's duration without the host's per-launch latency (eager events around single
+    launches where capture is not possible or --no-graph is given); then exactly `steps` steps,
+    replayed from graphs of up to 96 consecutive steps, are timed on the host clock between
+    synchronisations."""
+    copies = len(per_layer)
 
-    for _ in range(warmup):
-        step()
+    def step(i):
+        return [run() for _, _, run in per_layer[i % copies]]
+
+    for i in range(warmup):
+        step(i)
     torch.cuda.synchronize()
     bad = errors()
     if bad:
         sys.exit(f"bench.py: decoder error word set for {bad}")
-    per_kernel_ms, timing = {}, "HIP events around 10 launches per graph replay"
+    per_kernel_ms = {}
+    timing = f"HIP events around 12 launches per graph replay, over {copies} device copies of the matrices in turn"
     if graph:
         try:
-            for label, _, run in units:
+            for j, (label, _, _) in enumerate(per_layer[0]):
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g):
-                    for _ in range(10):
-                        run()
+                    for i in range(12):
+                        per_layer[i % copies][j][2]()
                 g.replay()
                 torch.cuda.synchronize()
                 a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -741,48 +772,56 @@ def time_launches(torch, units, steps, warmup, graph, errors):
                     g.replay()
                 b.record()
                 torch.cuda.synchronize()
-                per_kernel_ms[label] = a.elapsed_time(b) / (10 * replays)
+                per_kernel_ms[label] = a.elapsed_time(b) / (12 * replays)
         except Exception as exc:
             log(f"graph capture failed ({exc}); timing eager launches")
             per_kernel_ms = {}
     if not per_kernel_ms:
         timing = "HIP events around single eager launches"
-        starts = [[torch.cuda.Event(enable_timing=True) for _ in units] for _ in range(steps)]
-        ends = [[torch.cuda.Event(enable_timing=True) for _ in units] for _ in range(steps)]
+        n_units = len(per_layer[0])
+        starts = [[torch.cuda.Event(enable_timing=True) for _ in range(n_units)] for _ in range(steps)]
+        ends = [[torch.cuda.Event(enable_timing=True) for _ in range(n_units)] for _ in range(steps)]
         torch.cuda.synchronize()
         for s_ in range(steps):
-            for j, (_, _, run) in enumerate(units):
+            for j, (_, _, run) in enumerate(per_layer[s_ % copies]):
                 starts[s_][j].record()
                 run()
                 ends[s_][j].record()
         torch.cuda.synchronize()
         per_kernel_ms = {label: float(np.mean([starts[s_][j].elapsed_time(ends[s_][j]) for s_ in range(steps)]))
-                         for j, (label, _, _) in enumerate(units)}
+                         for j, (label, _, _) in enumerate(per_layer[0])}
     launch = "eager"
     wall = None
     if graph:
-        # the same step captured once and replayed: the launches of a step are submitted together,
-        # which takes the host's per-launch latency out of the gaps between kernels
+        # consecutive steps captured once and replayed: the launches are submitted together, which
+        # takes the host's per-launch latency out of the gaps between kernels
         try:
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
-                step()
-            g.replay()
+            chunk = min(steps, 96) // copies * copies or steps  # whole turns through the copies
+            plan = [(chunk, steps // chunk)] + ([(steps % chunk, 1)] if steps % chunk else [])
+            graphs = []
+            for length, times in plan:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    for i in range(length):
+                        step(i)
+                g.replay()
+                graphs.append((g, times))
             torch.cuda.synchronize()
         except Exception as exc:  # keep the eager figure
             log(f"graph capture failed ({exc}); reporting the eager steps")
         else:
             wall0 = time.perf_counter()
-            for _ in range(steps):
-                g.replay()
+            for g, times in graphs:
+                for _ in range(times):
+                    g.replay()
             torch.cuda.synchronize()
             wall = time.perf_counter() - wall0
             launch = "hip graph replay"
     if wall is None:
         torch.cuda.synchronize()
         wall0 = time.perf_counter()
-        for _ in range(steps):
-            step()
+        for i in range(steps):
+            step(i)
         torch.cuda.synchronize()
         wall = time.perf_counter() - wall0
     bad = errors()
