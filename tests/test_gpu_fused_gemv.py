@@ -136,3 +136,35 @@ def test_residual_buffer_off_a_16_byte_boundary_gives_the_same_bits():
     for m in (1, 2, 4):
         x = torch.from_numpy(bf16_words(np.random.default_rng(m).normal(0, 1, size=(m, 768)))).view(torch.bfloat16).cuda()
         assert torch.equal(other.gemv(x, check=True), t.gemv(x, check=True))
+
+
+def test_scan_variants_and_the_whole_range_promise(oracle):
+    """A context that is one symbol of frequency 65536 needs the scan that knows such entries;
+    the planner flags the frame and the launches pick the kernel variant.  Products of a frame
+    with such contexts are right; with the flag cleared from the host (a broken promise) the
+    short scan runs out of its trip limit, the kernels finish normally and the segments miss
+    their checkpoints."""
+    import torch
+    from georefine_amd import bitexact_context_codec as codec
+    rng = np.random.default_rng(31)
+    words = weight_like(rng, 64, 512)
+    words[:, :128] = 0x3F80  # with four column classes by magnitude: one class of constant columns
+    words[::2, :128] = 0xBF80  # (the sign is in the residual: the main symbol stays the same)
+    frame, t = _tensor(words, 1, 4)
+    assert t.fused is not None and t.fused.whole_range == 1, t.fused_plan
+    plain_frame, plain = _tensor(weight_like(rng, 64, 512), 1, 4)
+    assert plain.fused.whole_range == 0
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(20, 512)))).view(torch.bfloat16).cuda()
+    dense = torch.from_numpy(words).view(torch.bfloat16).cuda().float()
+    want = torch.nn.functional.linear(x.float(), dense)
+    scale = torch.nn.functional.linear(x.float().abs(), dense.abs())
+    for y in (t.gemv(x[:1], check=True), t.gemv(x[:2], check=True), t.gemm(x, check=True)):
+        n = y.shape[0]
+        assert bool((y.float() - want[:n]).abs().le(1e-2 * want[:n].abs().clamp_min(1e-3 * scale[:n]) + 1e-30).all())
+    assert np.array_equal(t.decode().view(torch.uint16).cpu().numpy(), words)
+    t.fused.whole_range = 0  # forced from the host; every kernel still exits normally
+    print("whole_range cleared on a frame that has such contexts", flush=True)
+    with pytest.raises(codec.CodecError):
+        t.gemv(x[:1], check=True)
+    with pytest.raises(codec.CodecError):
+        t.gemm(x, check=True)
