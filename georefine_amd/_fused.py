@@ -404,6 +404,7 @@ class FramePlan:
         (m = 0: the store sink).  ``waves``: the wave-unit scheme of the GEMV, one tiling for
         every row count (launches carry at most two rows each)."""
         if waves and m:
+            self._wave_limits()
             threads, p, r, n_slabs, n_tiles, cap, lds = choose_wave_tiling(
                 self.spr, self.class_rows, self._cap,
                 lambda t_, p_, r_, s_, cap_: lds_bytes_waves(self.nc, self.lognb, self.tabn, WAVE_ROWS_PER_PASS, t_, p_,
@@ -433,9 +434,15 @@ class FramePlan:
         return dict(threads=-(-p // 64) * 64, lanes_per_row=p, rows_per_tile=1, n_slabs=-(-self.spr // p),
                     piece_cap=cap), lds
 
+    def _wave_limits(self):
+        """Kernels over wave tilings address rows and segments with 24-bit multiplies."""
+        if self.rows >= 1 << 24 or self.cols >= 1 << 24:
+            raise FusedUnsupported("wave tilings take fewer than 2^24 rows and columns")
+
     def gemm_tiling(self):
         """The one tiling every fused GEMM launch uses, whatever its row count: the order in
         which an output element accumulates follows the tiling, so it must not change with M."""
+        self._wave_limits()
         threads, p, r, n_slabs, n_tiles, cap, lds = choose_gemm_tiling(
             self.spr, self.class_rows, lambda lanes: self.quad_cap(),
             lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, p_, r_, cap_),
@@ -459,6 +466,9 @@ def plan_group(plans, m=None, gemm=False, waves=False):
     cap_fn = lambda lanes: max(pl._cap(lanes) for pl in plans)
     table = max(pl.table_bytes() for pl in plans)
     scheme = SCHEME_SLABS
+    if gemm or waves:
+        for pl in plans:
+            pl._wave_limits()
     if gemm:
         scheme = SCHEME_WAVES
         lds_fn = lambda p_, r_, cap_: max(lds_bytes_gemm(pl.nc, pl.lognb, pl.tabn, p_, r_, cap_) for pl in plans)
