@@ -1,16 +1,17 @@
 // Kernels and launchers of the fused sinks, generic over the segment walker: the same
 // bodies serve the context codec (grf::SegmentWalk) and the predictive codec (its walker
 // in fused_ppcx.hip).  A walker provides prefetch(frame, segment, first element, first
-// column), start(piece offset, staged-from offset), begin16(t, S) + half<0|1>(params,
-// pair[4]) for the two halves of a group of 16 symbols (decode16 = all three) and
-// ended_on_checkpoint(frame).
+// column, segment's position in its row), start(piece offset, staged-from offset),
+// begin16(t, S) + half<0|1, scan kind>(params, pair[4]) for the two halves of a group of
+// 16 symbols (decode16 = all three) and ended_on_checkpoint(frame).
 //
-// GEMV: reduction order of one output element, fixed for every M and for every tiling:
-// the S products of a segment are folded into one fp32 accumulator two columns at a
-// time in increasing k (v_dot2c_f32_bf16: acc += w[k]*x[k] + w[k+1]*x[k+1]); the K/S
-// segment partials of a row are then added in segment order 0..K/S-1 by one thread
-// (slab after slab into a running sum); bias is added in fp32 and the sum is rounded
-// to BF16 once.
+// GEMV: reduction order of one output element, fixed for every M: the S products of a
+// segment are folded into one fp32 accumulator two columns at a time in increasing k
+// (v_dot2c_f32_bf16: acc += w[k]*x[k] + w[k+1]*x[k+1]).  Slab tilings then add the K/S
+// segment partials of a row in segment order 0..K/S-1 by one thread (slab after slab into
+// a running sum); wave tilings add the P partials of a unit pairwise, neighbours first,
+// and the units' sums of a row in slab order (fused_wave_body).  Bias is added in fp32 and
+// the sum is rounded to BF16 once.
 //
 // GEMM, batch invariance (the contract of GS/bi_csrc/bi_gemm.cuh:1-17): output element
 // (m, n) is the sum, in quad order, of one fp32 accumulator per quad of lane-segments;
