@@ -208,11 +208,15 @@ typedef struct grf_bctx_fused {
  *   scheme      GRF_TILE_SLABS: lane (r, p) of the workgroup walks segment b*lanes_per_row + p
  *               of the tile's row r in slab b, the whole workgroup slab by slab
  *               (threads >= rows_per_tile*lanes_per_row).
- *               GRF_TILE_WAVES (GEMV only): a wave is a unit of 64/lanes_per_row rows by
+ *               GRF_TILE_WAVES, GEMV: a wave is a unit of 64/lanes_per_row rows by
  *               lanes_per_row segments (lanes_per_row a power of two, 4..64); the waves of
  *               the workgroup take the tile's units (row group g, slab b) in turn and share
  *               nothing but the lookup tables, so there is no barrier between the table copy
  *               and the final row sums.
+ *               GRF_TILE_WAVES, GEMM: a wave keeps 16 rows of the tile and four of a slab's
+ *               lanes_per_row segments for the whole launch and stages its own stream pieces
+ *               (see grf_bctx_gemm for threads and piece_cap).
+ *               Wave tilings take matrices with fewer than 2^24 rows and 2^24 columns.
  * n_slabs = ceil(segs_per_row / lanes_per_row) in both schemes. */
 #define GRF_TILE_SLABS 0
 #define GRF_TILE_WAVES 1
@@ -257,9 +261,11 @@ int grf_bctx_fused_gather(const grf_bctx_fused *frame, const grf_fused_tiling *t
  * with one tiling, row m of y is a function of row m of x and of W only.  x must be
  * 8-byte aligned with ldx a multiple of 4.  More than 128 rows run as several launches.
  *
- * A tiling for this function has threads = 64 * ceil(rows_per_tile / 16) *
- * ceil(lanes_per_row / 4): a wave walks four lane-segments of 16 rows and feeds the words
- * it decodes to the matrix cores from its registers.  workspace: device memory, 16-byte
+ * A tiling for this function has scheme = GRF_TILE_WAVES, threads = 64 *
+ * ceil(rows_per_tile / 16) * ceil(lanes_per_row / 4), and a piece_cap that holds the longest
+ * stream piece of four consecutive segments of a row (from its 16-byte aligned start, + 8):
+ * a wave walks four lane-segments of 16 rows and feeds the words it decodes to the matrix
+ * cores from its registers.  workspace: device memory, 16-byte
  * aligned, at least grf_gemm_workspace_bytes(cols, m_rows) bytes; each launch first writes
  * its activation rows there in operand order (a copy of x: cols * 32 + 256 bytes per 16 rows),
  * so calls that share a workspace must be ordered on one stream. */
