@@ -703,10 +703,21 @@ inline void launch_pack(const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint32
                      chunks, xp);
 }
 
+// The lane's A operands of one half group: tile j of the packed activations at byte offset
+// `at` + 256 j of `xp`.  Up to four tiles: a uniform base and a 32-bit lane offset (the packed
+// copy is a few MB), which keeps a 64-bit address out of the registers that the walk needs;
+// with eight tiles the compiler does better with the address.
 template <int MT>
-__device__ __forceinline__ void gemm_load_x(uint4 (&xa)[MT], const uint4 *xl) {
+__device__ __forceinline__ void gemm_load_x(uint4 (&xa)[MT], const uint4 *xp, uint32_t at) {
+  const uint8_t *base = reinterpret_cast<const uint8_t *>(xp);
+  if constexpr (MT <= 4) {
 #pragma unroll
-  for (int j = 0; j < MT; ++j) xa[j] = xl[j * 16];
+    for (int j = 0; j < MT; ++j) xa[j] = *reinterpret_cast<const uint4 *>(base + (at + (uint32_t)j * 256u));
+  } else {
+    const uint4 *xl = reinterpret_cast<const uint4 *>(base + (size_t)at);
+#pragma unroll
+    for (int j = 0; j < MT; ++j) xa[j] = xl[j * 16];
+  }
 }
 
 template <int MT>
@@ -811,10 +822,15 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     // they read the chunk of zeros that ends the packed copy and never move on.  The load
     // after a segment's last half group reads the chunk that follows it, at most that one.
     const bool feeds = p4 < nseg;
-    const uint32_t x_step = feeds ? m_pad : 0;
-    const uint4 *xl = xp + (size_t)(feeds ? col0 / 8 : K / 8) * m_pad + lane % 16;
+    const uint32_t x_step = feeds ? m_pad * 16 : 0;  // bytes from one 8-column chunk to the next
+    // (the lane's number is worked out again here rather than kept in a register over the walks)
+    uint32_t ln = __lane_id();
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" : "+v"(ln));
+#endif
+    uint32_t xl = ((feeds ? col0 / 8 : K / 8) * m_pad + ln % 16) * 16;
     uint4 xa[MT];
-    gemm_load_x<MT>(xa, xl);
+    gemm_load_x<MT>(xa, xp, xl);
     for (uint32_t t = 0; t < S; t += 16) {
       uint32_t lo[4] = {0u, 0u, 0u, 0u}, hi[4] = {0u, 0u, 0u, 0u};
       if (active) {
@@ -823,11 +839,11 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
       }
       gemm_contract<MT>(acc, xa, lo);
       xl += x_step;
-      gemm_load_x<MT>(xa, xl);
+      gemm_load_x<MT>(xa, xp, xl);
       if (active) w.template half<1, SCAN>(q, hi);
       gemm_contract<MT>(acc, xa, hi);
       xl += x_step;
-      gemm_load_x<MT>(xa, xl);
+      gemm_load_x<MT>(xa, xp, xl);
     }
     if (active && !w.ended_on_checkpoint(f)) bad |= GRF_ERR_CHECKPOINT;
   }
@@ -839,16 +855,23 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   // four activation tiles at a time, which is what the LDS allocation is sized for
   constexpr int CT = MT < (int)kSumTiles ? MT : (int)kSumTiles;
   float *sums = reinterpret_cast<float *>(lds);
+  // (the thread's coordinates are worked out again rather than kept in registers, or spilled,
+  // over the walk)
+  uint32_t lane2 = __lane_id();
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("" : "+v"(lane2));
+#endif
+  const uint32_t tid2 = wave * 64 + lane2;
 #pragma unroll
   for (int c0 = 0; c0 < MT; c0 += CT) {
     __syncthreads();  // tables and stream bytes (or the previous chunk's sums) are done with
 #pragma unroll
     for (int jj = 0; jj < CT; ++jj)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) sums[((wave * CT + jj) * 4 + v) * 64 + lane] = acc[c0 + jj][v];
+      for (int v = 0; v < 4; ++v) sums[((wave * CT + jj) * 4 + v) * 64 + lane2] = acc[c0 + jj][v];
     __syncthreads();
     const uint32_t per_block = CT * 256;  // values of one row block: [tile jj][v][lane]
-    for (uint32_t i = tid; i < shape.row_blocks * per_block; i += nthreads) {
+    for (uint32_t i = tid2; i < shape.row_blocks * per_block; i += nthreads) {
       const uint32_t blk = i / per_block, within = i % per_block;
       const uint32_t jj = within / 256, v = (within / 64) % 4, ln = within % 64;
       const uint32_t n_local = blk * 16 + ln % 16, m = (c0 + jj) * 16 + (ln / 16) * 4 + v;
