@@ -293,29 +293,39 @@ def choose_wave_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=6
 
 
 GEMM_WAVES_PER_SIMD = int(os.environ.get("GEOREFINE_GEMM_WAVES", "6"))
+# a single matrix's GEMM may be cut along K ("0": never; experiments and tests of the uncut kernel)
+GEMM_SPLIT = os.environ.get("GEOREFINE_FUSED_GEMM_SPLIT", "1") != "0"
 
 
-def choose_gemm_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=64, table_bytes=0):
+GEMM_K_PARTS = (1, 2, 3, 4, 6, 8)  # cuts along K the planner tries for a single matrix
+
+
+def choose_gemm_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=64, table_bytes=0, split=False):
     """Tiling of the GEMM kernel: workgroups of (row blocks of 16) x (quads of 4
     lane-segments) waves.  Same model as choose_tiling, counted in waves: a wave is busy
     for as long as its busiest lane, so idle lanes inside a wave are free, idle waves and
-    idle CUs are not."""
+    idle CUs are not.  With ``split`` the launch may also be cut into k parts along K (every
+    row tile k times, each copy walking a k-th of the slabs, the parts' sums added by a small
+    second kernel): a matrix with few rows then fills the machine with full blocks of sixteen
+    rows.  Returns (threads, lanes per row, rows per tile, slabs, tiles of the launch, piece
+    capacity, LDS bytes, k)."""
     best = None
     total_rows = sum(int(c) for c in class_rows)
-    forced = os.environ.get("GEOREFINE_FUSED_GEMM_TILING")  # "lanes_per_row,rows": experiments only
-    choices = None
+    forced = os.environ.get("GEOREFINE_FUSED_GEMM_TILING")  # "lanes_per_row,rows[,k_parts]": experiments only
     if forced:
-        p_, r_ = (int(v) for v in forced.split(","))
-        choices = [(min(p_, spr), r_)]
+        values = [int(v) for v in forced.split(",")]
+        choices = [(min(values[0], spr), values[1], values[2] if len(values) > 2 and split else 1)]
     else:
-        choices = [(min(4 * quads, spr), 16 * blocks) for quads in range(1, -(-spr // 4) + 1)
-                   for blocks in range(1, 17) if quads * blocks <= 16]
-    for p, r in dict.fromkeys(choices):
+        choices = [(min(4 * quads, spr), 16 * blocks, k) for quads in range(1, -(-spr // 4) + 1)
+                   for blocks in range(1, 17) if quads * blocks <= 16
+                   for k in (GEMM_K_PARTS if split else (1,))]
+    for p, r, k in dict.fromkeys(choices):
         row_blocks, quads, threads = gemm_shape(p, r)
         if threads > 1024:
             continue
         n_slabs = -(-spr // p)
-        tiles = _tiles(class_rows, r)
+        if k > n_slabs:
+            continue
         cap = piece_cap_fn(p)
         lds = lds_fn(p, r, cap)
         if lds > MAX_LDS:
@@ -323,16 +333,19 @@ def choose_gemm_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=6
         per_simd = -(-(threads // 64) // 4)
         per_cu = max(1, min(GEMM_WAVES_PER_SIMD // per_simd, MAX_LDS // lds))
         slots = cus * per_cu
-        rounds = -(-tiles // slots)
-        r_used = r if forced else _spread_rows(class_rows, r, rounds * slots, floor=16 * (row_blocks - 1) + 1)
-        tiles_used = _tiles(class_rows, r_used)
+        rounds = -(-(_tiles(class_rows, r) * k) // slots)
+        r_used = r if forced else _spread_rows(class_rows, r, rounds * slots // k, floor=16 * (row_blocks - 1) + 1)
+        tiles_used = _tiles(class_rows, r_used) * k
+        slabs_each = -(-n_slabs // k)
         # work = lane-steps; capacity = every wave slot of every round for the whole walk
         work = total_rows * spr
-        paid = rounds * slots * (threads // 64) * 16 * 4 * n_slabs
+        paid = rounds * slots * (threads // 64) * 16 * 4 * slabs_each
         waves = per_cu * (threads // 64)
-        score = work / paid * min(1.0, waves / 24) * _walk_share(n_slabs, seg_len, table_bytes)
+        score = work / paid * min(1.0, waves / 24) * _walk_share(slabs_each, seg_len, table_bytes)
+        if k > 1:  # the second kernel, and every part's sums written and read once more
+            score *= 0.97 - 0.015 * k
         if best is None or score > best[0] + 1e-9:
-            best = (score, threads, p, r_used, n_slabs, tiles_used, cap, lds_fn(p, r_used, cap))
+            best = (score, threads, p, r_used, n_slabs, tiles_used, cap, lds_fn(p, r_used, cap), k)
     if best is None:
         raise FusedUnsupported("no GEMM tiling fits in LDS")
     return best[1:]
@@ -443,15 +456,15 @@ class FramePlan:
         """The one tiling every fused GEMM launch uses, whatever its row count: the order in
         which an output element accumulates follows the tiling, so it must not change with M."""
         self._wave_limits()
-        threads, p, r, n_slabs, n_tiles, cap, lds = choose_gemm_tiling(
+        threads, p, r, n_slabs, n_tiles, cap, lds, k = choose_gemm_tiling(
             self.spr, self.class_rows, lambda lanes: self.quad_cap(),
             lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, p_, r_, cap_),
-            seg_len=self.seg_len, table_bytes=self.table_bytes())
-        tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
-        assert len(tile_class) == n_tiles
+            seg_len=self.seg_len, table_bytes=self.table_bytes(), split=GEMM_SPLIT)
+        tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)  # the row tiles; the launch has k of each
+        assert len(tile_class) * k == n_tiles
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
-                                 n_tiles=n_tiles, piece_cap=cap, scheme=SCHEME_WAVES), lds=lds)
+                                 n_tiles=n_tiles, piece_cap=cap, scheme=SCHEME_WAVES, k_parts=k), lds=lds)
 
 
 def plan_group(plans, m=None, gemm=False, waves=False):
@@ -473,8 +486,8 @@ def plan_group(plans, m=None, gemm=False, waves=False):
         scheme = SCHEME_WAVES
         lds_fn = lambda p_, r_, cap_: max(lds_bytes_gemm(pl.nc, pl.lognb, pl.tabn, p_, r_, cap_) for pl in plans)
         quad_cap = max(pl.quad_cap() for pl in plans)
-        threads, p, r, n_slabs, _, cap, lds = choose_gemm_tiling(first.spr, class_rows, lambda lanes: quad_cap, lds_fn,
-                                                                 seg_len=first.seg_len, table_bytes=table)
+        threads, p, r, n_slabs, _, cap, lds, _ = choose_gemm_tiling(first.spr, class_rows, lambda lanes: quad_cap, lds_fn,
+                                                                    seg_len=first.seg_len, table_bytes=table)
     elif waves:
         scheme = SCHEME_WAVES
         lds_fn = lambda t_, p_, r_, s_, cap_: max(lds_bytes_waves(pl.nc, pl.lognb, pl.tabn, WAVE_ROWS_PER_PASS, t_, p_, r_,

@@ -37,7 +37,7 @@ class GrfBctxFused(ctypes.Structure):
 class GrfFusedTiling(ctypes.Structure):
     _fields_ = [("tile_rows", ctypes.c_void_p), ("tile_class", ctypes.c_void_p)] + [
         (name, ctypes.c_uint32) for name in (
-            "threads", "lanes_per_row", "rows_per_tile", "n_slabs", "n_tiles", "piece_cap", "scheme")]
+            "threads", "lanes_per_row", "rows_per_tile", "n_slabs", "n_tiles", "piece_cap", "scheme", "k_parts")]
 
 
 class GrfPpcxFused(ctypes.Structure):
@@ -50,7 +50,7 @@ class GrfPpcxFused(ctypes.Structure):
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
                   "grf_bctx_fused_decode", "grf_bctx_fused_gather", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
-                  "grf_gemm_workspace_bytes", "grf_bctx_gemm_noalloc", "grf_gemm_noalloc_limit_bytes", "grf_pack_activations", "grf_bctx_gemv_group", "grf_bctx_gemm_group",
+                  "grf_gemm_workspace_bytes", "grf_gemm_workspace_bytes_split", "grf_bctx_gemm_noalloc", "grf_gemm_noalloc_limit_bytes", "grf_pack_activations", "grf_bctx_gemv_group", "grf_bctx_gemm_group",
                   "grf_ppcx_bins", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_last_error",
                   "grf_abi_version")
 
@@ -73,6 +73,8 @@ def declare(L):
     L.grf_bctx_gemm_lds_bytes.restype = u32
     L.grf_gemm_workspace_bytes.argtypes = [u32, u32]
     L.grf_gemm_workspace_bytes.restype = ctypes.c_size_t
+    L.grf_gemm_workspace_bytes_split.argtypes = [u32, u32, u32, u32]
+    L.grf_gemm_workspace_bytes_split.restype = ctypes.c_size_t
     L.grf_bctx_gemm_noalloc.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, vp, u32, u32, vp, u32, vp, vp, vp]
     L.grf_bctx_gemm_noalloc.restype = i
     L.grf_gemm_noalloc_limit_bytes.argtypes = []

@@ -149,6 +149,16 @@ class PackedActivations:
         if status:
             raise base.CodecError(f"device launch failed ({status}): " + lib.grf_last_error().decode(errors="replace"))
 
+    def ensure(self, nbytes):
+        """Room behind the packed rows for a consumer whose launch is cut along K (its parts'
+        sums live in the same workspace): a larger buffer with the packed rows copied over."""
+        import torch
+        if self.buffer.numel() < nbytes:
+            larger = torch.empty(nbytes, device=self.buffer.device, dtype=torch.uint8)
+            larger[:self.buffer.numel()] = self.buffer
+            self.buffer = larger
+        return self.buffer
+
 
 class HipContextTensor:
     """A BCTX-coded BF16 matrix resident on one MI355X."""
@@ -395,9 +405,12 @@ class HipContextTensor:
         y = torch.empty((packed.rows, self.shape[0]), device=self.device, dtype=torch.bfloat16)
         if check:  # between checks the word keeps what earlier launches reported
             self.error.zero_()
-        self._launch(self._lib.grf_bctx_gemm, ctypes.byref(self.fused), ctypes.byref(self._gemm_tiling()[0]), None, 0,
+        tiling = self._gemm_tiling()[0]
+        space = packed.ensure(self._lib.grf_gemm_workspace_bytes_split(self.shape[1], self.shape[0], tiling.k_parts,
+                                                                       packed.rows))
+        self._launch(self._lib.grf_bctx_gemm, ctypes.byref(self.fused), ctypes.byref(tiling), None, 0,
                      packed.rows, y.data_ptr(), y.stride(0), bias.data_ptr() if bias is not None else None,
-                     packed.buffer.data_ptr(), packed.buffer.numel(), self.error.data_ptr())
+                     space.data_ptr(), space.numel(), self.error.data_ptr())
         self._check(check)
         return y.reshape(*packed.lead, self.shape[0])
 
@@ -409,8 +422,9 @@ class HipContextTensor:
             if check:  # between checks the word keeps what earlier launches reported
                 self.error.zero_()
             extra = ()
-            if workspace:  # transient: the activations in the matrix cores' operand order
-                size = self._lib.grf_gemm_workspace_bytes(self.shape[1], x2.shape[0])
+            if workspace:  # transient: the activations in the matrix cores' operand order (+ the parts' sums)
+                size = self._lib.grf_gemm_workspace_bytes_split(self.shape[1], self.shape[0], tiling.k_parts,
+                                                                x2.shape[0])
                 packed = torch.empty(size, device=self.device, dtype=torch.uint8)
                 extra = (packed.data_ptr(), size)
             self._launch(fn, ctypes.byref(self.fused), ctypes.byref(tiling), x2.data_ptr(), x2.stride(0),

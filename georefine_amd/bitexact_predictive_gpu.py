@@ -346,11 +346,11 @@ class HipPredictiveTensor:
                     extra = ()
                     if use_gemm:
                         fn, tiling = self._lib.grf_ppcx_gemm, self._tiling_for("gemm")[0]
+                        size = self._lib.grf_gemm_workspace_bytes_split(self.shape[1], self.shape[0], tiling.k_parts, m)
                         if packed is not None:
-                            space = packed.buffer
-                        else:  # transient: the activations in the matrix cores' operand order
-                            space = torch.empty(self._lib.grf_gemm_workspace_bytes(self.shape[1], m),
-                                                device=self.device, dtype=torch.uint8)
+                            space = packed.ensure(size)
+                        else:  # transient: the activations in the matrix cores' operand order (+ the parts' sums)
+                            space = torch.empty(size, device=self.device, dtype=torch.uint8)
                         extra = (space.data_ptr(), space.numel())
                     else:
                         fn = self._lib.grf_ppcx_gemv

@@ -41,6 +41,9 @@ uint32_t grf_bctx_gemm_lds_bytes(const grf_bctx_fused *frame, const grf_fused_ti
 }
 
 size_t grf_gemm_workspace_bytes(uint32_t cols, uint32_t m_rows) { return grf::gemm_workspace_bytes(cols, m_rows); }
+size_t grf_gemm_workspace_bytes_split(uint32_t cols, uint32_t rows, uint32_t k_parts, uint32_t m_rows) {
+  return grf::gemm_workspace_bytes_split(cols, rows, k_parts, m_rows);
+}
 
 int grf_pack_activations(const uint16_t *x, uint32_t ldx, uint32_t m_rows, uint32_t cols, void *workspace,
                          size_t workspace_bytes, void *hip_stream) {
@@ -65,11 +68,11 @@ int grf_bctx_gemm_noalloc(const grf_bctx_fused *frame, const grf_fused_tiling *t
                           void *hip_stream) {
   if (!frame || !tiling || !x || !y || !error)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_bctx_gemm_noalloc: null argument");
-  if (grf::gemm_workspace_bytes(frame->cols, m_rows) > kScratchBytes)
+  if (grf::gemm_workspace_bytes_split(frame->cols, frame->rows, tiling->k_parts, m_rows) > kScratchBytes)
     return grf::set_error(GRF_UNSUPPORTED,
-                          "grf_bctx_gemm_noalloc: the packed activations of one launch exceed the 8 MiB scratch "
-                          "(grf_gemm_workspace_bytes(cols, m_rows) > grf_gemm_noalloc_limit_bytes()); use grf_bctx_gemm "
-                          "with a workspace");
+                          "grf_bctx_gemm_noalloc: the packed activations (and partial sums) of one launch exceed the "
+                          "8 MiB scratch (grf_gemm_workspace_bytes_split(cols, rows, k_parts, m_rows) > "
+                          "grf_gemm_noalloc_limit_bytes()); use grf_bctx_gemm with a workspace");
   if (int rc = grf::check_fused_frame(*frame, *tiling, "grf_bctx_gemm_noalloc", grf::kGemmTiling)) return rc;
   void *ptr = nullptr;
   if (int rc = scratch_address(&ptr)) return rc;

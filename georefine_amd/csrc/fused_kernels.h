@@ -736,14 +736,25 @@ __device__ __forceinline__ void gemm_contract(float4v (&acc)[MT], const uint4 (&
 }
 
 // MT: 16-row activation tiles of this launch (m_rows <= 16 * MT, xp packed with m_pad = 16 * MT)
+// With g.k_parts > 1 the launch's tiles are k_parts copies of the row tiles, part-major: copy
+// `part` walks the slabs [part * spp, (part + 1) * spp) with spp = ceil(n_slabs / k_parts) and
+// leaves its sums as fp32 in `partials` [k_parts][m_rows][rows]; gemm_sum_parts_kernel adds the
+// parts in order, then the bias, and rounds.  That lets a matrix with few rows be cut along K
+// until its tiles fill the machine with full blocks of sixteen rows, in a fixed order of
+// additions (the tiling is the matrix's, whatever the batch).
 template <class Walk, int MT, int SCAN>
 __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fused &f, const grf_fused_tiling &g,
                                                 const uint4 *xp, uint32_t m_rows, uint16_t *y, uint32_t ldy,
-                                                const uint16_t *bias, int32_t *error, uint32_t tile) {
+                                                const uint16_t *bias, float *partials, int32_t *error,
+                                                uint32_t launch_tile) {
   const GemmLdsLayout L(f, g);
   const GemmShape shape(g);
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
+  const uint32_t parts = g.k_parts > 1 ? g.k_parts : 1u, row_tiles = g.n_tiles / parts;
+  const uint32_t part = launch_tile / row_tiles, tile = launch_tile - part * row_tiles;  // (uniform: scalar divisions)
+  const uint32_t per_part = (g.n_slabs + parts - 1) / parts;
+  const uint32_t b_first = part * per_part, b_past = min(g.n_slabs, b_first + per_part);
   const uint32_t cls = g.tile_class[tile];
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f), f.whole_range};
   constexpr uint32_t m_pad = MT * 16;
@@ -776,7 +787,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     g1 = grf::fused_index_entry(f.seg_offset, base + (any ? min(4u, min(P - quad * 4, f.segs_per_row - first)) : 0));
   };
   uint32_t g0, g1;
-  span_of(0, g0, g1);  // started before the table copy so that the latencies overlap
+  span_of(b_first, g0, g1);  // started before the table copy so that the latencies overlap
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
 
   float4v acc[MT];
@@ -786,7 +797,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   __syncthreads();  // the tables are in place
   const uint32_t later_half = blockIdx.x >= gridDim.x / 2 ? 1u : 0u;
 
-  for (uint32_t b = 0; b < g.n_slabs; ++b) {
+  for (uint32_t b = b_first; b < b_past; ++b) {
     const uint32_t first_seg = b * P + quad * 4;
     if (first_seg >= f.segs_per_row || quad * 4 >= P) break;  // uniform: this wave's quad has no segment from here on
     const uint32_t nseg = min(4u, min(P - quad * 4, f.segs_per_row - first_seg));
@@ -809,7 +820,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     // walking priority as in the GEMV: the slabs still to do, + 1 for the later-started half of
     // the grid (left alone, the older of the two workgroups on a compute unit runs ahead and
     // leaves the other the unit at half occupancy)
-    switch (min(3u, (g.n_slabs - 1 - b) + later_half)) {
+    switch (min(3u, (b_past - 1 - b) + later_half)) {
       case 0: __builtin_amdgcn_s_setprio(0); break;
       case 1: __builtin_amdgcn_s_setprio(1); break;
       case 2: __builtin_amdgcn_s_setprio(2); break;
@@ -880,6 +891,10 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
       // wave index of (quad, block) is quad * row_blocks + block
       float sum = sums[(blk * CT) * 256 + within];
       for (uint32_t qd = 1; qd < shape.quads; ++qd) sum += sums[((qd * shape.row_blocks + blk) * CT) * 256 + within];
+      if (parts > 1) {  // this part's share: the parts meet in gemm_sum_parts_kernel
+        partials[((size_t)part * m_rows + m) * f.rows + orow] = sum;
+        continue;
+      }
       if (bias) sum += __uint_as_float((uint32_t)bias[orow] << 16);
       y[(size_t)m * ldy + orow] = round_bf16(sum);
     }
@@ -891,9 +906,9 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
 template <class Walk, int MT, int SCAN>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_per_eu(6))) void fused_gemm_kernel(
     grf_bctx_fused f, grf_fused_tiling g, const uint4 *xp, uint32_t m_rows, uint16_t *y, uint32_t ldy,
-    const uint16_t *bias, int32_t *error) {
+    const uint16_t *bias, float *partials, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  fused_gemm_body<Walk, MT, SCAN>(lds, f, g, xp, m_rows, y, ldy, bias, error, blockIdx.x);
+  fused_gemm_body<Walk, MT, SCAN>(lds, f, g, xp, m_rows, y, ldy, bias, partials, error, blockIdx.x);
 }
 
 // Eight activation tiles: the accumulators and operands alone take 64 registers, so fewer
@@ -902,9 +917,9 @@ template <class Walk, int MT, int SCAN>
 __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_wide_kernel(grf_bctx_fused f, grf_fused_tiling g,
                                                                                  const uint4 *xp, uint32_t m_rows,
                                                                                  uint16_t *y, uint32_t ldy,
-                                                                                 const uint16_t *bias, int32_t *error) {
+                                                                                 const uint16_t *bias, float *partials, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
-  fused_gemm_body<Walk, MT, SCAN>(lds, f, g, xp, m_rows, y, ldy, bias, error, blockIdx.x);
+  fused_gemm_body<Walk, MT, SCAN>(lds, f, g, xp, m_rows, y, ldy, bias, partials, error, blockIdx.x);
 }
 
 template <class Walk, int MT, int SCAN>
@@ -912,8 +927,8 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) __attribute__((amdgpu_waves_
     FusedGroup a, const uint4 *xp, uint32_t m_rows, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t i = group_member(a, blockIdx.x);
-  fused_gemm_body<Walk, MT, SCAN>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], error,
-                            blockIdx.x - a.first_tile[i]);
+  fused_gemm_body<Walk, MT, SCAN>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], nullptr, error,
+                                  blockIdx.x - a.first_tile[i]);
 }
 
 template <class Walk, int MT, int SCAN>
@@ -921,13 +936,28 @@ __global__ __launch_bounds__(grf::kFusedMaxThreads) void fused_gemm_wide_group_k
                                                                                        uint32_t m_rows, int32_t *error) {
   extern __shared__ __align__(16) uint8_t lds[];
   const uint32_t i = group_member(a, blockIdx.x);
-  fused_gemm_body<Walk, MT, SCAN>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], error,
-                            blockIdx.x - a.first_tile[i]);
+  fused_gemm_body<Walk, MT, SCAN>(lds, a.f[i], a.g[i], xp, m_rows, a.y[i], a.ldy[i], a.bias[i], nullptr, error,
+                                  blockIdx.x - a.first_tile[i]);
+}
+
+// y[m][n] = bf16(partials[0][m][n] + partials[1][m][n] + ... + bias[n]): the parts of a
+// K-split launch, added in part order
+static __global__ __launch_bounds__(256) void gemm_sum_parts_kernel(const float *partials, uint32_t parts, uint32_t m_rows,
+                                                                    uint32_t rows, const uint16_t *bias, uint16_t *y,
+                                                                    uint32_t ldy) {
+  const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= m_rows * rows) return;
+  const uint32_t m = i / rows, n = i - m * rows;
+  float sum = partials[i];
+  for (uint32_t p = 1; p < parts; ++p) sum += partials[(size_t)p * m_rows * rows + i];
+  if (bias) sum += __uint_as_float((uint32_t)bias[n] << 16);
+  y[(size_t)m * ldy + n] = round_bf16(sum);
 }
 
 template <class Walk, int MT>
 int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
-                     uint16_t *y, uint32_t ldy, const uint16_t *bias, uint4 *xp, int32_t *error, hipStream_t s) {
+                     uint16_t *y, uint32_t ldy, const uint16_t *bias, uint4 *xp, float *partials, int32_t *error,
+                     hipStream_t s) {
   const GemmLdsLayout L(f, g);
   if (L.total > 160 * 1024) return grf::set_error(GRF_UNSUPPORTED, "fused GEMM: LDS demand exceeds 160 KiB");
   if (x) launch_pack(x, ldx, m_rows, f.cols, MT * 16, xp, s);  // else the caller packed these rows already
@@ -939,12 +969,16 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
     }();
     if (L.total > 64 * 1024)
       if (int rc = allow_full_lds<kernel>()) return rc;
-    hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, xp, m_rows, y, ldy, bias, error);
+    hipLaunchKernelGGL(kernel, dim3(g.n_tiles), dim3(g.threads), L.total, s, f, g, xp, m_rows, y, ldy, bias, partials,
+                       error);
     return GRF_OK;
   };
   if (int rc = f.whole_range ? launch(std::integral_constant<int, grf::kScanAny>{})
                              : launch(std::integral_constant<int, grf::kScanNoWholeRange>{}))
     return rc;
+  if (g.k_parts > 1)
+    hipLaunchKernelGGL(gemm_sum_parts_kernel, dim3((m_rows * f.rows + 255) / 256), dim3(256), 0, s, partials, g.k_parts,
+                       m_rows, f.rows, bias, y, ldy);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("fused GEMM: ") + hipGetErrorString(e));
   return GRF_OK;
@@ -954,6 +988,16 @@ int launch_gemm_rows(const grf_bctx_fused &f, const grf_fused_tiling &g, const u
 inline size_t gemm_workspace_bytes(uint32_t cols, uint32_t m_rows) {
   const uint32_t m = m_rows > kMaxRowsPerLaunch ? kMaxRowsPerLaunch : m_rows;
   return (size_t)(cols / 8 + 1) * gemm_tiles(m) * 16 * 16;
+}
+// ... and of the whole workspace of a launch cut into k_parts along K: the packed copy, then
+// (from the next multiple of 256) the parts' fp32 sums [k_parts][rows of the launch][rows]
+inline size_t gemm_partials_offset(uint32_t cols, uint32_t m_rows) {
+  return (gemm_workspace_bytes(cols, m_rows) + 255) / 256 * 256;
+}
+inline size_t gemm_workspace_bytes_split(uint32_t cols, uint32_t rows, uint32_t k_parts, uint32_t m_rows) {
+  if (k_parts <= 1) return gemm_workspace_bytes(cols, m_rows);
+  const uint32_t m = m_rows > kMaxRowsPerLaunch ? kMaxRowsPerLaunch : m_rows;
+  return gemm_partials_offset(cols, m_rows) + (size_t)k_parts * m * rows * 4;
 }
 
 // y = x W^T (+ bias) for any number of activation rows, 128 per launch.  `workspace` holds
@@ -973,18 +1017,24 @@ int launch_gemm(const char *who, const grf_bctx_fused &f, const grf_fused_tiling
   if (GemmShape(g).threads != g.threads || g.threads > (uint32_t)grf::kFusedMaxThreads)
     return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) +
                                                 ": tiling threads must be 64 x ceil(rows_per_tile / 16) x ceil(lanes_per_row / 4)");
-  if (!workspace || ((uintptr_t)workspace & 15) || workspace_bytes < gemm_workspace_bytes(f.cols, m_rows))
+  if (g.k_parts > 1 && (g.n_tiles % g.k_parts || g.k_parts > g.n_slabs))
+    return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": k_parts must divide n_tiles and be at most n_slabs");
+  if (!workspace || ((uintptr_t)workspace & 15) ||
+      workspace_bytes < gemm_workspace_bytes_split(f.cols, f.rows, g.k_parts, m_rows))
     return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": workspace missing, misaligned or too small");
   uint4 *xp = static_cast<uint4 *>(workspace);
+  float *partials = g.k_parts > 1 ? reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) +
+                                                              gemm_partials_offset(f.cols, m_rows))
+                                  : nullptr;
   for (uint32_t m0 = 0; m0 < m_rows; m0 += kMaxRowsPerLaunch) {
     const uint32_t m = m_rows - m0 < kMaxRowsPerLaunch ? m_rows - m0 : kMaxRowsPerLaunch;
     const uint16_t *xs = x ? x + (size_t)m0 * ldx : nullptr;
     uint16_t *ys = y + (size_t)m0 * ldy;
     int rc;
-    if (m <= 16) rc = launch_gemm_rows<Walk, 1>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
-    else if (m <= 32) rc = launch_gemm_rows<Walk, 2>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
-    else if (m <= 64) rc = launch_gemm_rows<Walk, 4>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
-    else rc = launch_gemm_rows<Walk, 8>(f, g, xs, ldx, m, ys, ldy, bias, xp, error, s);
+    if (m <= 16) rc = launch_gemm_rows<Walk, 1>(f, g, xs, ldx, m, ys, ldy, bias, xp, partials, error, s);
+    else if (m <= 32) rc = launch_gemm_rows<Walk, 2>(f, g, xs, ldx, m, ys, ldy, bias, xp, partials, error, s);
+    else if (m <= 64) rc = launch_gemm_rows<Walk, 4>(f, g, xs, ldx, m, ys, ldy, bias, xp, partials, error, s);
+    else rc = launch_gemm_rows<Walk, 8>(f, g, xs, ldx, m, ys, ldy, bias, xp, partials, error, s);
     if (rc) return rc;
   }
   return GRF_OK;
@@ -1032,6 +1082,7 @@ inline int build_group(const char *who, const GroupSpec &spec, bool gemm, FusedG
     if (f.cols != spec.frames[0]->cols) return bad("members must have one width");
     if (g.threads != spec.tilings[0]->threads) return bad("member tilings must share one thread count");
     if (g.scheme != spec.tilings[0]->scheme) return bad("member tilings must share one scheme");
+    if (g.k_parts > 1) return bad("grouped launches take tilings that are not cut along K (k_parts <= 1)");
     if (gemm && GemmShape(g).threads != g.threads)
       return bad("tiling threads must be 64 x ceil(rows_per_tile / 16) x ceil(lanes_per_row / 4)");
     if (spec.ldy[i] < f.rows) return bad("ldy is smaller than the row count");

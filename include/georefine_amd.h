@@ -217,6 +217,12 @@ typedef struct grf_bctx_fused {
  *               lanes_per_row segments for the whole launch and stages its own stream pieces
  *               (see grf_bctx_gemm for threads and piece_cap).
  *               Wave tilings take matrices with fewer than 2^24 rows and 2^24 columns.
+ *   k_parts     0 or 1: every tile walks all slabs.  k > 1 (grf_bctx_gemm / grf_ppcx_gemm only):
+ *               the launch is cut along K: tile_rows / tile_class describe n_tiles / k row
+ *               tiles, which must hold every row of the matrix once; launch tile t is row tile
+ *               t mod (n_tiles / k), part t / (n_tiles / k), and walks the slabs [part * s,
+ *               (part + 1) * s), s = ceil(n_slabs / k).  The parts' sums are added in part order
+ *               by a second kernel, in the workspace (grf_gemm_workspace_bytes_split).
  * n_slabs = ceil(segs_per_row / lanes_per_row) in both schemes. */
 #define GRF_TILE_SLABS 0
 #define GRF_TILE_WAVES 1
@@ -227,6 +233,7 @@ typedef struct grf_fused_tiling {
   uint32_t lanes_per_row, rows_per_tile, n_slabs, n_tiles;
   uint32_t piece_cap;
   uint32_t scheme;
+  uint32_t k_parts;
 } grf_fused_tiling;
 
 /* Fused decode-GEMV, the slot the reference leaves for "a backend with a fused GEMM"
@@ -266,21 +273,28 @@ int grf_bctx_fused_gather(const grf_bctx_fused *frame, const grf_fused_tiling *t
  * stream piece of four consecutive segments of a row (from its 16-byte aligned start, + 8):
  * a wave walks four lane-segments of 16 rows and feeds the words it decodes to the matrix
  * cores from its registers.  workspace: device memory, 16-byte
- * aligned, at least grf_gemm_workspace_bytes(cols, m_rows) bytes; each launch first writes
+ * aligned, at least grf_gemm_workspace_bytes(cols, m_rows) bytes (grf_gemm_workspace_bytes_split
+ * for a tiling with k_parts > 1); each launch first writes
  * its activation rows there in operand order (a copy of x: cols * 32 + 256 bytes per 16 rows),
  * so calls that share a workspace must be ordered on one stream. */
 int grf_bctx_gemm(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, const uint16_t *x, uint32_t ldx,
                   uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
                   size_t workspace_bytes, int32_t *error, void *hip_stream);
 size_t grf_gemm_workspace_bytes(uint32_t cols, uint32_t m_rows);
+/* The workspace of a launch with a tiling cut into k_parts along K: the packed activations,
+ * then (from the next multiple of 256 bytes) the parts' fp32 sums [k_parts][min(m_rows, 128)][rows].
+ * Equal to grf_gemm_workspace_bytes for k_parts <= 1.  With x == NULL the caller has packed
+ * the rows into the front of a workspace of this size. */
+size_t grf_gemm_workspace_bytes_split(uint32_t cols, uint32_t rows, uint32_t k_parts, uint32_t m_rows);
 
 /* grf_bctx_gemm without the workspace argument, for callers that cannot allocate device
  * memory (code under HIP graph capture, tight serving loops, harnesses that forbid it).  No
  * counterpart in the reference.  The packed activations go to an 8 MiB array that is part of
  * the library's device image (every GPU the library runs on holds its copy until the process
  * ends); the call allocates and frees nothing.  It fails with GRF_UNSUPPORTED when
- * grf_gemm_workspace_bytes(cols, min(m_rows, 128)) exceeds grf_gemm_noalloc_limit_bytes()
- * (128 rows: matrices up to 32 752 columns; 64 rows: twice that).  x must not be NULL.  All
+ * grf_gemm_workspace_bytes_split(cols, rows, k_parts, min(m_rows, 128)) exceeds
+ * grf_gemm_noalloc_limit_bytes() (a tiling that is not cut along K, 128 rows: matrices up to
+ * 32 752 columns; 64 rows: twice that).  x must not be NULL.  All
  * calls on one GPU share the array: calls that overlap on one GPU (two streams, two threads)
  * race; calls on one stream are ordered.  Results are those of grf_bctx_gemm, bit for bit. */
 int grf_bctx_gemm_noalloc(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, const uint16_t *x, uint32_t ldx,

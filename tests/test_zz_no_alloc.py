@@ -32,7 +32,7 @@ def test_noalloc_gemm_matches_the_workspace_entry_point_twice():
     for rows in (96, 17):  # the second call is smaller: rows of the first must not show through
         print(f"rows={rows}", flush=True)
         x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(rows, 1280)))).view(torch.bfloat16).cuda()
-        size = lib.grf_gemm_workspace_bytes(1280, rows)
+        size = lib.grf_gemm_workspace_bytes_split(1280, t.shape[0], t._gemm_tiling()[0].k_parts, rows)
         workspace = torch.empty(size, device="cuda:0", dtype=torch.uint8)
         want, got = (torch.zeros((rows, t.shape[0]), device="cuda:0", dtype=torch.bfloat16) for _ in range(2))
         status, _ = _call(t, lib, x, want, lib.grf_bctx_gemm, workspace.data_ptr(), size)
