@@ -113,3 +113,60 @@ def test_packed_activations_serve_several_matrices(oracle):
     with pytest.raises(ValueError):
         narrow.gemm(packed)
 
+
+
+@pytest.mark.parametrize("shape,forced", [((96, 2176), "8,32,4"), ((200, 1280), "4,48,5"), ((64, 4096), "16,16,3"),
+                                          ((320, 17408), "24,32,3")],
+                         ids=lambda v: v if isinstance(v, str) else f"{v[0]}x{v[1]}")
+def test_gemm_cut_along_k(oracle, monkeypatch, shape, forced):
+    """A launch cut into k parts along K (every row tile k times, each copy a k-th of the slabs,
+    the parts added in order by a second kernel): right against float64, rows independent of the
+    batch and of packing, bias applied once, the same matrix uncut within rounding of it; the C
+    entry point refuses a workspace sized for an uncut launch."""
+    import ctypes
+    import torch
+    from georefine_amd import _fused
+    from georefine_amd.bitexact_context_gpu import PackedActivations
+    rng = np.random.default_rng(shape[0] * 3 + shape[1])
+    words = weight_like(rng, *shape)
+    monkeypatch.setattr(_fused, "GEMM_SPLIT", False)  # tilings are planned when a tensor is bound
+    frame, plain = _tensor(words)
+    assert plain._gemm_tiling()[0].k_parts <= 1
+    monkeypatch.setattr(_fused, "GEMM_SPLIT", True)
+    monkeypatch.setenv("GEOREFINE_FUSED_GEMM_TILING", forced)
+    t = plain.clone()
+    tiling = t._gemm_tiling()[0]
+    print("gemm tiling", t._gemm_tiling()[3], flush=True)
+    assert tiling.k_parts == int(forced.split(",")[2]) and tiling.n_tiles % tiling.k_parts == 0
+    monkeypatch.delenv("GEOREFINE_FUSED_GEMM_TILING")
+    w64 = words_to_float(oracle.bctx_decode(frame)).astype(np.float64)
+    xw = bf16_words(rng.normal(0, 1, size=(140, shape[1])))
+    x = torch.from_numpy(xw).view(torch.bfloat16).cuda()
+    bias = torch.from_numpy(bf16_words(rng.normal(0, 1, size=shape[0]))).view(torch.bfloat16).cuda()
+    xf = words_to_float(xw).astype(np.float64)
+    ref = xf @ w64.T + words_to_float(bias.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    scale = np.abs(xf) @ np.abs(w64).T + 1.0
+    y_all = t.gemm(x, bias, check=True)
+    got = words_to_float(y_all.view(torch.uint16).cpu().numpy()).astype(np.float64)
+    assert np.all(np.abs(got - ref) <= 1e-2 * np.maximum(np.abs(ref), 1e-3 * scale) + 1e-30)
+    for m in (1, 16, 17, 64, 128, 129):
+        assert torch.equal(t.gemm(x[:m], bias, check=True).view(torch.uint16), y_all[:m].view(torch.uint16)), m
+    packed = PackedActivations(x[:40])
+    assert torch.equal(t.gemm(packed, bias, check=True).view(torch.uint16), y_all[:40].view(torch.uint16))
+    uncut = words_to_float(plain.gemm(x, bias, check=True).view(torch.uint16).cpu().numpy()).astype(np.float64)
+    assert np.all(np.abs(got - uncut) <= 1e-2 * np.maximum(np.abs(ref), 1e-3 * scale) + 1e-30)
+    # the C entry point wants room for the parts' sums
+    lib = t._lib
+    small = lib.grf_gemm_workspace_bytes(shape[1], 64)
+    need = lib.grf_gemm_workspace_bytes_split(shape[1], shape[0], tiling.k_parts, 64)
+    assert need >= small + tiling.k_parts * 64 * shape[0] * 4
+    space = torch.empty(need, device="cuda:0", dtype=torch.uint8)
+    y = torch.empty((64, shape[0]), device="cuda:0", dtype=torch.bfloat16)
+    args = (ctypes.byref(t.fused), ctypes.byref(tiling), x.data_ptr(), x.stride(0), 64, y.data_ptr(), y.stride(0),
+            bias.data_ptr())
+    stream = torch.cuda.current_stream().cuda_stream
+    assert lib.grf_bctx_gemm(*args, space.data_ptr(), small, t.error.data_ptr(), stream) != 0
+    assert b"workspace" in lib.grf_last_error()
+    assert lib.grf_bctx_gemm(*args, space.data_ptr(), need, t.error.data_ptr(), stream) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(y.view(torch.uint16), y_all[:64].view(torch.uint16))
