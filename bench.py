@@ -72,10 +72,12 @@ def algorithmic_bytes(t, m):
     b = t.buffers
     n = lambda k: b[k].numel() * b[k].element_size()
     rows, cols = t.shape
-    payload = t._main_bytes + n("residual_stream")
+    # (the resident residual array starts every row class on a multiple of 16 rows: the rows it
+    # holds beyond the matrix's are never read and are not counted)
+    payload = t._main_bytes + min(n("residual_stream"), rows * cols * 3 // 4)
     _, tile_rows, tile_class, _ = t._tiling(m) if m <= GEMV_UP_TO else t._gemm_tiling()
     index = (n("fused_seg_state") + n("fused_seg_offset") + tile_rows.numel() * tile_rows.element_size()
-             + tile_class.numel() * tile_class.element_size())
+             + tile_class.numel() * tile_class.element_size() + (n("row_pos") if "row_pos" in b else 0))
     tables = n("fused_lut") + n("fused_tab")
     labels = cols
     io = m * cols * 2 + m * rows * 2

@@ -111,7 +111,7 @@ def lds_bytes_waves(nc, lognb, tabn, m, threads, p, r, n_slabs, piece_cap):
     total = a16(nc * (a16((tabn + 1) * 8) + (1 << lognb)))
     total = a16(total + threads // 64 * (64 // p) * piece_cap)
     total = a16(total + r * n_slabs * m * 4)
-    total = a16(total + r * 4)
+    total = a16(total + r * 8)
     return total
 
 
@@ -273,7 +273,7 @@ def choose_wave_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=6
         cap = piece_cap_fn(p)
         for threads in (1024, 768, 512):
             nwaves = threads // 64
-            for r in range(rpw, 129):
+            for r in range(rpw, 129, rpw):  # whole units: their rows are then the blocks of the residual order
                 groups = -(-r // rpw)
                 lds = lds_fn(threads, p, r, n_slabs, cap)
                 if lds > MAX_LDS:
@@ -351,6 +351,20 @@ def choose_gemm_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=6
     return best[1:]
 
 
+def order_residuals(raw, rows, cols, seg_len, block, position, held):
+    """The packed 6-bit residuals of a frame (12-byte groups of 16 fields, frame order) in the
+    order the tile walker reads them: rows at their positions, in blocks of ``block`` rows;
+    inside a block by position in the segment, then by segment, then by row -- group t of
+    segment s of position q at (((q // block * G + t) * spr + s) * block + q % block) * 12 with
+    G = seg_len // 16.  A permutation of groups (no field is touched); positions that no row
+    has hold zeros."""
+    spr, groups = cols // seg_len, seg_len // 16
+    ordered = np.zeros((held, groups, spr, 12), dtype=np.uint8)
+    ordered[position] = np.asarray(raw).reshape(rows, spr, groups, 12).transpose(0, 2, 1, 3)
+    ordered = ordered.reshape(held // block, block, groups, spr, 12).transpose(0, 2, 3, 1, 4)
+    return np.ascontiguousarray(ordered).reshape(-1)
+
+
 def build_tiles(row_class, nr, r):
     """Rows grouped by class (index order inside a class), cut into tiles of r rows."""
     order = np.argsort(row_class, kind="stable").astype(np.uint32)
@@ -391,6 +405,25 @@ class FramePlan:
         self.row_class = np.asarray(row_class)
         self.class_rows = np.bincount(self.row_class, minlength=nr)
         self._caps = {}
+
+    def residual_order(self):
+        """(block rows B, row positions u32[rows], rows of the array) of the resident residual
+        order: the rows by class, index order inside a class, as every tiling takes them, each
+        class starting on a multiple of 16; B = the rows of a wave unit of the GEMV (1 where
+        the GEMV has no wave tiling), so that a unit's rows are the rows of one block."""
+        try:
+            block = 64 // self.tiling(1, waves=True)["scalars"]["lanes_per_row"]
+        except FusedUnsupported:
+            block = 1
+        order = np.argsort(self.row_class, kind="stable")
+        starts = np.zeros(self.nr + 1, dtype=np.int64)
+        for rho in range(self.nr):
+            starts[rho + 1] = (starts[rho] + int(self.class_rows[rho]) + 15) // 16 * 16
+        first = np.concatenate(([0], np.cumsum(self.class_rows)[:-1]))  # of each class, in `order`
+        sorted_class = self.row_class[order]
+        position = np.empty(self.rows, dtype=np.uint32)
+        position[order] = (starts[sorted_class] + np.arange(self.rows) - first[sorted_class]).astype(np.uint32)
+        return block, position, int(starts[-1])
 
     def table_bytes(self):
         """LDS bytes of one row class's lookup tables (what every workgroup copies first)."""

@@ -14,9 +14,9 @@ class GrfStream(ctypes.Structure):
 
 class GrfBctxFrame(ctypes.Structure):
     _fields_ = [("main", GrfStream), ("residual", GrfStream), ("row_class", ctypes.c_void_p),
-                ("col_class", ctypes.c_void_p), ("rows", ctypes.c_uint32), ("cols", ctypes.c_uint32),
-                ("nc", ctypes.c_uint32), ("mode", ctypes.c_uint32), ("stride", ctypes.c_uint32),
-                ("raw6_segment", ctypes.c_uint32)]
+                ("col_class", ctypes.c_void_p), ("raw6_row_pos", ctypes.c_void_p), ("rows", ctypes.c_uint32),
+                ("cols", ctypes.c_uint32), ("nc", ctypes.c_uint32), ("mode", ctypes.c_uint32),
+                ("stride", ctypes.c_uint32), ("raw6_segment", ctypes.c_uint32), ("raw6_block_rows", ctypes.c_uint32)]
 
 
 class GrfPpcxFrame(ctypes.Structure):
@@ -28,7 +28,7 @@ class GrfPpcxFrame(ctypes.Structure):
 class GrfBctxFused(ctypes.Structure):
     _fields_ = [("main_bytes", ctypes.c_void_p), ("raw6", ctypes.c_void_p), ("seg_state", ctypes.c_void_p),
                 ("seg_offset", ctypes.c_void_p), ("lut", ctypes.c_void_p), ("tab", ctypes.c_void_p),
-                ("col_class", ctypes.c_void_p)] + [
+                ("col_class", ctypes.c_void_p), ("row_pos", ctypes.c_void_p)] + [
         (name, ctypes.c_uint32) for name in (
             "main_n_bytes", "rows", "cols", "nr", "nc", "seg_len", "segs_per_row", "shift", "lognb", "tabn",
             "raw_interleaved", "whole_range")]

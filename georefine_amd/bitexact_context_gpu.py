@@ -203,21 +203,24 @@ class HipContextTensor:
                 indexed.pop("fused_states", None)
                 indexed.pop("fused_offsets", None)
         self._main_bytes = len(indexed["main_stream"]) if "main_stream" in indexed else 0
-        self._raw6_segment = 0
+        self._raw6_segment, self._raw6_block = 0, 0
         if plan is not None:  # the fused kernels read 16-byte vectors: pad the stream's allocation
             indexed["main_stream"] = np.concatenate((indexed["main_stream"], np.zeros(16, dtype=np.uint8)))
-            # The packed residuals in the order the tile walker reads them: a row's 12-byte groups
-            # of 16 fields by position in the segment first, then by segment (a permutation of
-            # groups, no field is touched).  Lanes of a row walk neighbouring segments in step,
-            # so they then read neighbouring bytes and a 128-byte line is used in one visit; in
-            # the frame's order a line came back from memory about twice per launch.
+            # The packed residuals in the order the tile walker reads them (a permutation of the
+            # 12-byte groups of 16 fields, no field is touched): rows by class as the tilings take
+            # them, in blocks of as many rows as a wave unit of the GEMV has; inside a block by
+            # position in the segment, then by segment, then by row.  The lanes of a unit walk
+            # neighbouring segments of the block's rows in step, so they read one run of bytes per
+            # visit and a 128-byte line is used in a single visit; in the frame's order a line came
+            # back from memory about twice per launch.
             rows_, cols_ = self.shape
             seg = indexed["fused_segment"]
             raw = indexed["residual_stream"]
             if raw.size == rows_ * cols_ * 3 // 4:
-                groups = raw.reshape(rows_, cols_ // seg, seg // 16, 12)
-                indexed["residual_stream"] = np.ascontiguousarray(groups.transpose(0, 2, 1, 3)).reshape(-1)
-                self._raw6_segment = seg
+                block, position, held = plan.residual_order()
+                indexed["residual_stream"] = _fused.order_residuals(raw, rows_, cols_, seg, block, position, held)
+                indexed["row_pos"] = position
+                self._raw6_segment, self._raw6_block = seg, block
             indexed.update(fused_seg_state=plan.seg_state, fused_seg_offset=plan.seg_offset, fused_lut=plan.lut,
                            fused_tab=plan.tab)
         for name, array in indexed.items():
@@ -247,7 +250,8 @@ class HipContextTensor:
             f.col_class = self.buffers["columns"].data_ptr()
             f.rows, f.cols = self.shape
             f.nc, f.mode, f.stride = self.nc, self.resident_mode, self.stride
-            f.raw6_segment = self._raw6_segment
+            f.raw6_segment, f.raw6_block_rows = self._raw6_segment, self._raw6_block
+            f.raw6_row_pos = self.buffers["row_pos"].data_ptr() if self._raw6_segment else None
             f.main.n_bytes = self._main_bytes
             self._frame = f
         self._tilings = {}
@@ -259,7 +263,8 @@ class HipContextTensor:
             d.seg_state, d.seg_offset = b["fused_seg_state"].data_ptr(), b["fused_seg_offset"].data_ptr()
             d.lut, d.tab, d.col_class = b["fused_lut"].data_ptr(), b["fused_tab"].data_ptr(), b["columns"].data_ptr()
             d.main_n_bytes = self._main_bytes
-            d.raw_interleaved = 1 if self._raw6_segment else 0
+            d.raw_interleaved = self._raw6_block if self._raw6_segment else 0
+            d.row_pos = b["row_pos"].data_ptr() if self._raw6_segment else None
             for key, value in plan.scalars().items():
                 setattr(d, key, value)
             self.fused = d

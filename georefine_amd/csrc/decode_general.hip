@@ -26,12 +26,13 @@ constexpr int kThreads = 256;
 
 // MODE128: residual is a second rANS stream whose context is the main symbol.
 // Index of element (row, col) among the packed 6-bit fields: the frame's own order, or, for
-// a tensor that keeps them for the fused kernels, groups of 16 ordered by their position in
-// the segment before the segment's number.
+// a tensor that keeps them for the fused kernels, groups of 16 in blocks of rows, ordered by
+// their position in the segment, the segment's number and the row inside the block.
 __device__ __forceinline__ uint64_t raw6_index(const grf_bctx_frame &f, uint32_t row, uint32_t col) {
   if (!f.raw6_segment) return (uint64_t)row * f.cols + col;
-  const uint32_t S = f.raw6_segment, spr = f.cols / S;
-  const uint64_t group = ((uint64_t)row * (S / 16) + (col % S) / 16) * spr + col / S;
+  const uint32_t S = f.raw6_segment, spr = f.cols / S, B = f.raw6_block_rows ? f.raw6_block_rows : 1;
+  const uint32_t q = f.raw6_row_pos ? f.raw6_row_pos[row] : row, within = q % B;
+  const uint64_t group = (uint64_t)(q - within) * (f.cols / 16) + ((uint64_t)((col % S) / 16) * spr + col / S) * B + within;
   return group * 16 + col % 16;
 }
 
@@ -179,7 +180,7 @@ int launch_status(const char *what) {
 extern "C" {
 
 const char *grf_last_error(void) { return grf::g_error.c_str(); }
-int grf_abi_version(void) { return 1; }
+int grf_abi_version(void) { return 2; }
 
 int grf_bctx_decode(const grf_bctx_frame *frame, const int64_t *block_ids, uint32_t count, uint16_t *out,
                     int32_t *error, void *hip_stream) {
@@ -191,8 +192,13 @@ int grf_bctx_decode(const grf_bctx_frame *frame, const int64_t *block_ids, uint3
   if (!stream_ok(f.main, true) || !stream_ok(f.residual, f.mode == 128))
     return fail(GRF_BAD_ARGUMENT, "grf_bctx_decode: incomplete stream descriptor");
   const uint64_t n = (uint64_t)f.rows * f.cols;
-  if (f.mode == 0 && f.residual.n_bytes != (n * 6 + 7) / 8)
+  // (in the fused kernels' order the array may hold rows beyond the matrix's: positions no row has)
+  if (f.mode == 0 && (f.raw6_segment ? f.residual.n_bytes < (n * 6 + 7) / 8 : f.residual.n_bytes != (n * 6 + 7) / 8))
     return fail(GRF_BAD_ARGUMENT, "grf_bctx_decode: packed residual length mismatch");
+  if (f.mode == 0 && f.raw6_segment &&
+      (f.raw6_segment % 16 || f.cols % f.raw6_segment || f.raw6_block_rows > 16 ||
+       (f.raw6_block_rows & (f.raw6_block_rows - 1))))
+    return fail(GRF_BAD_ARGUMENT, "grf_bctx_decode: residual order (segment length, block rows)");
   const uint64_t segments = (n + f.stride - 1) / f.stride;
   if (!count) return GRF_OK;
   if (!block_ids && count > segments) return fail(GRF_BAD_ARGUMENT, "grf_bctx_decode: count exceeds segments");

@@ -433,11 +433,12 @@ struct SegmentWalkT {
   uint32_t cw[4];
 
   // Global reads for segment `seg_` (elem0 / col0: its first element / column; seg_in_row =
-  // col0 / seg_len, which the caller has without dividing), issued before the wait for the
-  // stream bytes so that their latency overlaps it.
+  // col0 / seg_len, which the caller has without dividing; rpos: the row's position in the
+  // residual array, f.row_pos[row] or the row itself), issued before the wait for the stream
+  // bytes so that their latency overlaps it.
   // (A matrix has fewer than 2^32 elements, so element and byte offsets are 32-bit numbers.)
   __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t col0,
-                                           uint32_t seg_in_row) {
+                                           uint32_t seg_in_row, uint32_t rpos) {
     gofs = fused_index_entry(f.seg_offset, seg_);
     eofs = fused_index_entry(f.seg_offset, seg_ + 1);
     c.state = fused_index_entry(f.seg_state, seg_);
@@ -446,10 +447,14 @@ struct SegmentWalkT {
     // pair and one vector register, and no 64-bit address is worked out per group
     raw_base = f.raw6;
     cc_base = f.col_class;
-    if (f.raw_interleaved) {  // a row's groups ordered by position in the segment, then by segment
-      const uint32_t group = (elem0 - col0) / 16 + seg_in_row;
-      raw_off = ((group << 1) + group) << 2;  // * 12 without the quarter-rate 32-bit multiply
-      raw_stride = f.segs_per_row * 12;
+    if (f.raw_interleaved) {
+      // blocks of B rows (by position); inside a block the groups by position in the segment,
+      // then by segment, then by row: group t of segment s of position q at
+      // ((q / B * G + t) * segs_per_row + s) * B + q % B, G = seg_len / 16 groups per segment
+      const uint32_t B = f.raw_interleaved, within = rpos & (B - 1);
+      const uint32_t group = (rpos - within) * (f.cols / 16) + seg_in_row * B + within;  // (once per segment)
+      raw_off = ((group << 1) + group) << 2;  // * 12
+      raw_stride = f.segs_per_row * B * 12;
     } else {
       raw_off = elem0 / 4 * 3;
       raw_stride = 12;

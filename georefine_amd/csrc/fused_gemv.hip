@@ -33,6 +33,9 @@ int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const 
   if (f.tabn == 0 || f.tabn > 255) return bad("sparse table size");
   if (g.piece_cap % 16 || g.piece_cap < 16) return bad("piece capacity");
   if ((uint64_t)f.rows * f.cols > 0xFFFFFFFFull) return bad("matrix too large");
+  if (f.raw_interleaved > 16 || (f.raw_interleaved & (f.raw_interleaved - 1)))
+    return bad("raw_interleaved is 0 or a block of 1, 2, 4, 8 or 16 rows");
+  if (f.row_pos && !f.raw_interleaved) return bad("row positions belong to the interleaved residual order");
   return GRF_OK;
 }
 }  // namespace grf

@@ -88,6 +88,11 @@ struct ahead_of<grf::SegmentWalk> { using type = grf::SegmentWalkAhead; };
 constexpr uint32_t kAheadMaxRows = 4;
 // a segment's residuals are 48 bytes, read as three 16-byte vectors
 // (a segment's 48 residual bytes are contiguous only in the frame's own order)
+// Position of a row in the residual array (grf_bctx_fused.row_pos; the row itself without one).
+__device__ __forceinline__ uint32_t row_position(const grf_bctx_fused &f, uint32_t row) {
+  return f.row_pos && row != grf::kNoRow ? f.row_pos[row] : row;
+}
+
 inline bool reads_ahead(const grf_bctx_fused &f) { return f.seg_len == 64 && !f.raw_interleaved && !((uintptr_t)f.raw6 & 15); }
 
 // One workgroup's walk over tile `tile` of a frame.
@@ -105,6 +110,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
   const uint32_t r = tid / P, p = tid % P;
   uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
   if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
+  const uint32_t rpos = row_position(f, row);
   uint16_t *xs = reinterpret_cast<uint16_t *>(lds + L.xs);
   const uint32_t xpitch = S + grf::kXPad;
   const uint32_t width = P * S;
@@ -138,7 +144,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
     const uint64_t elem0 = (uint64_t)row * K + col0;
     Walk w;
     uint32_t a0 = 0;
-    if (walks) w.prefetch(f, seg_base + p, (uint32_t)elem0, col0, first_seg + p);
+    if (walks) w.prefetch(f, seg_base + p, (uint32_t)elem0, col0, first_seg + p, rpos);
     if (row != grf::kNoRow) {
       a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
       if (b + 1 < g.n_slabs)  // the next slab's byte range, while this one is walked
@@ -249,8 +255,8 @@ struct WaveLdsLayout {
     block_pitch = grf::fused_table_bytes(f) + (1u << f.lognb);
     stream = grf::align_up(f.nc * block_pitch, 16);                   // [waves][64 / P] row pieces
     sub = grf::align_up(stream + waves * rpw * g.piece_cap, 16);      // [rows_per_tile][n_slabs][m] unit sums
-    rows = grf::align_up(sub + g.rows_per_tile * g.n_slabs * m * 4, 16);  // [rows_per_tile] the tile's rows
-    total = grf::align_up(rows + g.rows_per_tile * 4, 16);
+    rows = grf::align_up(sub + g.rows_per_tile * g.n_slabs * m * 4, 16);  // [2][rows_per_tile] the tile's rows, their positions
+    total = grf::align_up(rows + g.rows_per_tile * 8, 16);
   }
 };
 
@@ -337,16 +343,19 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     if (b >= g.n_slabs) b -= g.n_slabs, ++grp;
   };
   uint32_t grp = wave / g.n_slabs, b = wave % g.n_slabs;  // this wave's first unit
-  uint32_t row, g0, g1;
+  uint32_t row, rpos, g0, g1;
   {
     const uint32_t slot0 = grp * rpw + rl;
     row = (wave < units && slot0 < R) ? g.tile_rows[tile * R + slot0] : grf::kNoRow;
     if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
     span_of(b, row, g0, g1);
+    rpos = row_position(f, row);
   }
   for (uint32_t i = tid; i < R; i += nthreads) {
-    const uint32_t rw = g.tile_rows[tile * R + i];
-    rows[i] = rw < f.rows ? rw : grf::kNoRow;
+    uint32_t rw = g.tile_rows[tile * R + i];
+    if (rw >= f.rows) rw = grf::kNoRow;
+    rows[i] = rw;
+    rows[R + i] = row_position(f, rw);
   }
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   __syncthreads();
@@ -366,7 +375,10 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     const uint32_t slot = grp * rpw + rl;
     const uint32_t first_seg = b << logp;
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
-    if (u != wave) row = slot < R ? rows[slot] : grf::kNoRow;  // (read again: cheaper than a register over the walk)
+    if (u != wave) {  // (read again: cheaper than registers over the walk)
+      row = slot < R ? rows[slot] : grf::kNoRow;
+      rpos = slot < R ? rows[R + slot] : 0;
+    }
     const bool walks = row != grf::kNoRow && p < nseg;
     const uint32_t col0 = mul24(first_seg + p, S);
     // The copy of the pieces goes first: its byte ranges arrived during the walk before, while
@@ -375,7 +387,7 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     Walk w;
     {  // every lane loads (see span_of); lanes that do not walk read segment 0's entries
       const uint32_t seg = walks ? mul24(row, f.segs_per_row) + first_seg + p : 0;
-      w.prefetch(f, seg, walks ? mul24(row, K) + col0 : 0, walks ? col0 : 0, walks ? first_seg + p : 0);
+      w.prefetch(f, seg, walks ? mul24(row, K) + col0 : 0, walks ? col0 : 0, walks ? first_seg + p : 0, walks ? rpos : 0);
     }
     if (walks) w.start(piece_off, a0);
     const uint32_t slot_base = grp * rpw, slab = b;  // this unit's, kept while the counters move on
@@ -769,6 +781,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   const uint32_t r = rb * 16 + lane % 16, p4 = lane / 16;
   uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
   if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
+  const uint32_t rpos = row_position(f, row);
 
   // A wave keeps its sixteen rows and its quad of lane-segments for the whole launch and goes
   // through the slabs on its own: in slab b it walks segments b * P + 4 * quad .. + 3 of every
@@ -811,7 +824,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     Walk w;
     {
       const uint32_t seg = active ? mul24(row, f.segs_per_row) + first_seg + p4 : 0;
-      w.prefetch(f, seg, active ? mul24(row, K) + col0 : 0, active ? col0 : 0, active ? first_seg + p4 : 0);
+      w.prefetch(f, seg, active ? mul24(row, K) + col0 : 0, active ? col0 : 0, active ? first_seg + p4 : 0, active ? rpos : 0);
     }
     if (active) w.start(piece_off, a0);  // (a0: of the lane's own row, which its four lanes share)
     span_of(b + 1, g0, g1);  // the next slab's byte range, on its way during this walk

@@ -115,7 +115,7 @@ struct PpcxWalk {
     return reinterpret_cast<const uint32_t *>(rawp + ((10 * g) & ~3u));
   }
   // global reads of the segment, issued before the wait for the slab's stream bytes
-  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t, uint32_t) {
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t, uint32_t, uint32_t) {
     gofs = grf::fused_index_entry(f.seg_offset, seg_);
     eofs = grf::fused_index_entry(f.seg_offset, seg_ + 1);
     c.state = grf::fused_index_entry(f.seg_state, seg_);

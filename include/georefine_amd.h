@@ -112,17 +112,20 @@ typedef struct grf_stream {
  * stream and the other residual fields are unused; mode 128: residual is a full stream.
  * raw6_segment (mode 0): 0 when the 6-bit fields are in the frame's own order (element e at
  * bit 6 e); S > 0 when the 12-byte groups of 16 fields are kept in the order the fused
- * kernels read them (see grf_bctx_fused.raw_interleaved) for segments of S symbols. */
+ * kernels read them for segments of S symbols: raw6_block_rows and raw6_row_pos are then
+ * grf_bctx_fused.raw_interleaved and grf_bctx_fused.row_pos of the same tensor. */
 typedef struct grf_bctx_frame {
   grf_stream main;
   grf_stream residual;
   const uint8_t *row_class;
   const uint8_t *col_class;
+  const uint32_t *raw6_row_pos;
   uint32_t rows, cols;
   uint32_t nc;
   uint32_t mode;
   uint32_t stride;
   uint32_t raw6_segment;
+  uint32_t raw6_block_rows;
 } grf_bctx_frame;
 
 /* Replaces the Triton launch of decode_words (GCR/bitexact_context_gpu.py:149-150,
@@ -171,10 +174,16 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  *                                            high32 = symbol<<5; unused entries: 0
  *   col_class   u8  [cols]
  * raw_interleaved: 0 = raw6 in the frame's order (the 12-byte group g of row r at
- * (r * cols / 16 + g) * 12); 1 = a row's groups ordered by position in the segment first:
- * group t of segment s of row r at ((r * seg_len / 16 + t) * segs_per_row + s) * 12, so that
- * the lanes of a row, which are at the same position of neighbouring segments, read
- * neighbouring bytes and every 128-byte line is used in one visit.
+ * (r * cols / 16 + g) * 12); B = 1, 2, 4, 8 or 16 = in blocks of B rows, and inside a block
+ * by position in the segment first, then by segment, then by row: with q the row's position
+ * (row_pos[r], or r itself when row_pos is null) and G = seg_len / 16, group t of segment s
+ * lies at (((q / B * G + t) * segs_per_row + s) * B + q % B) * 12.  The lanes of a wave unit
+ * of the GEMV (B = 64 / lanes_per_row rows, at the same position of neighbouring segments)
+ * then read one run of 768 bytes per visit, and every 128-byte line is used in a single visit.
+ * row_pos: u32 [rows], a one-to-one map of the rows to positions below
+ * ceil(max position / B) * B (the array holds that many rows; positions no row has are never
+ * read).  The host side orders the rows by row class, as the tilings do, and starts every
+ * class on a multiple of 16, so that the rows of a unit are the rows of a block.
  * whole_range: nonzero if some context is a single symbol of frequency 65536 (entry field 0,
  * the state does not change there); 0 promises there is none, and the scan for lanes whose
  * lookup byte names a neighbour of their symbol then leaves that case out.
@@ -189,6 +198,7 @@ typedef struct grf_bctx_fused {
   const uint8_t *lut;
   const uint64_t *tab;
   const uint8_t *col_class;
+  const uint32_t *row_pos;
   uint32_t main_n_bytes;
   uint32_t rows, cols;
   uint32_t nr, nc;

@@ -189,14 +189,16 @@ def test_planner_takes_the_fewest_slabs_among_tilings_it_scores_alike(monkeypatc
 
 def test_wave_planner_on_the_benchmark_shapes(monkeypatch):
     """17408 x 5120 and 5120 x 17408 in four row classes: two workgroups of twelve waves per
-    compute unit, one round of workgroups, the units of a tile shared out evenly."""
+    compute unit, one round of workgroups, the units of a tile shared out evenly; a tile is a
+    whole number of units (the rows of a unit are a block of the resident residual order)."""
     monkeypatch.delenv("GEOREFINE_FUSED_WAVE_TILING", raising=False)
-    for rows, spr, want in ((17408, 80, (768, 16, 34)), (5120, 272, (768, 32, 10))):
+    for rows, spr, want in ((17408, 80, (768, 16, 36)), (5120, 272, (768, 32, 10))):
         cap = lambda lanes: (16 + 54 * lanes + 8 + 15) // 16 * 16
         lds = lambda t, p, r, s, c: _fused.lds_bytes_waves(16, 9, 200, 2, t, p, r, s, c)
         threads, p, r, n_slabs, n_tiles, _, total = _fused.choose_wave_tiling(
             spr, np.asarray([rows // 4] * 4), cap, lds, seg_len=64, table_bytes=53 * 1024)
-        assert (threads, p, r) == want and n_tiles == 512 and n_slabs == -(-spr // p)
+        assert (threads, p, r) == want and n_slabs == -(-spr // p) and r % (64 // p) == 0
+        assert n_tiles == 4 * -(-(rows // 4) // r) and 480 <= n_tiles <= 512
         assert total * 2 <= _fused.MAX_LDS
 
 
@@ -223,3 +225,34 @@ def test_group_plans_share_one_tile_shape_and_keep_every_member_complete():
     other = _plan(weight_like(rng, 32, 1280))[1]
     with pytest.raises(_fused.FusedUnsupported):
         _fused.plan_group([plans[0], other], m=1)
+
+
+@pytest.mark.parametrize("shape,nr", [((200, 1280), 16), ((96, 640), 4), ((33, 256), 1)],
+                         ids=lambda v: f"{v[0]}x{v[1]}" if isinstance(v, tuple) else f"nr{v}")
+def test_resident_residual_order(shape, nr):
+    """Positions: one per row, rows of a class in index order on consecutive positions, every
+    class from a multiple of 16 on, in the tilings' class order; every 12-byte group then lies
+    where the address rule of the header puts it, for each block size."""
+    rng = np.random.default_rng(shape[0])
+    ix, plan = _plan(weight_like(rng, *shape), nr=nr)
+    block, position, held = plan.residual_order()
+    assert block in (1, 2, 4, 8, 16) and held % 16 == 0 and held >= shape[0]
+    assert len(set(position.tolist())) == shape[0] and int(position.max()) < held
+    tile_rows, tile_class = _fused.build_tiles(plan.row_class, nr, 1)  # the tilings' order of the rows
+    in_order = position[tile_rows]
+    assert np.all(np.diff(in_order.astype(np.int64)) > 0)
+    for rho in range(nr):
+        of_class = in_order[tile_class == rho]
+        if of_class.size:
+            assert of_class[0] % 16 == 0 and np.all(np.diff(of_class.astype(np.int64)) == 1)
+    rows, cols = shape
+    seg, spr, groups = 64, cols // 64, 4
+    raw = rng.integers(0, 256, size=rows * cols * 3 // 4, dtype=np.uint8)
+    by_frame = raw.reshape(rows, spr, groups, 12)
+    for b in (1, 2, 4, 8, 16):
+        ordered = _fused.order_residuals(raw, rows, cols, seg, b, position, held)
+        assert ordered.size == held * cols * 3 // 4
+        for r, s, t in zip(rng.integers(0, rows, 64), rng.integers(0, spr, 64), rng.integers(0, groups, 64)):
+            q = int(position[r])
+            at = (((q // b * groups + t) * spr + s) * b + q % b) * 12
+            assert np.array_equal(ordered[at:at + 12], by_frame[r, s, t]), (b, r, s, t)
