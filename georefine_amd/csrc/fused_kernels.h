@@ -260,6 +260,10 @@ struct WaveLdsLayout {
   }
 };
 
+// Bytes of activations (all rows of a pass) above which the wave-unit GEMV numbers its units by
+// slab first: half the first-level cache of a compute unit.
+constexpr uint32_t kUnitsBySlabBytes = 16 * 1024;
+
 // Product of two numbers below 2^24 whose product is below 2^32 (row and segment indices of a
 // wave tiling: check_fused_frame holds rows and columns to that): the 24-bit multiply issues
 // at full rate, the 32-bit one at a quarter of it.
@@ -310,18 +314,26 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
   const uint32_t P = g.lanes_per_row, rpw = 64 / P, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f), f.whole_range};
-  // P is a power of two: lane coordinates by shift and mask.  A unit u = (row group grp, slab b)
-  // with u = grp * n_slabs + b; a wave steps through its units u = wave, wave + nwaves, ... by
-  // adding (nwaves / n_slabs, nwaves % n_slabs) with a carry, in scalar registers: divisions by
-  // values only known at run time cost some twenty vector instructions each, and there were
-  // six of them per unit.
+  // P is a power of two: lane coordinates by shift and mask.  A unit is (row group grp, slab b),
+  // numbered u = grp * n_slabs + b or, for long rows, u = b * groups + grp; a wave steps through
+  // its units u = wave, wave + nwaves, ... by adding (nwaves / n, nwaves % n) to the pair with a
+  // carry, in scalar registers: divisions by values only known at run time cost some twenty
+  // vector instructions each, and there were six of them per unit.
+  // Which numbering: the waves of a compute unit work on neighbouring units, and every lane
+  // reads its segment's 128 bytes of x in eight visits.  Numbered by row group first, twelve
+  // waves are spread over every slab of the row, and once x outgrows the 32 KiB first-level
+  // cache those lines come from the L2 again on most visits; numbered by slab first they share
+  // two or three slabs' worth of x (5120 x 17408: 71 -> 65 us).  Short rows keep the first
+  // numbering, where neighbouring waves also share the lines at the ends of their stream pieces.
   const uint32_t logp = 31 - __builtin_clz(P);
   const uint32_t rl = lane >> logp, p = lane & (P - 1);
   float *sub = reinterpret_cast<float *>(lds + L.sub);
   uint32_t *rows = reinterpret_cast<uint32_t *>(lds + L.rows);
   const uint32_t piece_off = L.stream + (wave * rpw + rl) * g.piece_cap;
   const uint32_t groups = (R + rpw - 1) / rpw, units = groups * g.n_slabs;
-  const uint32_t step_grp = nwaves / g.n_slabs, step_b = nwaves % g.n_slabs;
+  const bool by_slab = K * 2u * M > kUnitsBySlabBytes;
+  const uint32_t n_minor = by_slab ? groups : g.n_slabs;
+  const uint32_t step_major = nwaves / n_minor, step_minor = nwaves % n_minor;
   uint32_t bad = 0;
 
   // The byte range [g0, g1) of a unit's row piece is the first of two dependent reads before
@@ -338,11 +350,12 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     g1 = grf::fused_index_entry(f.seg_offset, seg_base + past);  // (no row: an empty range)
   };
   auto advance = [&](uint32_t &grp, uint32_t &b) {  // the unit nwaves further on
-    grp += step_grp;
-    b += step_b;
-    if (b >= g.n_slabs) b -= g.n_slabs, ++grp;
+    uint32_t &major = by_slab ? b : grp, &minor = by_slab ? grp : b;
+    major += step_major;
+    minor += step_minor;
+    if (minor >= n_minor) minor -= n_minor, ++major;
   };
-  uint32_t grp = wave / g.n_slabs, b = wave % g.n_slabs;  // this wave's first unit
+  uint32_t grp = by_slab ? wave % n_minor : wave / n_minor, b = by_slab ? wave / n_minor : wave % n_minor;  // the first unit
   uint32_t row, rpos, g0, g1;
   {
     const uint32_t slot0 = grp * rpw + rl;
