@@ -61,7 +61,10 @@ def test_fused_decode_rare_symbols_forward_scan(oracle):
     assert np.array_equal(t.decode(general=True).view(torch.uint16).cpu().numpy(), words)
 
 
-@pytest.mark.parametrize("shape", [(64, 256), (512, 1280), (100, 384), (16, 2176)], ids=lambda s: f"{s[0]}x{s[1]}")
+# (rows of 12288 and 6144: the activations outgrow half the first-level cache and the wave units
+# are numbered by slab first, from one row on and from two rows on)
+@pytest.mark.parametrize("shape", [(64, 256), (512, 1280), (100, 384), (16, 2176), (40, 12288), (72, 6144)],
+                         ids=lambda s: f"{s[0]}x{s[1]}")
 def test_gemv_matches_float64_and_is_m_invariant(oracle, shape):
     import torch
     rng = np.random.default_rng(shape[1])
