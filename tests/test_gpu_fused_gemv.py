@@ -171,3 +171,48 @@ def test_scan_variants_and_the_whole_range_promise(oracle):
         t.gemv(x[:1], check=True)
     with pytest.raises(codec.CodecError):
         t.gemm(x, check=True)
+
+
+def test_residual_order_fields_are_checked_and_any_block_size_decodes(oracle):
+    """The residual order is a property of the arrays, not of a tiling: the same frame held in
+    blocks of 1, 2, 4, 8 or 16 rows gives the same words and products through every kernel; a
+    block size that is not one of those, or positions without the interleaved order, are refused
+    before anything is launched."""
+    import copy
+    import ctypes
+    import torch
+    from georefine_amd import _fused
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd.bitexact_context_gpu import index_frame
+    rng = np.random.default_rng(77)
+    words = weight_like(rng, 104, 1024)
+    frame, t = _tensor(words)
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(20, 1024)))).view(torch.bfloat16).cuda()
+    want_v, want_m = t.gemv(x[:2], check=True), t.gemm(x, check=True)
+    indexed = index_frame(frame, 1024, fused_segment=t.fused_plan["seg_len"], raw6_residual=True)
+    block0, position, held = t._plan.residual_order()
+    for block in (1, 2, 4, 8, 16):
+        other = copy.copy(t)
+        other.buffers = dict(t.buffers)
+        ordered = _fused.order_residuals(indexed["residual_stream"], 104, 1024, t.fused_plan["seg_len"], block,
+                                         position, held)
+        other.buffers["residual_stream"] = torch.from_numpy(ordered).cuda()
+        other._raw6_block = block
+        other._bind()
+        assert other.fused.raw_interleaved == block
+        assert np.array_equal(other.decode().view(torch.uint16).cpu().numpy(), words), block
+        assert np.array_equal(other.decode(general=True).view(torch.uint16).cpu().numpy(), words), block
+        assert torch.equal(other.gemv(x[:2], check=True), want_v), block
+        assert torch.equal(other.gemm(x, check=True), want_m), block
+    y = torch.empty(1, 104, dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    call = lambda f: t._lib.grf_bctx_gemv(ctypes.byref(f), ctypes.byref(t._tiling(1)[0]), x.data_ptr(), x.stride(0), 1,
+                                          y.data_ptr(), y.stride(0), None, t.error.data_ptr(), stream)
+    bad = type(t.fused).from_buffer_copy(t.fused)
+    bad.raw_interleaved = 3
+    assert call(bad) != 0 and b"raw_interleaved" in t._lib.grf_last_error()
+    bad = type(t.fused).from_buffer_copy(t.fused)
+    bad.raw_interleaved = 0
+    assert call(bad) != 0 and b"positions" in t._lib.grf_last_error()
+    assert call(t.fused) == 0
+    torch.cuda.synchronize()
