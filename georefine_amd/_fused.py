@@ -250,13 +250,27 @@ WAVE_ROWS_PER_PASS = 2  # activation rows one launch of the wave-unit kernel car
 WAVE_UNIT_OVERHEAD = 8  # decode steps' worth of staging, reduction and bookkeeping per unit
 
 
+WAVE_PIECE_OVERHEAD = 1.7   # decode steps' worth of staging per row piece of a unit (fitted, see below)
+WAVE_LATENCY_RATIO = 4.5    # a lone wave's time for a step / its share of a saturated SIMD's issue time
+
+
 def choose_wave_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=64, table_bytes=0):
     """Tiling of the wave-unit GEMV: a wave walks units of 64 / P rows x P consecutive
     segments (P a power of two) and the waves of a workgroup share out the units of its tile
-    without meeting at a barrier.  Modelled time = rounds of workgroups x (table copy + the
-    busiest wave's units x steps per unit), at the speed the resident wave count allows;
-    the score is the share of the paid lane-steps that decode a symbol."""
-    total_rows = sum(int(c) for c in class_rows)
+    without meeting at a barrier; a tile is a whole number of units (a unit's rows are then a
+    block of the resident residual order).
+
+    Modelled time, in decode steps of one SIMD: a launch is bounded by the chain of units its
+    busiest wave walks one after the other (each step a round trip of dependent instructions
+    and LDS reads: WAVE_LATENCY_RATIO issue slots) and by the instructions all waves of a
+    compute unit issue on its four SIMDs; the two are joined as a cubic mean, and the busiest
+    wave counts half by its own units and half by the average (waves that finish leave the
+    rest the machine).  A unit costs its steps, WAVE_UNIT_OVERHEAD, and WAVE_PIECE_OVERHEAD
+    per row piece it stages.  Fitted on a sweep of 120 forced tilings each of 6144 x 5120,
+    5120 x 6144, 1024 x 5120, 17408 x 5120 and 5120 x 17408 on the GPU: the model's choice is
+    the fastest measured tiling for four of them and 9 % off for the smallest (rank
+    correlation 0.89 to 0.99); counting paid lane-steps alone, as before, chose tilings 16 %
+    and 29 % slower than the best for the two middle shapes."""
     forced = os.environ.get("GEOREFINE_FUSED_WAVE_TILING")  # "threads,lanes_per_row,rows": experiments only
     if forced:
         t_, p_, r_ = (int(v) for v in forced.split(","))
@@ -264,29 +278,31 @@ def choose_wave_tiling(spr, class_rows, piece_cap_fn, lds_fn, cus=256, seg_len=6
         n_slabs = -(-spr // p_)
         return t_, p_, r_, n_slabs, _tiles(class_rows, r_), cap, lds_fn(t_, p_, r_, n_slabs, cap)
     best = None
-    unit_steps = seg_len + WAVE_UNIT_OVERHEAD
+    table_steps = 3 + table_bytes / 12288
     for p in (4, 8, 16, 32, 64):
         if p > 4 and p // 2 >= spr:
             continue  # half the lanes of every unit would idle
         rpw = 64 // p
         n_slabs = -(-spr // p)
         cap = piece_cap_fn(p)
+        unit_steps = seg_len + WAVE_UNIT_OVERHEAD + WAVE_PIECE_OVERHEAD * rpw
         for threads in (1024, 768, 512):
             nwaves = threads // 64
-            for r in range(rpw, 129, rpw):  # whole units: their rows are then the blocks of the residual order
-                groups = -(-r // rpw)
+            for r in range(rpw, 129, rpw):
                 lds = lds_fn(threads, p, r, n_slabs, cap)
                 if lds > MAX_LDS:
                     break
-                per_cu = max(1, min(24 // nwaves, MAX_LDS // lds))  # six waves per SIMD by registers
-                slots = cus * per_cu
+                # six waves per SIMD by registers; a little LDS stays with the system
+                per_cu = max(1, min(24 // nwaves, (MAX_LDS - 1024) // lds))
                 tiles = _tiles(class_rows, r)
-                rounds = -(-tiles // slots)
-                unit_rounds = -(-(groups * n_slabs) // nwaves)
-                paid = rounds * slots * nwaves * 64 * (unit_rounds * unit_steps + 3 + table_bytes / 12288)
-                score = total_rows * spr * seg_len / paid * min(1.0, per_cu * nwaves / 24)
-                if best is None or score > best[0] * 1.0001:
-                    best = (score, threads, p, r, n_slabs, tiles, cap, lds)
+                rounds = -(-tiles // (cus * per_cu))
+                units = -(-r // rpw) * n_slabs
+                busiest = 0.5 * -(-units // nwaves) + 0.5 * units / nwaves
+                chain = rounds * (busiest * unit_steps + table_steps) * WAVE_LATENCY_RATIO
+                issue = tiles / cus * (units * unit_steps + nwaves * table_steps) / 4
+                time = (chain ** 3 + issue ** 3) ** (1 / 3)
+                if best is None or time < best[0] * 0.9999:
+                    best = (time, threads, p, r, n_slabs, tiles, cap, lds)
     if best is None:
         raise FusedUnsupported("no wave-unit tiling fits in LDS")
     return best[1:]
