@@ -167,14 +167,18 @@ def test_serving_modules_with_fused_and_predictive_weights(oracle):
     assert out.shape == (2, 256)
 
 
+@pytest.mark.parametrize("cut", [None, "8,32,4"], ids=["planned", "cut4"])
 @pytest.mark.parametrize("mode", [0, 1])
-def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle, mode):
+def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle, monkeypatch, mode, cut):
     """The predictive walker behind the GEMV and GEMM sinks: within 1e-2 of the dense product
     of the decoded target (the tolerance of the fused products), GEMV rows bit-equal for
-    M = 1..8, GEMM rows bit-equal for every batch."""
+    M = 1..8, GEMM rows bit-equal for every batch -- with the planner's GEMM tiling and with one
+    forced to four parts along K."""
     import torch
     from georefine_amd import bitexact_predictive_codec as codec
     from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
+    if cut:
+        monkeypatch.setenv("GEOREFINE_FUSED_GEMM_TILING", cut)
     rng = np.random.default_rng(40 + mode)
     target = weight_like(rng, 200, 1280)
     tf = (target.astype(np.uint32) << 16).view(np.float32)
@@ -198,6 +202,8 @@ def test_ppcx_fused_products_match_dense_and_rows_do_not_depend_on_batch(oracle,
         assert torch.equal(t.gemv(ref_dev, x[:m], bias).view(torch.uint16), y8[:m].view(torch.uint16))
     assert torch.equal(t.linear(ref_dev, x[:1], bias).view(torch.uint16), y8[:1].view(torch.uint16))  # one row: the GEMV
     y40 = t.linear(ref_dev, x, bias, check=True, batch_invariant=True)  # the matrix-core kernel
+    if cut:
+        assert t._tiling_for("gemm")[0].k_parts == int(cut.split(",")[2])
     assert torch.equal(t.linear(ref_dev, x, bias, check=True).view(torch.uint16), y40.view(torch.uint16))  # default to 128 rows
     assert close(y40, 40)
     many = torch.cat([x, x, x, x[:10]])                                  # 130 rows: decode + dense by default
