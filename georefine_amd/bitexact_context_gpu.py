@@ -164,6 +164,7 @@ class HipContextTensor:
     """A BCTX-coded BF16 matrix resident on one MI355X."""
 
     GEMV_UP_TO = 2    # activation rows linear() gives to the vector-ALU kernel
+    GEMM_TWO_ROWS_FROM = 8192  # row length from which two activation rows go to the matrix-core kernel
     DENSE_ABOVE = 128  # activation rows above which linear() decodes to a dense transient
 
     def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None):
@@ -460,9 +461,9 @@ class HipContextTensor:
     def linear(self, x, bias=None, *, check=False, batch_invariant=False):
         """y = x @ W.T (+ bias) with W decoded inside the kernel; x is BF16 [..., K].
 
-        One or two activation rows run the fused decode-GEMV, up to 128 the fused decode-GEMM
-        (one launch; from three rows on it is faster than the GEMV, whose cost grows with every
-        row); above that a fused decode to a dense transient followed by the library matmul is
+        One or two activation rows run the fused decode-GEMV (two rows of 8192 columns or more:
+        the GEMM), up to 128 the fused decode-GEMM (one launch; from three rows on it is faster
+        than the GEMV, whose cost grows with every row); above that a fused decode to a dense transient followed by the library matmul is
         faster (a second GEMM launch would decode the matrix again).  ``batch_invariant=True`` sends
         every row count through the GEMM so that a row's output never depends on the batch
         it arrives in.  Frames the fused kernels cannot take are decoded on the device and
@@ -473,7 +474,10 @@ class HipContextTensor:
         m = math.prod(x.shape[:-1])
         if self.fused is None or (m > self.DENSE_ABOVE and not batch_invariant):
             return F.linear(x.to(self.device), self.decode(check=check), bias)
-        if batch_invariant or m > self.GEMV_UP_TO or m == 0:
+        # (two rows of a long-row matrix: the GEMV's second row costs it 44 % at K = 17408, where its
+        # activations no longer stay in the first-level cache, and the GEMM is the faster of the two)
+        long_rows = m == 2 and self.shape[1] >= self.GEMM_TWO_ROWS_FROM
+        if batch_invariant or m > self.GEMV_UP_TO or m == 0 or long_rows:
             return self.gemm(x, bias, check=check)
         return self.gemv(x, bias, check=check)
 

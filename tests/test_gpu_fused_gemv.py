@@ -216,3 +216,15 @@ def test_residual_order_fields_are_checked_and_any_block_size_decodes(oracle):
     assert call(bad) != 0 and b"positions" in t._lib.grf_last_error()
     assert call(t.fused) == 0
     torch.cuda.synchronize()
+
+
+def test_two_rows_take_the_gemv_on_short_rows_and_the_gemm_on_long_ones():
+    import torch
+    rng = np.random.default_rng(9)
+    for shape, long_rows in (((48, 1024), False), ((24, 8192), True)):
+        _, t = _tensor(weight_like(rng, *shape))
+        x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(2, shape[1])))).view(torch.bfloat16).cuda()
+        y = t.linear(x, check=True)
+        same_as = t.gemm(x, check=True) if long_rows else t.gemv(x, check=True)
+        assert torch.equal(y.view(torch.uint16), same_as.view(torch.uint16))
+        assert torch.equal(t.linear(x[:1]).view(torch.uint16), t.gemv(x[:1]).view(torch.uint16))
