@@ -1,7 +1,8 @@
 // Kernels and launchers of the fused sinks, generic over the segment walker: the same
 // bodies serve the context codec (grf::SegmentWalk) and the predictive codec (its walker
 // in fused_ppcx.hip).  A walker provides prefetch(frame, segment, first element, first
-// column, segment's position in its row), start(piece offset, staged-from offset),
+// column, segment's number in its row, the row's position in the residual order),
+// start(piece offset, staged-from offset),
 // begin16(t, S) + half<0|1, scan kind>(params, pair[4]) for the two halves of a group of
 // 16 symbols (decode16 = all three) and ended_on_checkpoint(frame).
 //
