@@ -256,3 +256,17 @@ def test_resident_residual_order(shape, nr):
             q = int(position[r])
             at = (((q // b * groups + t) * spr + s) * b + q % b) * 12
             assert np.array_equal(ordered[at:at + 12], by_frame[r, s, t]), (b, r, s, t)
+
+
+def test_wave_planner_prefers_wide_units_for_attention_size_matrices(monkeypatch):
+    """6144 x 5120 and 5120 x 6144 in sixteen classes: tilings of one round of workgroups whose
+    waves walk at most two units tie on lane-steps; the modelled time also counts the row pieces a
+    unit stages and the average number of units per wave, and picks units of 4 x 16 and 2 x 32
+    (measured: the fastest of 120 forced tilings each; 16 rows x 4 segments took 16-29 % longer)."""
+    monkeypatch.delenv("GEOREFINE_FUSED_WAVE_TILING", raising=False)
+    for rows, spr, want in ((6144, 80, (768, 16, 12)), (5120, 96, (768, 32, 10))):
+        cap = lambda lanes: (16 + 46 * lanes + 8 + 15) // 16 * 16
+        lds = lambda t, p, r, s, c: _fused.lds_bytes_waves(4, 13, 100, 2, t, p, r, s, c)
+        threads, p, r, n_slabs, n_tiles, _, total = _fused.choose_wave_tiling(
+            spr, np.asarray([rows // 16] * 16), cap, lds, seg_len=64, table_bytes=4 * (101 * 8 + 8192))
+        assert (threads, p, r) == want and n_tiles == 512 and total * 2 <= _fused.MAX_LDS
