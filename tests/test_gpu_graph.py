@@ -9,8 +9,13 @@ from conftest import bf16_words, weight_like
 pytestmark = pytest.mark.gpu
 
 
-def test_captured_products_replay_bit_for_bit():
+@pytest.mark.parametrize("cut", [None, "8,32,2"], ids=["planned", "cut2"])
+def test_captured_products_replay_bit_for_bit(monkeypatch, cut):
+    """(``cut``: the GEMM tilings forced to two parts along K, i.e. a second kernel per product
+    that adds the parts from the workspace.)"""
     import torch
+    if cut:
+        monkeypatch.setenv("GEOREFINE_FUSED_GEMM_TILING", cut)
     from georefine_amd import bitexact_context_codec as codec
     from georefine_amd import bitexact_predictive_codec as ppcx
     from georefine_amd.bitexact_context_gpu import HipContextTensor
@@ -28,6 +33,8 @@ def test_captured_products_replay_bit_for_bit():
         return torch.from_numpy(bf16_words(rng.normal(0, 1, size=(rows, 1024)))).view(torch.bfloat16).cuda()
 
     x1, x40 = draw(1), draw(40)
+    if cut:
+        assert t._gemm_tiling()[0].k_parts == 2 and p._tiling_for("gemm")[0].k_parts == 2
 
     def step():
         return (t.gemv(x1), t.gemm(x40), t.decode(check=False), p.gemm(ref_dev, x40), p.decode(ref_dev, check=False))
