@@ -555,3 +555,34 @@ def plan_group(plans, m=None, gemm=False, waves=False):
                             scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
                                          n_tiles=len(tile_class), piece_cap=cap, scheme=scheme), lds=lds))
     return tilings
+
+
+VALIDATE_USES = {"decode": 0, "gemv": 1, "gemm": 2, "gather": 3}
+
+
+def validate_host(plan, tiling, use, *, row_pos=None, block=0, main_bytes=None):
+    """The device library's host-side validator (``grf_bctx_fused_validate_host``) on a plan and
+    one of its tilings (as ``FramePlan.tiling`` / ``gemm_tiling`` return them): what the kernels
+    take on trust from the index and the tiling arrays -- offsets in order and inside the
+    stream, every staged piece within ``piece_cap``, rows and classes of the tiles, the LDS
+    demand.  Needs no GPU.  Raises ``FusedUnsupported`` with the library's message."""
+    import ctypes
+    from . import _hip_abi, _native
+    lib = _native.hip()
+    f = _hip_abi.GrfBctxFused()
+    for key, value in plan.scalars().items():
+        setattr(f, key, value)
+    f.main_n_bytes = int(plan.seg_offset[-1]) if main_bytes is None else main_bytes
+    f.raw_interleaved = block
+    g = _hip_abi.GrfFusedTiling()
+    for key, value in tiling["scalars"].items():
+        setattr(g, key, value)
+    arrays = [np.ascontiguousarray(plan.seg_offset, dtype=np.uint32),
+              np.ascontiguousarray(tiling["tile_rows"], dtype=np.uint32),
+              np.ascontiguousarray(tiling["tile_class"], dtype=np.uint8),
+              np.ascontiguousarray(plan.row_class, dtype=np.uint8),
+              None if row_pos is None else np.ascontiguousarray(row_pos, dtype=np.uint32)]
+    status = lib.grf_bctx_fused_validate_host(ctypes.byref(f), ctypes.byref(g), VALIDATE_USES[use],
+                                              *[a.ctypes.data if a is not None else None for a in arrays])
+    if status:
+        raise FusedUnsupported(lib.grf_last_error().decode(errors="replace"))

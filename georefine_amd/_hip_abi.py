@@ -49,7 +49,7 @@ class GrfPpcxFused(ctypes.Structure):
 
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
-                  "grf_bctx_fused_decode", "grf_bctx_fused_gather", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
+                  "grf_bctx_fused_decode", "grf_bctx_fused_gather", "grf_bctx_fused_validate_host", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
                   "grf_gemm_workspace_bytes", "grf_gemm_workspace_bytes_split", "grf_bctx_gemm_noalloc", "grf_gemm_noalloc_limit_bytes", "grf_pack_activations", "grf_bctx_gemv_group", "grf_bctx_gemm_group",
                   "grf_ppcx_bins", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_last_error",
                   "grf_abi_version")
@@ -89,6 +89,8 @@ def declare(L):
     L.grf_bctx_fused_decode.restype = i
     L.grf_bctx_fused_gather.argtypes = L.grf_bctx_fused_decode.argtypes
     L.grf_bctx_fused_gather.restype = i
+    L.grf_bctx_fused_validate_host.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, i, vp, vp, vp, vp, vp]
+    L.grf_bctx_fused_validate_host.restype = i
     L.grf_bctx_fused_lds_bytes.argtypes = [ctypes.POINTER(GrfBctxFused), tiling, u32]
     L.grf_bctx_fused_lds_bytes.restype = u32
     L.grf_ppcx_bins.argtypes = [vp, vp, vp, u32, u32, vp, vp]

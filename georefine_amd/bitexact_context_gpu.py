@@ -122,6 +122,33 @@ def _device_stream(buffers, name, vocab, nctx):
     return s
 
 
+GEMV_UP_TO = 2             # activation rows linear() gives to the vector-ALU kernel
+GEMM_TWO_ROWS_FROM = 8192  # row length from which two activation rows go to the matrix-core kernel
+DENSE_ABOVE = 128          # activation rows above which linear() decodes to a dense transient
+
+
+def route_rows(m, cols, invariant=False):
+    """The kernel family that takes ``m`` activation rows of a matrix with ``cols`` columns:
+    ``"gemv"`` (vector ALUs), ``"gemm"`` (matrix cores) or ``"dense"`` (fused decode + library
+    matmul).  One rule for single matrices and grouped launches.
+
+    ``invariant``: every row count takes the matrix-core kernel, whose accumulation order per
+    output element is fixed by the matrix alone -- row m of an M-row call then has the bits of
+    the one-row call (the property GS/miv_gemv.py:1-9 states for M <= 8 and
+    GS/bi_csrc/bi_gemm.cuh:1-17 for any M: a speculative verify pass at M = k + 1 reproduces the
+    decode steps).  Without it the fastest family per row count is chosen: the GEMV for one
+    row and for two rows of a short-row matrix (its second row costs 44 % at K = 17408, where
+    its activations no longer stay in the first-level cache), the GEMM to 128 rows, the dense
+    route above; rows are then bit-equal only between calls that take the same family."""
+    if invariant:
+        return "gemm"
+    if m > DENSE_ABOVE:
+        return "dense"
+    if m == 0 or m > GEMV_UP_TO or (m == 2 and cols >= GEMM_TWO_ROWS_FROM):
+        return "gemm"
+    return "gemv"
+
+
 class PackedActivations:
     """Activation rows copied once into the operand order of the matrix-core kernels, for
     several coded matrices that take the same input (q/k/v, gate/up): ``gemm`` and
@@ -163,15 +190,17 @@ class PackedActivations:
 class HipContextTensor:
     """A BCTX-coded BF16 matrix resident on one MI355X."""
 
-    GEMV_UP_TO = 2    # activation rows linear() gives to the vector-ALU kernel
-    GEMM_TWO_ROWS_FROM = 8192  # row length from which two activation rows go to the matrix-core kernel
-    DENSE_ABOVE = 128  # activation rows above which linear() decodes to a dense transient
+    GEMV_UP_TO, GEMM_TWO_ROWS_FROM, DENSE_ABOVE = GEMV_UP_TO, GEMM_TWO_ROWS_FROM, DENSE_ABOVE
 
-    def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None):
+    def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None,
+                 m_invariant=False):
         import torch
         if not torch.cuda.is_available():
             raise RuntimeError("a ROCm GPU is required")
         self._lib = _native.hip()  # fails loudly when the device library is absent
+        # linear()'s default routing: True sends every row count to the matrix-core kernel, so
+        # that a row's output bits never depend on the rows it arrives with (route_rows)
+        self.m_invariant = bool(m_invariant)
         segment = None
         if fused:
             try:
@@ -458,26 +487,29 @@ class HipContextTensor:
             return self._packed_call(x, bias, check)
         return self._fused_call(self._lib.grf_bctx_gemm, self._gemm_tiling()[0], x, bias, check, workspace=True)
 
-    def linear(self, x, bias=None, *, check=False, batch_invariant=False):
+    def linear(self, x, bias=None, *, check=False, batch_invariant=None):
         """y = x @ W.T (+ bias) with W decoded inside the kernel; x is BF16 [..., K].
 
-        One or two activation rows run the fused decode-GEMV (two rows of 8192 columns or more:
-        the GEMM), up to 128 the fused decode-GEMM (one launch; from three rows on it is faster
-        than the GEMV, whose cost grows with every row); above that a fused decode to a dense transient followed by the library matmul is
-        faster (a second GEMM launch would decode the matrix again).  ``batch_invariant=True`` sends
-        every row count through the GEMM so that a row's output never depends on the batch
-        it arrives in.  Frames the fused kernels cannot take are decoded on the device and
-        multiplied densely.  ``check=True`` reads the error word back (a host sync)."""
+        The row count picks the kernel family (``route_rows``): by default the fastest one --
+        the fused decode-GEMV for one row (and two rows of a short-row matrix), the fused
+        decode-GEMM to 128 rows (one launch), above that a fused decode to a dense transient
+        and the library matmul (a second GEMM launch would decode the matrix again).
+        ``batch_invariant=True`` -- or the tensor's ``m_invariant`` policy, which is the default
+        when the argument is left out -- sends every row count through the GEMM, so that a
+        row's output never depends on the batch it arrives in: ``linear(x[:1])`` is
+        ``linear(x[:6])[:1]`` bit for bit.  Frames the fused kernels cannot take are decoded on
+        the device and multiplied densely.  ``check=True`` reads the error word back (a host
+        sync)."""
         import torch.nn.functional as F
         if isinstance(x, PackedActivations):  # packed for the matrix-core kernel, which is what it gets
             return self.gemm(x, bias, check=check)
+        if batch_invariant is None:
+            batch_invariant = self.m_invariant
         m = math.prod(x.shape[:-1])
-        if self.fused is None or (m > self.DENSE_ABOVE and not batch_invariant):
+        route = "dense" if self.fused is None else route_rows(m, self.shape[1], batch_invariant)
+        if route == "dense":
             return F.linear(x.to(self.device), self.decode(check=check), bias)
-        # (two rows of a long-row matrix: the GEMV's second row costs it 44 % at K = 17408, where its
-        # activations no longer stay in the first-level cache, and the GEMM is the faster of the two)
-        long_rows = m == 2 and self.shape[1] >= self.GEMM_TWO_ROWS_FROM
-        if batch_invariant or m > self.GEMV_UP_TO or m == 0 or long_rows:
+        if route == "gemm":
             return self.gemm(x, bias, check=check)
         return self.gemv(x, bias, check=check)
 
@@ -527,10 +559,7 @@ class HipLinearGroup:
     on their own.  They must have been indexed with one segment length
     (``HipContextTensor(..., fused_segment=...)``)."""
 
-    GEMV_UP_TO = HipContextTensor.GEMV_UP_TO
-    DENSE_ABOVE = HipContextTensor.DENSE_ABOVE
-
-    def __init__(self, tensors):
+    def __init__(self, tensors, *, m_invariant=None):
         import torch
         self.tensors = list(tensors)
         if not 1 <= len(self.tensors) <= 4:
@@ -542,6 +571,9 @@ class HipLinearGroup:
             if t.shape[1] != first.shape[1] or t.device != first.device:
                 raise ValueError("group members need one width and one device")
         self.device, self._lib = first.device, first._lib
+        # the members' policy unless given: a group of members that keep rows bit-equal across
+        # row counts does so too
+        self.m_invariant = any(t.m_invariant for t in self.tensors) if m_invariant is None else bool(m_invariant)
         self.error = torch.zeros((), device=self.device, dtype=torch.int32)
         self._tilings, self._pointer_arrays = {}, {}
         for key in (1, 2, "gemm"):
@@ -580,11 +612,11 @@ class HipLinearGroup:
         bias = (ctypes.c_void_p * n)(*[b.data_ptr() if b is not None else None for b in biases])
         return frames, tiles, ys, ldy, bias
 
-    def linear(self, x, biases=None, *, check=False, batch_invariant=False):
+    def linear(self, x, biases=None, *, check=False, batch_invariant=None):
         """[x @ W.T (+ bias) for every member]; x is BF16 [..., K] or ``PackedActivations``.
-        Row counts are routed as in ``HipContextTensor.linear``: the GEMV to 2 rows, the
-        matrix-core kernel to 128 (every count with ``batch_invariant``), the members' own
-        decode + matmul above."""
+        Row counts are routed by the rule of ``HipContextTensor.linear`` (``route_rows``), so a
+        member gets the kernel family, and with it the bits, of its own ``linear``; above 128
+        rows the members' own decode + matmul."""
         import torch
         n = len(self.tensors)
         biases = list(biases) if biases is not None else [None] * n
@@ -594,8 +626,11 @@ class HipLinearGroup:
         m = packed.rows if packed else math.prod(x.shape[:-1])
         lead = packed.lead if packed else tuple(x.shape[:-1])
         cols = self.tensors[0].shape[1]
-        if packed is None and m > self.DENSE_ABOVE and not batch_invariant:
-            return [t.linear(x, b, check=check) for t, b in zip(self.tensors, biases)]
+        if batch_invariant is None:
+            batch_invariant = self.m_invariant
+        route = "gemm" if packed is not None else route_rows(m, cols, batch_invariant)
+        if route == "dense":
+            return [t.linear(x, b, check=check, batch_invariant=False) for t, b in zip(self.tensors, biases)]
         if packed is not None:
             if packed.cols != cols or packed.buffer.device != self.device:
                 raise ValueError("packed activations of another width or device")
@@ -611,7 +646,7 @@ class HipLinearGroup:
         if m:
             if check:
                 self.error.zero_()
-            use_gemm = packed is not None or batch_invariant or m > self.GEMV_UP_TO
+            use_gemm = route == "gemm"
             with torch.cuda.device(self.device):
                 stream = torch.cuda.current_stream(self.device).cuda_stream
                 if use_gemm:

@@ -56,19 +56,28 @@ MTP_LINEAR_PATHS = {
 
 class BCTXLinear(nn.Module):
     """A bias-free linear whose weight is a coded tensor (GCR/bitexact_context_mtp.py:279-295).
-    ``calls`` counts forwards; the receipt uses it to prove that every matrix ran."""
+    ``calls`` counts forwards; the receipt uses it to prove that every matrix ran.
 
-    def __init__(self, tensor, name: str):
+    ``m_invariant`` (default on): every row count goes through one kernel family, so that row m
+    of a verify pass over k + 1 draft rows has the bits of the one-row decode step that
+    proposed it (the property GS/miv_gemv.py:1-9 exists for); off, the tensor's own routing
+    picks the fastest kernel per row count."""
+
+    def __init__(self, tensor, name: str, *, m_invariant=True):
         super().__init__()
         self.tensor = tensor
         self.name = str(name)
         self.calls = 0
+        self.m_invariant = bool(m_invariant)
 
     def forward(self, x):
         self.calls += 1
         fused = getattr(self.tensor, "linear", None)
         if fused is not None and x.dtype == torch.bfloat16:
-            return fused(x)
+            try:
+                return fused(x, batch_invariant=True) if self.m_invariant else fused(x)
+            except TypeError:  # a tensor class whose linear() has no such switch
+                return fused(x)
         weight = self.tensor.decode()
         if tuple(weight.shape) != tuple(self.tensor.shape):
             raise ValueError(f"decoded shape changed for {self.name}")
@@ -132,15 +141,17 @@ def _owner(module, dotted):
 
 
 def load_bctx_mtp(manifest_path, frame_root, text_config, *, device="cuda:0", tensor_cls=None,
-                  checkpoint_stride=1024, skeleton=None):
+                  checkpoint_stride=1024, skeleton=None, m_invariant=True):
     """Build the MTP head from its fifteen frames alone (GCR/bitexact_context_mtp.py:327-400).
 
     ``manifest_path`` names a JSON manifest whose ``tensors`` list holds the ``mtp.*`` entries
     (name, shape, dtype "BF16", frame, frame_bytes, frame_sha256, source_sha256); frames are
     read below ``frame_root``.  ``tensor_cls(frame, stride=, device=)`` makes the device tensor
     (default ``HipContextTensor``); ``skeleton(text_config)`` makes the module tree on the meta
-    device (default ``QwenMTP``).  Same checks, same receipt fields and the same errors as the
-    reference; the receipt is kept on the module as ``_bctx_receipt``."""
+    device (default ``QwenMTP``).  ``m_invariant`` is handed to every ``BCTXLinear``: on (the
+    default) a row's output does not depend on how many rows a forward carries.  Same checks,
+    same receipt fields and the same errors as the reference; the receipt is kept on the module
+    as ``_bctx_receipt`` (plus ``m_invariant``)."""
     if tensor_cls is None:
         from .bitexact_context_gpu import HipContextTensor
         tensor_cls = HipContextTensor
@@ -169,7 +180,7 @@ def load_bctx_mtp(manifest_path, frame_root, text_config, *, device="cuda:0", te
             dense = getattr(parent, attr)
             if tuple(dense.weight.shape) != shape or dense.bias is not None:
                 raise ValueError(f"QwenMTP linear skeleton incompatible with {name}")
-            setattr(parent, attr, BCTXLinear(tensor, name))
+            setattr(parent, attr, BCTXLinear(tensor, name, m_invariant=m_invariant))
             continue
         value = tensor.decode()
         if tuple(value.shape) != geometry or value.dtype != torch.bfloat16:
@@ -201,6 +212,7 @@ def load_bctx_mtp(manifest_path, frame_root, text_config, *, device="cuda:0", te
         "source_sha256": {n: t.source_sha256 for n, t in tensors.items()},
         "linear_calls": {n: 0 for n in MTP_LINEAR_PATHS},
         "loaded_from_bctx_only": True,
+        "m_invariant": bool(m_invariant),
     }
     return mtp
 

@@ -141,7 +141,7 @@ class HipPredictiveTensor:
     DENSE_ABOVE = 128  # activation rows above which linear() decodes to a dense transient
 
     def __init__(self, frame, reference_uint16_numpy, stride=1024, device="cuda:0", *, fused=True,
-                 fused_segment=None, resident_contexts=True):
+                 fused_segment=None, resident_contexts=True, m_invariant=False):
         if not isinstance(stride, int) or not 1 <= stride <= 65536:
             raise codec.CodecError("invalid checkpoint stride")
         ix = _read_frame(frame, reference_uint16_numpy, stride, fused=fused, fused_segment=fused_segment)
@@ -149,6 +149,7 @@ class HipPredictiveTensor:
         if not torch.cuda.is_available():
             raise RuntimeError("a ROCm GPU is required")
         self._lib = _native.hip()
+        self.m_invariant = bool(m_invariant)  # linear()'s default for batch_invariant
         self.shape = ix["shape"]
         self.n = math.prod(self.shape)
         self.stride, self.mode = stride, ix["mode"]
@@ -288,7 +289,7 @@ class HipPredictiveTensor:
             raise ValueError("reference device tensor shape/dtype mismatch")
         return ref
 
-    def linear(self, reference_bf16_device, x, bias=None, *, check=False, batch_invariant=False):
+    def linear(self, reference_bf16_device, x, bias=None, *, check=False, batch_invariant=None):
         """y = x W^T + bias with W decoded on the fly against the reference: the fused GEMV for
         one activation row, the fused GEMM (matrix cores, one launch) for up to 128; above that
         the fused decode to a dense transient plus the library matmul is faster, unless
@@ -298,6 +299,8 @@ class HipPredictiveTensor:
         from .bitexact_context_gpu import PackedActivations
         if isinstance(x, PackedActivations):  # packed for the matrix-core kernel, which is what it gets
             return self._product(reference_bf16_device, x, bias, check, True)
+        if batch_invariant is None:  # the tensor's policy
+            batch_invariant = self.m_invariant
         m = math.prod(x.shape[:-1])
         if self.fused is None or x.dtype != torch.bfloat16 or (m > self.DENSE_ABOVE and not batch_invariant):
             return torch.nn.functional.linear(x, self.decode(reference_bf16_device, check=check), bias)

@@ -191,11 +191,12 @@ __device__ __forceinline__ bool fused_lane_in(uint64_t mask) {
 // known not to hold it, so the step comes first and the test after.  The tables cover every
 // slot (the host checks that the frequencies of a context add up to 65536), so the scan ends;
 // the trip limit only keeps a wave from spinning on tables that were overwritten.
+constexpr uint32_t kScanTrips = 256;  // entries a table can have (its index is a byte)
 __device__ __forceinline__ void fused_scan(uint32_t state, StepFetch &s, uint32_t &rel) {
   const uint32_t slot = state & 0xFFFFu;
   uint32_t ta = s.ta;
   v2u32 e = s.e0;
-  uint32_t left = 256;
+  uint32_t left = kScanTrips;
   do {
     ta += (int32_t)rel < 0 ? -8 : 8;
     e = *reinterpret_cast<lds_v2u32 *>(ta);
@@ -206,11 +207,14 @@ __device__ __forceinline__ void fused_scan(uint32_t state, StepFetch &s, uint32_
 // The same for frames in which a context may be a single symbol of frequency 65536 (field 0,
 // start 0): such an entry always reports a miss and is not left; it returns rel = state, so
 // that the update freq16 * (state >> 16) + rel leaves the state as it is.
+// The trip limit is the other scan's: a table has at most 256 entries, so a scan that has
+// not ended by then is walking memory that is not a table; the segment then misses its
+// checkpoint and the launch reports GRF_ERR_CHECKPOINT instead of spinning.
 __device__ __forceinline__ void fused_scan_whole(uint32_t state, StepFetch &s, uint32_t &rel) {
   const uint32_t slot = state & 0xFFFFu;
   uint32_t ta = s.ta;
   v2u32 e = s.e0;
-  for (;;) {
+  for (uint32_t left = kScanTrips; left; --left) {
     const uint32_t freq = e.x >> 16;
     rel = slot - (e.x & 0xFFFFu);
     if (freq == 0) rel = state;

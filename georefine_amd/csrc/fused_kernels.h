@@ -8,11 +8,13 @@
 //
 // GEMV: reduction order of one output element, fixed for every M: the S products of a
 // segment are folded into one fp32 accumulator two columns at a time in increasing k
-// (v_dot2c_f32_bf16: acc += w[k]*x[k] + w[k+1]*x[k+1]).  Slab tilings then add the K/S
-// segment partials of a row in segment order 0..K/S-1 by one thread (slab after slab into
-// a running sum); wave tilings add the P partials of a unit pairwise, neighbours first,
-// and the units' sums of a row in slab order (fused_wave_body).  Bias is added in fp32 and
-// the sum is rounded to BF16 once.
+// (v_dot2c_f32_bf16: acc += w[k]*x[k] + w[k+1]*x[k+1]).  Wave tilings (the GEMV the host
+// side uses) then add a row's segment partials as one pairwise tree per aligned block of 64
+// segments and the blocks in increasing order, whatever the tiling (fused_wave_body).  Slab
+// tilings (kept for experiments) add the K/S segment partials of a row in segment order
+// 0..K/S-1 by one thread, slab after slab into a running sum: a different order, so their
+// outputs agree with the wave tilings' to rounding, not bit for bit.  Bias is added in fp32
+// and the sum is rounded to BF16 once.
 //
 // GEMM, batch invariance (the contract of GS/bi_csrc/bi_gemm.cuh:1-17): output element
 // (m, n) is the sum, in quad order, of one fp32 accumulator per quad of lane-segments;
@@ -29,6 +31,7 @@
 #include <algorithm>
 #include <atomic>
 #include <string>
+#include <vector>
 
 #include <type_traits>
 
@@ -38,7 +41,9 @@ namespace grf {
 int set_error(int code, const std::string &what);                                          // decode_general.hip
 // fused_gemv.hip; wave_units: the entry point takes GRF_TILE_WAVES tilings
 enum TilingUse { kSlabTiling, kGemvTiling, kGemmTiling };  // what an entry point does with the tiling it is given
-int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who, TilingUse use = kSlabTiling);
+// pointers: also refuse null device pointers (a host-side validation has none to give)
+int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const char *who, TilingUse use = kSlabTiling,
+                      bool pointers = true);
 
 // A kernel may ask for more than 64 KiB of dynamic LDS only after its limit has been raised;
 // done once per kernel and device (not per launch: it is a driver call, and a launch that
@@ -244,10 +249,12 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
 // others walk.
 //
 // Reduction order of one output element: the S products of a segment as in the other GEMV;
-// the P segment partials of a unit pairwise, neighbours first (lane distances 1, 2, 4, ...);
-// the units' sums of a row in slab order; bias; one rounding.  The tiling fixes P per matrix,
-// and more than two activation rows run as passes of two, so the order depends neither on the
-// activation row count nor on how rows are dealt to workgroups.
+// the segment partials of a row pairwise, neighbours first, over aligned blocks of 64 segments
+// (a segment the row does not have counts as +0.0); the blocks' sums in increasing order;
+// bias; one rounding.  A unit does the part of that tree that lies inside its P segments
+// (lane distances 1, 2, 4, ...), the tile's last step the rest, so the bits of an output do not
+// depend on P, on how rows are dealt to workgroups, on whether the matrix shares its launch
+// with others, or on the activation row count (more than two rows run as passes of two).
 struct WaveLdsLayout {
   uint32_t blocks, block_pitch, stream, sub, rows, total;
   __host__ __device__ WaveLdsLayout(const grf_bctx_fused &f, const grf_fused_tiling &g, uint32_t m) {
@@ -481,13 +488,29 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     }
   }
   __syncthreads();
+  // A row's unit sums -> its output.  The order is the same for every tiling: the tree that a
+  // unit began over its P segments is carried on over aligned blocks of 64 segments (64 / P
+  // unit sums, pairwise, neighbours first; a unit the row does not have counts as +0.0, like
+  // the lanes without a segment inside a unit), and the blocks' sums are added in
+  // increasing order.
+  const uint32_t per_block = 64u >> logp;  // unit sums of a row per block of 64 segments: 1..16
   for (uint32_t i = tid; i < R * M; i += nthreads) {
     const uint32_t rr = i / M, m = i % M;
     const uint32_t orow = rows[rr];
     if (orow == grf::kNoRow) continue;
     const float *sp = sub + (rr * g.n_slabs) * M + m;
-    float sum = sp[0];
-    for (uint32_t b = 1; b < g.n_slabs; ++b) sum += sp[b * M];
+    float sum = 0.f;
+    for (uint32_t b0 = 0; b0 < g.n_slabs; b0 += per_block) {
+      float v[16];
+#pragma unroll
+      for (uint32_t k = 0; k < 16; ++k) v[k] = (k < per_block && b0 + k < g.n_slabs) ? sp[(b0 + k) * M] : 0.f;
+#pragma unroll
+      for (uint32_t w = 1; w < 16; w <<= 1)
+#pragma unroll
+        for (uint32_t k = 0; k < 16; k += 2 * w)
+          if (w < per_block) v[k] += v[k + w];
+      sum = b0 ? sum + v[0] : v[0];
+    }
     if (bias) sum += __uint_as_float((uint32_t)bias[orow] << 16);
     y[(size_t)m * ldy + orow] = round_bf16(sum);
   }

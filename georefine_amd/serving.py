@@ -82,10 +82,12 @@ def decode_errors(model):
 
 
 class BctxLinear(nn.Module):
-    """Linear layer whose weight stays compressed; ``batch_invariant`` sends every call
-    through the matrix-core kernel so a row never depends on its batch."""
+    """Linear layer whose weight stays compressed; ``batch_invariant=True`` sends every call
+    through the matrix-core kernel so a row never depends on its batch, ``False`` lets the row
+    count pick the fastest kernel, ``None`` leaves the choice to the tensor's own policy
+    (``HipContextTensor.m_invariant``)."""
 
-    def __init__(self, tensor, bias=None, *, batch_invariant=False):
+    def __init__(self, tensor, bias=None, *, batch_invariant=None):
         super().__init__()
         if len(tensor.shape) != 2:
             raise ContextServingError("linear BCTX weight must be rank two")
@@ -187,7 +189,7 @@ class PredictiveContextTensor:
             self.predictor = default_predictor
         return self.predictor(refs[0], refs[1], self.coefficients)
 
-    def linear(self, x, bias=None, *, check=False, batch_invariant=False):
+    def linear(self, x, bias=None, *, check=False, batch_invariant=None):
         """x W^T + bias.  A frame stored untransposed goes through the native tensor's fused
         product: one launch that decodes and contracts, with the contexts of the reference read
         from the plane kept at load (a native tensor without that plane gets the reference
@@ -248,7 +250,12 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
     one tensor, e.g. ``[("q_proj", "k_proj", "v_proj"), ("gate_proj", "up_proj")]``: wherever a
     module has all the children of a tuple as coded linears of one input width (and the device
     tensors support it), they are indexed with one segment length and multiplied in one
-    launch (``SharedProducts``); the receipt lists them under ``shared_launches``.  What this loader leaves to the caller is the model
+    launch (``SharedProducts``); the receipt lists them under ``shared_launches``.
+    ``batch_invariant=True`` is the M-invariant policy: every coded linear sends every row count
+    through the matrix-core kernel, so a verify pass over k + 1 rows reproduces the one-row
+    decode steps bit for bit (GS/miv_gemv.py:1-9); the default lets the row count pick the
+    fastest kernel, and rows are then bit-equal only between calls of the same kernel family
+    (``bitexact_context_gpu.route_rows``).  The receipt records the choice.  What this loader leaves to the caller is the model
     construction itself (the reference reads a Transformers config and generation config
     from the package's sidecars): ``model_factory`` returns the module to fill."""
     import hashlib
@@ -567,6 +574,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         "general_kernel_tensors": sorted(n for n, r in consumed.items()
                                          if r.get("fused") is False and r.get("frame_mode") != 1),
         "shared_launches": shared_launches,
+        "batch_invariant": bool(batch_invariant),
     }
     return model, receipt
 

@@ -259,6 +259,27 @@ int grf_bctx_gemv(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
                   uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, int32_t *error,
                   void *hip_stream);
 
+/* Host-side check of a caller-built frame and tiling before their first launch; no reference
+ * counterpart (the reference builds its descriptors in Python and launches Triton).  The entry
+ * points check the scalars of the two structures on every call; what the kernels take on
+ * trust from the arrays behind them is checked here, on HOST copies of those arrays (the
+ * structures' own pointers are device addresses and are not read; they may be null):
+ *   seg_offset  u32 [rows*segs_per_row + 1]: never decreasing, first entry >= 4, last entry
+ *               == main_n_bytes (a kernel copies [offset[s] & ~15, offset[s + lanes]) to LDS)
+ *   tile_rows / tile_class  as in grf_fused_tiling (for k_parts > 1: the n_tiles / k_parts row
+ *               tiles): slots name rows of the matrix, every row exactly once (use 3: any rows,
+ *               any number of times), classes below nr
+ *   row_class   u8 [rows] or NULL: when given, every row must be of its tile's class
+ *   row_pos     u32 [rows] or NULL: when given, one-to-one
+ * and every stream piece the launch stages (lanes_per_row segments of a row for use 0, 1 and
+ * 3, four segments for use 2) must fit piece_cap, and the launch's LDS demand 160 KiB.
+ * use: 0 = grf_bctx_fused_decode, 1 = grf_bctx_gemv(_group), 2 = grf_bctx_gemm(_group,
+ * _noalloc), 3 = grf_bctx_fused_gather.  Returns GRF_OK or GRF_BAD_ARGUMENT / GRF_UNSUPPORTED
+ * with the reason in grf_last_error().  Runs without a GPU. */
+int grf_bctx_fused_validate_host(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, int use,
+                                 const uint32_t *seg_offset, const uint32_t *tile_rows, const uint8_t *tile_class,
+                                 const uint8_t *row_class, const uint32_t *row_pos);
+
 /* Same walker with a store sink: out[rows*cols] BF16 words (decode() for fused frames). */
 int grf_bctx_fused_decode(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, uint16_t *out,
                           int32_t *error, void *hip_stream);
@@ -344,8 +365,9 @@ uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_t
  *   main_bytes  the frame's main rANS stream, readable for 16 bytes past main_n_bytes
  *   raw5        packed 5-bit residuals, MSB first, readable for 16 bytes past the end
  *   seg_state / seg_offset  as in grf_bctx_fused, contexts label[row]*16 + bin
- *   lut  u8 [n_labels][16 << lognb], tab u32 [n_labels][16][tabn+1][4]   as in grf_bctx_fused,
- *        with the symbol's bits in the BF16 word (sign, exponent, mantissa 6..5) for symbol<<5
+ *   lut  u8 [n_labels][16 << lognb], tab u64 [n_labels][16][tabn+1]   as in grf_bctx_fused:
+ *        low32 = start | (freq & 0xFFFF)<<16, high32 = the symbol's bits in the BF16 word
+ *        (sign, exponent, mantissa bits 6..5) in place of symbol<<5
  * seg_len must be a multiple of 32.  Tilings are built over row labels. */
 typedef struct grf_ppcx_fused {
   const uint8_t *main_bytes;

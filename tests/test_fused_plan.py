@@ -270,3 +270,60 @@ def test_wave_planner_prefers_wide_units_for_attention_size_matrices(monkeypatch
         threads, p, r, n_slabs, n_tiles, _, total = _fused.choose_wave_tiling(
             spr, np.asarray([rows // 16] * 16), cap, lds, seg_len=64, table_bytes=4 * (101 * 8 + 8192))
         assert (threads, p, r) == want and n_tiles == 512 and total * 2 <= _fused.MAX_LDS
+
+
+def test_host_validator_accepts_planned_tilings_and_names_what_is_wrong():
+    """grf_bctx_fused_validate_host on host copies of the index and tiling arrays: the planner's
+    own tilings pass for every entry point; offsets out of order, a piece that outgrows
+    piece_cap, a row in two tiles or in none, a row of another class, an index that does not
+    end on the stream's length and positions shared by two rows are each refused by name."""
+    words = weight_like(np.random.default_rng(3), 96, 768)
+    ix, plan = _plan(words)
+    block, position, held = plan.residual_order()
+    tilings = {"decode": plan.tiling(0), "gemv": plan.tiling(1, waves=True), "gemm": plan.gemm_tiling(),
+               "gather": plan.tiling(0)}
+    for use, tiling in tilings.items():
+        _fused.validate_host(plan, tiling, use, row_pos=position, block=block)
+
+    def refused(match, use="gemv", tiling=None, **kw):
+        with pytest.raises(_fused.FusedUnsupported, match=match):
+            _fused.validate_host(plan, tiling or tilings[use], use, **kw)
+
+    keep = plan.seg_offset.copy()
+    try:
+        plan.seg_offset[5], plan.seg_offset[6] = keep[6] + 3, keep[5]
+        refused("decrease")
+        plan.seg_offset[:] = keep
+        plan.seg_offset[-1] += 1
+        refused("stream's length", main_bytes=int(keep[-1]))
+        plan.seg_offset[:] = keep
+        plan.seg_offset[0] = 0
+        refused("initial state")
+    finally:
+        plan.seg_offset[:] = keep
+    for use in ("decode", "gemv", "gemm"):
+        small = dict(tilings[use], scalars=dict(tilings[use]["scalars"], piece_cap=16))
+        refused("piece_cap is 16", use, small)
+    twice = dict(tilings["gemv"], tile_rows=tilings["gemv"]["tile_rows"].copy())
+    real = np.flatnonzero(twice["tile_rows"] != 0xFFFFFFFF)
+    twice["tile_rows"][real[1]] = twice["tile_rows"][real[0]]
+    refused("two slots|not of its tile", "gemv", twice)
+    again = dict(tilings["gather"], tile_rows=tilings["gather"]["tile_rows"].copy())
+    slots = np.flatnonzero(again["tile_rows"] != 0xFFFFFFFF)
+    same_tile = slots[slots // again["scalars"]["rows_per_tile"] == slots[0] // again["scalars"]["rows_per_tile"]]
+    if same_tile.size > 1:  # a gather may name a row any number of times; the store sink may not
+        again["tile_rows"][same_tile[1]] = again["tile_rows"][same_tile[0]]
+        _fused.validate_host(plan, again, "gather")
+        refused("two slots", "decode", again)
+    missing = dict(tilings["gemm"], tile_rows=tilings["gemm"]["tile_rows"].copy())
+    missing["tile_rows"][np.flatnonzero(missing["tile_rows"] != 0xFFFFFFFF)[0]] = 0xFFFFFFFF
+    refused("in no tile", "gemm", missing)
+    outside = dict(tilings["decode"], tile_rows=tilings["decode"]["tile_rows"].copy())
+    outside["tile_rows"][np.flatnonzero(outside["tile_rows"] != 0xFFFFFFFF)[0]] = 96
+    refused("does not have", "decode", outside)
+    other = dict(tilings["gemv"], tile_class=(tilings["gemv"]["tile_class"] + 1) % 16)
+    refused("not of its tile's class", "gemv", other)
+    shared = position.copy()
+    shared[1] = shared[0]
+    refused("share residual position", row_pos=shared, block=block)
+    refused("interleaved residual order", row_pos=position, block=0)

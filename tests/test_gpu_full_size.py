@@ -80,6 +80,11 @@ def test_mlp_matrices_decode_digest_and_gemv(index, shape):
     # the matrix-core product of the same rows agrees within the tolerance (not bit for bit:
     # a VALU chain and an MFMA accumulate round differently)
     _check_products(t, x, (1, 8), lambda v: t.gemm(v, check=True))
+    # the M-invariant policy: the one-row call is the first row of the six-row call, bit for bit
+    t.m_invariant = True
+    y6 = t.linear(x[:6], check=True).view(torch.uint16)
+    assert torch.equal(t.linear(x[:1]).view(torch.uint16), y6[:1])
+    assert torch.equal(t.linear(x[:2]).view(torch.uint16), y6[:2])
 
 
 @pytest.mark.parametrize("name,shape", [("q", (6144, 5120)), ("k", (1024, 5120)), ("o", (5120, 6144))])

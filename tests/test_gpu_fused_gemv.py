@@ -228,3 +228,59 @@ def test_two_rows_take_the_gemv_on_short_rows_and_the_gemm_on_long_ones():
         same_as = t.gemm(x, check=True) if long_rows else t.gemv(x, check=True)
         assert torch.equal(y.view(torch.uint16), same_as.view(torch.uint16))
         assert torch.equal(t.linear(x[:1]).view(torch.uint16), t.gemv(x[:1]).view(torch.uint16))
+
+
+@pytest.mark.parametrize("shape", [(72, 5120), (40, 6144), (24, 17408)], ids=lambda s: f"{s[0]}x{s[1]}")
+def test_gemv_bits_do_not_depend_on_the_tiling(monkeypatch, shape):
+    """A row's segment sums are added as one tree per aligned block of 64 segments and the
+    blocks in order, whatever the unit shape: tilings forced to 4, 8, 16, 32 and 64 lanes per
+    row (row lengths of 80, 96 and 272 segments: blocks that are not full, too) and different
+    tile heights all give the planner's bits.  A member of a grouped launch, whose lanes per
+    row are planned for the group, therefore has the bits of its own launch."""
+    import torch
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd.bitexact_context_gpu import HipContextTensor
+    rng = np.random.default_rng(shape[1])
+    words = weight_like(rng, *shape)
+    frame = codec.encode(words)
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(2, shape[1])))).view(torch.bfloat16).cuda()
+    monkeypatch.delenv("GEOREFINE_FUSED_WAVE_TILING", raising=False)
+    planned = HipContextTensor(frame, stride=1024, device="cuda:0", fused_segment=64)
+    want = planned.gemv(x, check=True).view(torch.uint16)
+    seen = {planned._tiling(1)[3]["lanes_per_row"]}
+    for lanes, rows in ((4, 16), (8, 24), (16, 8), (32, 6), (64, 5)):
+        monkeypatch.setenv("GEOREFINE_FUSED_WAVE_TILING", f"768,{lanes},{-(-rows // (64 // lanes)) * (64 // lanes)}")
+        forced = HipContextTensor(frame, stride=1024, device="cuda:0", fused_segment=64)
+        assert forced._tiling(1)[3]["lanes_per_row"] == lanes
+        seen.add(lanes)
+        got = forced.gemv(x, check=True).view(torch.uint16)
+        assert torch.equal(got, want), f"{lanes} lanes per row"
+        assert torch.equal(forced.gemv(x[:1]).view(torch.uint16), want[:1])
+    assert seen == {4, 8, 16, 32, 64}
+
+
+def test_m_invariant_policy_makes_rows_bit_equal_across_row_counts():
+    """Under the M-invariant policy (tensor attribute, or batch_invariant=True per call) the
+    first row of a six-row call is the one-row call bit for bit, on a matrix whose rows are long
+    enough that the default routing would change kernel family between those calls; the
+    default routing is only required to stay within the tolerance."""
+    import torch
+    from georefine_amd.bitexact_context_gpu import route_rows
+    rng = np.random.default_rng(31)
+    words = weight_like(rng, 48, 8704)
+    frame, t = _tensor(words, fused_segment=64)
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(8, 8704)))).view(torch.bfloat16).cuda()
+    assert [route_rows(m, 8704) for m in (1, 2, 3, 6, 128, 129)] == ["gemv", "gemm", "gemm", "gemm", "gemm", "dense"]
+    assert [route_rows(m, 5120) for m in (1, 2, 3)] == ["gemv", "gemv", "gemm"]
+    assert {route_rows(m, 8704, True) for m in (1, 2, 6, 300)} == {"gemm"}
+    assert not t.m_invariant
+    y6 = t.linear(x[:6], batch_invariant=True, check=True)
+    for m in (1, 2, 3, 8):
+        assert torch.equal(t.linear(x[:m], batch_invariant=True).view(torch.uint16)[:min(m, 6)],
+                           y6.view(torch.uint16)[:min(m, 6)])
+    t.m_invariant = True
+    assert torch.equal(t.linear(x[:1]).view(torch.uint16), y6[:1].view(torch.uint16))
+    assert torch.equal(t.linear(x[:6]).view(torch.uint16), y6.view(torch.uint16))
+    t.m_invariant = False
+    loose = t.linear(x[:1], check=True).float()
+    assert torch.allclose(loose, y6[:1].float(), rtol=2e-2, atol=1e-3)

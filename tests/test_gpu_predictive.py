@@ -49,7 +49,10 @@ def test_ppcx_decode_matches_oracle(oracle, name, target, ref, mode, stride):
     from georefine_amd import bitexact_predictive_codec as codec
     from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
     if stride == 1 and target.size > 20000:
-        pytest.skip("one checkpoint per symbol is only exercised on the small cases")
+        # one checkpoint per symbol: every fourth row of the 65 536-word case (16 384 words: every
+        # low byte under every fourth high byte, both signs, every exponent), so that the index
+        # stays a few hundred kilobytes
+        target, ref = np.ascontiguousarray(target[::4]), np.ascontiguousarray(ref[::4])
     frame = _frame_for_mode(codec, target, ref, mode)
     expect = oracle.ppcx_decode(frame, ref)
     assert np.array_equal(expect, target)
