@@ -13,9 +13,12 @@ Prints ONE JSON line: metric = compressed bytes consumed per second (GB/s), with
 the achieved fraction of the 8 TB/s HBM roofline for the dominant kernel and a
 CPU baseline (the CPU oracle's decode + matvec on the host cores).
 
-After the warm-up, K eager steps give the per-launch durations (HIP events on the
-launch stream); the K timed steps are then replays of one HIP graph of a step
-(--no-graph times the eager steps instead).
+The K timed steps are replays of HIP graphs of consecutive steps (--no-graph times eager
+steps instead); the per-launch durations come from device timestamps inside a graph of the
+same steps.  The default run adds the other configurations of the metric to the same line:
+`batch64` (the MLP step at batch 64, fused GEMM), `attention` (q/k/v/o at batch 1..128 through
+the batch-invariant GEMM), `ppcx` (a predictive frame, products with 1 and 96 rows) and `stack`
+(every coded linear of a 64-layer model resident at once, one pass at batch 64).
 """
 from __future__ import annotations
 
@@ -63,19 +66,38 @@ def synth_weights(index, rows, cols):
     return out
 
 
+def synth_weights_f32(seed, rows, cols):
+    """The same distribution drawn in float32 (twice as fast; other values than synth_weights
+    gives for a seed): for the whole-stack workload, whose set-up is mostly this."""
+    rng = np.random.default_rng(seed)
+    out = np.empty((rows, cols), dtype=np.uint16)
+    scale = rng.lognormal(0.0, 0.5, size=(rows, 1)).astype(np.float32) * np.float32(0.02)
+    step = 4096
+    for lo in range(0, rows, step):
+        hi = min(rows, lo + step)
+        w = rng.standard_normal(size=(hi - lo, cols), dtype=np.float32) * scale[lo:hi]
+        mask = rng.random((hi - lo, cols), dtype=np.float32) < np.float32(1e-3)
+        w = np.where(mask, w * np.float32(10.0), w)
+        out[lo:hi] = bf16_words(w)
+    return out
+
+
 GEMV_UP_TO = 2  # rows linear() gives to the vector-ALU kernel; read from HipContextTensor once it is imported
 
 
-def algorithmic_bytes(t, m):
-    """Bytes one fused GEMV launch has to touch once: both streams, the fused index,
-    the per-class lookup tables, labels, activations and outputs."""
+def algorithmic_bytes(t, m, gemm=None):
+    """Bytes one fused GEMV / GEMM launch has to touch once: both streams, the fused index,
+    the per-class lookup tables, labels, activations and outputs.  ``gemm``: the launch runs
+    the matrix-core kernel (default: from the row count, as linear() routes)."""
     b = t.buffers
     n = lambda k: b[k].numel() * b[k].element_size()
     rows, cols = t.shape
     # (the resident residual array starts every row class on a multiple of 16 rows: the rows it
     # holds beyond the matrix's are never read and are not counted)
     payload = t._main_bytes + min(n("residual_stream"), rows * cols * 3 // 4)
-    _, tile_rows, tile_class, _ = t._tiling(m) if m <= GEMV_UP_TO else t._gemm_tiling()
+    if gemm is None:
+        gemm = m > GEMV_UP_TO
+    _, tile_rows, tile_class, _ = t._gemm_tiling() if gemm else t._tiling(m)
     index = (n("fused_seg_state") + n("fused_seg_offset") + tile_rows.numel() * tile_rows.element_size()
              + tile_class.numel() * tile_class.element_size() + (n("row_pos") if "row_pos" in b else 0))
     tables = n("fused_lut") + n("fused_tab")
@@ -226,19 +248,135 @@ def cpu_baseline(frames, words_of, x_words, min_seconds=8.0, max_frames=12):
     return result
 
 
-def run_predictive(args):
+def launch_fields(alg_total, ms):
+    gbps = alg_total / (ms * 1e-3) / 1e9
+    return {"ms": round(ms, 4), "alg_bytes": int(alg_total), "GBps": round(gbps, 2),
+            "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+
+
+def roofline_fields(alg_total, ms, kernel, traffic=None, traffic_source=None):
+    gbps = alg_total / (ms * 1e-3) / 1e9
+    out = {"bound": "hbm", "achieved": round(gbps, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+           "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": traffic, "kernel": kernel}
+    if traffic_source:
+        out["traffic_source"] = traffic_source
+    return out
+
+
+ATTENTION = {"q": (6144, 5120), "k": (1024, 5120), "v": (1024, 5120), "o": (5120, 6144)}
+ATTENTION_BATCHES = (1, 8, 32, 64, 128)
+
+
+def run_attention(args, as_dict=False):
+    """The attention projections -- q 5120->6144, k/v 5120->1024, o 6144->5120 -- at batch 1, 8,
+    32, 64 and 128 through the batch-invariant route: every row count runs the matrix-core GEMM
+    (q, k and v, which take the same rows, in one launch), and a row's output bits are checked
+    to be the same at every batch.  The batch-1 time of the default route (the VALU GEMV, whose
+    rows are bit-equal among themselves only) is reported beside it."""
+    import torch
+    from georefine_amd import bitexact_context_codec as codec
+    from georefine_amd.bitexact_context_gpu import HipContextTensor, HipLinearGroup
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs a ROCm GPU")
+    t0 = time.perf_counter()
+    base = {}
+    for i, (name, (rows, cols)) in enumerate(ATTENTION.items()):
+        # q, k and v share a launch, so they are indexed at one segment length
+        base[name] = HipContextTensor(codec.encode(synth_weights(10 + i, rows, cols)), stride=1024, device="cuda:0",
+                                      fused_segment=64)
+        if base[name].fused is None:
+            sys.exit(f"bench.py: {name} is not eligible for the fused kernels: {base[name].fused_reason}")
+    resident = sum(t.resident_bytes for t in base.values())
+    copies = max(1, -(-2 * LAST_LEVEL_CACHE_BYTES // resident))
+    sets = [base] + [{k: v.clone() for k, v in base.items()} for _ in range(copies - 1)]
+    groups = [HipLinearGroup([s_["q"], s_["k"], s_["v"]]) for s_ in sets]
+    log(f"attention: 4 matrices coded and resident in {time.perf_counter() - t0:.1f}s, {copies} device copies in turn")
+    rng = np.random.default_rng(7)
+    x = {k: torch.from_numpy(bf16_words(rng.normal(0, 1, size=(128, k)))).view(torch.bfloat16).cuda() for k in (5120, 6144)}
+    steps, warmup = max(10, args.steps // 2), max(4, args.warmup // 4)
+
+    def errors():
+        return sorted({n_ for s_ in sets for n_, t in s_.items() if t.error.item()}
+                      | {"q+k+v" for g in groups if g.error.item()})
+
+    def per_layer(m, invariant):
+        return [[("q+k+v", ["q", "k", "v"], lambda g=g: g.linear(x[5120][:m], batch_invariant=invariant)),
+                 ("o", ["o"], lambda t=s_["o"]: t.linear(x[6144][:m], batch_invariant=invariant))]
+                for s_, g in zip(sets, groups)]
+
+    def alg_of(m, gemm):
+        parts = {n_: algorithmic_bytes(base[n_], m, gemm=gemm)["total"] for n_ in ATTENTION}
+        return {"q+k+v": parts["q"] + parts["k"] + parts["v"] - 2 * m * 5120 * 2, "o": parts["o"]}
+
+    def one(m, invariant):
+        ms_step, per_ms, launch, timing, clocks = time_launches(torch, per_layer(m, invariant), steps, warmup,
+                                                                args.graph, errors)
+        alg = alg_of(m, invariant or m > GEMV_UP_TO)
+        dom = max(alg, key=lambda k: alg[k])
+        gemm = invariant or m > GEMV_UP_TO
+        kernel = ("grf::fused_gemm_group_kernel / fused_gemm_wide_group_kernel<grf::SegmentWalkT<false>, MT, 1>" if gemm
+                  else f"grf::fused_wave_group_kernel<grf::SegmentWalkT<false>, {min(m, 2)}, 1>")
+        total = sum(alg.values())
+        return {"ms_per_pass": round(ms_step, 4), "GBps": round(total / (ms_step * 1e-3) / 1e9, 2), "launch": launch,
+                "rows_per_s": round(m / (ms_step * 1e-3), 1), **clocks,
+                "per_kernel": {k: launch_fields(alg[k], per_ms[k]) for k in per_ms},
+                "roofline": roofline_fields(alg[dom], per_ms[dom], f"{kernel} on {dom}")}, timing
+
+    # a row's bits do not depend on the batch it arrives in: rows of every batch against batch 128
+    full = [groups[0].linear(x[5120], batch_invariant=True, check=True), base["o"].linear(x[6144], batch_invariant=True,
+                                                                                          check=True)]
+    equal = True
+    for m in ATTENTION_BATCHES:
+        ys = groups[0].linear(x[5120][:m], batch_invariant=True) + [base["o"].linear(x[6144][:m], batch_invariant=True)]
+        want = list(full[0]) + [full[1]]
+        equal = equal and all(torch.equal(y.view(torch.uint16), w[:m].view(torch.uint16)) for y, w in zip(ys, want))
+    if not equal:
+        sys.exit("bench.py: attention rows differ between batches on the batch-invariant route")
+    batches, timing = {}, ""
+    for m in ATTENTION_BATCHES:
+        batches[str(m)], timing = one(m, True)
+        log(f"attention batch {m}: {batches[str(m)]['ms_per_pass']} ms per pass")
+    default1, _ = one(1, False)
+    result = {
+        "config": {"workload": "attention projections q 5120->6144, k/v 5120->1024, o 6144->5120 (BCTX (16,4) frames), "
+                               "q/k/v in one launch, o in another; every batch through the matrix-core GEMM "
+                               "(batch-invariant route)",
+                   "batches": list(ATTENTION_BATCHES), "steps": steps, "warmup": warmup, "layer_copies": copies,
+                   "per_kernel_timing": timing},
+        "coded_resident_bytes": resident, "dense_bf16_bytes": sum(2 * r * c for r, c in ATTENTION.values()),
+        "rows_bit_equal_across_batches": bool(equal),
+        "batch_invariant": batches,
+        "default_route_batch1": default1,
+    }
+    sets.clear()
+    groups.clear()
+    base.clear()
+    torch.cuda.empty_cache()
+    if as_dict:
+        return result
+    print(json.dumps({"metric": "compressed-weight decode-GEMV GB/s", "value": batches["1"]["GBps"], "unit": "GB/s",
+                      "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": batches["1"]["ms_per_pass"],
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "u32 rANS state / bf16 weights / fp32 accumulate", "data": "synthetic", **result}), flush=True)
+
+
+PPCX_BATCHES = (1, 96)
+
+
+def run_predictive(args, as_dict=False):
     """A 5120 x 17408 target coded (PPCX) against a reference that is the target plus N(0, 0.002)
     noise, as a loaded model serves it: the tensor keeps the 4-bit context plane of its
     reference from load on, so no reference is resident or decoded.  One step = the product of
-    the coded target with `--batch` activation rows (default 96 = 16 users x (5 draft tokens
-    + 1), the verify shape): the activations packed, then the fused GEMM (one row: the GEMV)."""
+    the coded target with the activation rows, on three resident copies in turn: one row (the
+    fused GEMV) and 96 rows = 16 users x (5 draft tokens + 1), the verify shape (activations
+    packed, then the fused GEMM); --batch picks a single row count."""
     import torch
     from georefine_amd import bitexact_predictive_codec as ppcx
     from georefine_amd.bitexact_predictive_gpu import HipPredictiveTensor
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: needs a ROCm GPU")
-    m = args.batch or 96
+    batches = (args.batch,) if args.batch and not as_dict else PPCX_BATCHES
     rows, cols = 5120, 17408
     target = synth_weights(2, rows, cols)
     noise = np.random.default_rng(5).normal(0, 0.002, size=target.shape).astype(np.float32)
@@ -250,237 +388,283 @@ def run_predictive(args):
     if t.fused is None:
         sys.exit(f"bench.py: the frame is not eligible for the fused kernels: {t.fused_reason}")
     log(f"PPCX frame {len(frame)} B ({8 * len(frame) / target.size:.3f} bit/weight) mode {t.mode}; setup {time.perf_counter() - t0:.1f}s")
-    copies = [(t, None)]
-    for _ in range(2):  # three targets in rotation: more bytes than the caches hold
-        copies.append((HipPredictiveTensor(frame, ref, stride=1024, device="cuda:0"), None))
-    x = torch.from_numpy(bf16_words(np.random.default_rng(7).normal(0, 1, size=(m, cols)))).view(torch.bfloat16).cuda()
-
-    def step():
-        return [c.linear(r, x) for c, r in copies]
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+    copies = [t, t.clone(), t.clone()]  # three targets in rotation: more bytes than the caches hold
+    steps, warmup = (args.steps, args.warmup) if not as_dict else (max(10, args.steps // 2), max(4, args.warmup // 4))
+    x_all = torch.from_numpy(bf16_words(np.random.default_rng(7).normal(0, 1, size=(max(batches), cols)))).view(torch.bfloat16).cuda()
     dense = torch.from_numpy(target).view(torch.bfloat16).cuda().float()
-    want = torch.nn.functional.linear(x.float(), dense)
-    scale = torch.nn.functional.linear(x.float().abs(), dense.abs())
-    got = copies[0][0].linear(copies[0][1], x, check=True).float()
-    if not bool((got - want).abs().le(1e-2 * want.abs().clamp_min(1e-3 * scale)).all()):
-        sys.exit("bench.py: the fused product is outside 1e-2 of the dense product")
+    for m in batches:
+        want = torch.nn.functional.linear(x_all[:m].float(), dense)
+        scale = torch.nn.functional.linear(x_all[:m].float().abs(), dense.abs())
+        got = t.linear(None, x_all[:m], check=True).float()
+        if not bool((got - want).abs().le(1e-2 * want.abs().clamp_min(1e-3 * scale)).all()):
+            sys.exit(f"bench.py: the fused product with {m} rows is outside 1e-2 of the dense product")
     del dense, want, scale, got
-    events = []
-    torch.cuda.synchronize()
-    wall0 = time.perf_counter()
-    for _ in range(args.steps):
-        for c, r in copies:
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            c.linear(r, x)
-            b.record()
-            events.append((a, b))
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - wall0
-    launch = "eager"
-    if args.graph:
-        try:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                step()
-            graph.replay()
-            torch.cuda.synchronize()
-        except Exception as exc:
-            log(f"graph capture failed ({exc}); reporting the eager steps")
-        else:
-            wall0 = time.perf_counter()
-            for _ in range(args.steps):
-                graph.replay()
-            torch.cuda.synchronize()
-            wall = time.perf_counter() - wall0
-            launch = "hip graph replay"
-    for c, _ in copies:
-        if c.error.item():
-            sys.exit("bench.py: decoder error word set")
-    ms_product = float(np.mean([a.elapsed_time(b) for a, b in events]))
-    # bytes one product has to touch once: everything the tensor keeps on the device (the coded
-    # target, its index and tables, the 4-bit context plane of the reference), activations, outputs
     coded = t.resident_bytes
-    alg = coded + m * cols * 2 + m * rows * 2
-    ms_per_step = wall / args.steps * 1e3
-    value = len(copies) * alg / (ms_per_step * 1e-3) / 1e9
-    print(json.dumps({
-        "metric": "compressed-weight decode-GEMV GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
-        "data": "synthetic",
-        "config": {"workload": f"PPCX target 5120x17408 coded against a reference (target + N(0, 0.002)), product with "
-                               f"{m} activation rows as served: contexts of the reference resident as a 4-bit plane, no "
-                               f"dense reference; three targets in rotation", "batch": m, "launch": launch},
-        "ms_per_product": round(ms_per_step / len(copies), 4), "ms_per_product_eager_events": round(ms_product, 4),
-        "frame_bytes": len(frame), "resident_bytes": coded,
-        "context_plane_bytes": target.size // 2,
-        "algorithmic_bytes_per_product": alg, "tok_s_equiv_rows_per_s": round(m * len(copies) / (ms_per_step * 1e-3), 1),
-        # per product: the step's wall time over its products (under a graph the launches follow one
-        # another without host gaps; events around single eager launches, kept beside it, include them)
-        "roofline": {"bound": "hbm", "achieved": round(value, 2), "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": round(value / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": ("grf::fused_wave_kernel<PpcxWalk, 1, SCAN>" if m == 1 else
-                                "pack_activations_kernel + grf::fused_gemm_kernel / fused_gemm_wide_kernel<PpcxWalk, MT, SCAN>")
-                               + " (a product's share of the step)"},
-    }), flush=True)
+    out = {}
+    for m in batches:
+        x = x_all[:m]
+        per_layer = [[("product", ["target"], lambda c=c: c.linear(None, x))] for c in copies]
+        ms_step, per_ms, launch, timing, clocks = time_launches(
+            torch, per_layer, steps, warmup, args.graph, lambda: ["target"] if any(c.error.item() for c in copies) else [])
+        # bytes one product has to touch once: everything the tensor keeps on the device (the coded
+        # target, its index and tables, the 4-bit context plane of the reference), activations, outputs
+        alg = coded + m * cols * 2 + m * rows * 2
+        kernel = ("grf::fused_wave_kernel<PpcxWalk, 1, SCAN>" if m == 1 else
+                  "pack_activations_kernel + grf::fused_gemm_kernel / fused_gemm_wide_kernel<PpcxWalk, MT, SCAN> (+ gemm_sum_parts_kernel)")
+        traffic, source = recorded_traffic(False, m, kernel, prefix="ppcx")
+        out[str(m)] = {"ms_per_product": round(ms_step, 4), "launch": launch, "per_kernel_timing": timing, **clocks,
+                       "GBps": round(alg / (ms_step * 1e-3) / 1e9, 2), "rows_per_s": round(m / (ms_step * 1e-3), 1),
+                       "algorithmic_bytes_per_product": alg,
+                       "roofline": roofline_fields(alg, per_ms["product"], kernel + " (all launches of a product)", traffic, source)}
+        log(f"ppcx batch {m}: {ms_step:.4f} ms per product")
+    n = target.size
+    result = {
+        "config": {"workload": "PPCX target 5120x17408 coded against a reference (target + N(0, 0.002)), products as "
+                               "served: contexts of the reference resident as a 4-bit plane, no dense reference; three "
+                               "resident copies in turn", "batches": list(batches), "steps": steps, "warmup": warmup},
+        "frame_bytes": len(frame), "frame_bits_per_weight": round(8 * len(frame) / n, 3),
+        "resident_bytes": coded, "resident_bits_per_weight": round(8 * coded / n, 3),
+        "context_plane_bytes": n // 2, "frame_mode": t.mode, "resident_mode": t.resident_mode,
+        "batch": out,
+    }
+    copies.clear()
+    del t
+    torch.cuda.empty_cache()
+    if as_dict:
+        return result
+    first = out[str(batches[-1])]
+    print(json.dumps({"metric": "compressed-weight decode-GEMV GB/s", "value": first["GBps"], "unit": "GB/s", "n_gpus": 1,
+                      "steps": steps, "warmup": warmup, "ms_per_step": first["ms_per_product"], "higher_is_better": True,
+                      "scaling": "weak", "vs_baseline": None, "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
+                      "data": "synthetic", **result, "roofline": first["roofline"]}), flush=True)
 
 
-def run_stack(args, as_dict=False):
-    """Every coded linear of a 64-layer stack resident at once, one pass at batch 64.
+# The whole-stack workload.  "qwen": the linear shapes of the 27B model the reference serves
+# (GCR/bitexact_context_mtp.py:244-260 and the reference's kernel tuning tables): 16 full-attention
+# layers, 48 linear-attention layers, the vocabulary matrix twice (embedding and head).
+# "baseline": 64 layers of the attention and MLP shapes the other workloads use.
+MLP3 = {"gate": (17408, 5120), "up": (17408, 5120), "down": (5120, 17408)}
+STACKS = {
+    "qwen": {"attn": dict({"q": (12288, 5120), "k": (1024, 5120), "v": (1024, 5120), "o": (5120, 6144)}, **MLP3),
+             "gdn": dict({"in_proj": (16480, 5120), "out_proj": (5120, 6144)}, **MLP3),
+             "vocab": (248320, 5120), "attn_every": 4},
+    "baseline": {"attn": dict(LAYER), "gdn": None, "vocab": None, "attn_every": 1},
+}
+SHARED_INPUT = (("q", "k", "v"), ("gate", "up"))  # siblings that take the same rows: one launch each
 
-    Each layer holds q, k, v, o, gate, up and down as BCTX frames.  `--distinct-layers`
-    layers are generated and encoded from their own seeds; the others are device copies of
-    those in rotation (their own buffers, so a pass streams every layer's bytes from HBM,
-    but no further host encoding)."""
-    import torch
-    from concurrent.futures import ThreadPoolExecutor
+
+def stack_job(job):
+    """Worker process: one matrix drawn, encoded, validated, indexed and laid out for the kernels
+    (HipContextTensor.host_prepare needs no GPU); the result goes to a file."""
+    import pickle
     from georefine_amd import bitexact_context_codec as codec
     from georefine_amd.bitexact_context_gpu import HipContextTensor
+    key, seed, (rows, cols), residual, folder = job
+    frame = codec.encode(synth_weights_f32(seed, rows, cols), residual=residual)
+    prepared = HipContextTensor.host_prepare(frame, stride=1024, fused_segment=64)
+    path = os.path.join(folder, "_".join(map(str, key)) + ".pickle")
+    with open(path, "wb") as f:
+        pickle.dump((len(frame), prepared), f, protocol=pickle.HIGHEST_PROTOCOL)
+    return key, path
+
+
+class StackPrep:
+    """Host half of the whole-stack workload in worker processes: every distinct matrix is drawn,
+    encoded, validated, indexed and laid out for the kernels; the device objects are
+    constructed later from the results, by the process that owns the GPU.  Started before that
+    process touches the GPU (the workers are forked, and never touch it), it runs beside the
+    other workloads' GPU phases.  Processes, not threads: a busy thread would hold the
+    interpreter's lock for milliseconds at a time, which the timed regions of the other
+    workloads, themselves a few milliseconds long, cannot afford."""
+
+    def __init__(self, args):
+        import atexit
+        import multiprocessing
+        import shutil
+        import tempfile
+        from concurrent.futures import ProcessPoolExecutor
+        spec = STACKS[args.stack_shapes]
+        self.spec, self.t0 = spec, time.perf_counter()
+        kinds = [k for k in ("attn", "gdn") if spec[k]]
+        n_attn = sum(1 for i in range(args.layers) if spec["gdn"] is None or i % spec["attn_every"] == spec["attn_every"] - 1)
+        self.counts = {"attn": n_attn, "gdn": args.layers - n_attn}
+        self.distinct = {k: max(1, min(args.distinct_layers, self.counts[k])) for k in kinds if self.counts[k]}
+        self.folder = tempfile.mkdtemp(prefix="georefine_bench_", dir="/dev/shm" if os.path.isdir("/dev/shm") else None)
+        atexit.register(shutil.rmtree, self.folder, ignore_errors=True)
+        jobs = []
+        if spec["vocab"]:
+            jobs.append((("vocab", 0, "vocab"), 7777, spec["vocab"], "raw6", self.folder))  # the longest job first
+        for kind, count in self.distinct.items():
+            for d in range(count):
+                for j, (name, shape) in enumerate(spec[kind].items()):
+                    jobs.append(((kind, d, name), 100000 * (1 + kinds.index(kind)) + 100 * d + j, shape, "auto", self.folder))
+        # (the box's share of host cores is 16 whatever it reports; half of them)
+        self.pool = ProcessPoolExecutor(max_workers=max(1, min(8, (os.cpu_count() or 2) // 2)),
+                                        mp_context=multiprocessing.get_context("fork"))
+        self.futures = [self.pool.submit(stack_job, job) for job in jobs]
+        self.done = None
+
+    def results(self):
+        """{key: (frame bytes, prepared)}; waits for the workers."""
+        import pickle
+        if self.done is None:
+            paths = dict(f.result() for f in self.futures)
+            self.pool.shutdown()
+            log(f"stack: {len(paths)} distinct matrices drawn, encoded and indexed {time.perf_counter() - self.t0:.1f}s "
+                f"after the start")
+            self.done = paths
+        out = {}
+        for key, path in self.done.items():
+            with open(path, "rb") as f:
+                out[key] = pickle.load(f)
+            os.unlink(path)
+        return out
+
+    def wait(self):
+        if self.done is None:
+            self.done = dict(f.result() for f in self.futures)
+            self.pool.shutdown()
+            log(f"stack: {len(self.done)} distinct matrices drawn, encoded and indexed {time.perf_counter() - self.t0:.1f}s "
+                f"after the start")
+
+
+def run_stack(args, as_dict=False, prep=None):
+    """Every coded linear of a 64-layer model resident at once, one pass at batch 64: a row
+    gather from the embedding matrix, every layer's projections (siblings that take the same
+    rows share a launch), the head.  `--distinct-layers` layers of each kind are drawn and
+    encoded from their own seeds; the others are device copies of those in rotation (their own
+    buffers, so a pass streams every layer's bytes from HBM, but no further host encoding)."""
+    prep = prep or StackPrep(args)  # (forks its workers: before this process touches the GPU)
+    import torch
+    from georefine_amd.bitexact_context_gpu import HipContextTensor, HipLinearGroup
     global GEMV_UP_TO
     GEMV_UP_TO = HipContextTensor.GEMV_UP_TO
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: needs a ROCm GPU")
     m = args.batch or 64
+    spec = prep.spec
+    done = prep.results()
     t0 = time.perf_counter()
-
-    def coded(job):
-        layer, j, name = job
-        rows, cols = LAYER[name]
-        return job, codec.encode(synth_weights(100 * layer + j, rows, cols))
-
-    jobs = [(d, j, name) for d in range(args.distinct_layers) for j, name in enumerate(LAYER)]
-    with ThreadPoolExecutor(max_workers=min(8, len(jobs))) as pool:
-        frames = dict(pool.map(coded, jobs))
-    log(f"encoded {len(jobs)} matrices in {time.perf_counter() - t0:.1f}s")
-    t0 = time.perf_counter()
-    base = {}
-    for job in jobs:
-        # one segment length for every matrix, so that q/k/v and gate/up can share a launch
-        t = HipContextTensor(frames[job], stride=1024, device="cuda:0", fused_segment=64)
+    base, frame_len = {}, {}
+    for key, (frame_bytes, prepared) in done.items():
+        t = HipContextTensor(b"", stride=1024, device="cuda:0", prepared=prepared)
         if t.fused is None:
-            sys.exit(f"bench.py: {job} is not eligible for the fused kernels: {t.fused_reason}")
-        t._gemm_tiling()
-        base[job] = t
-    log(f"indexed and uploaded in {time.perf_counter() - t0:.1f}s")
-    layers = []
+            sys.exit(f"bench.py: {key} is not eligible for the fused kernels: {t.fused_reason}")
+        base[key], frame_len[key] = t, frame_bytes
+    done.clear()
+    log(f"stack: uploaded in {time.perf_counter() - t0:.1f}s")
+    gemm = m > GEMV_UP_TO
+    layers, used = [], {k: 0 for k in prep.distinct}
     for i in range(args.layers):
-        d = i % args.distinct_layers
-        src = {name: base[(d, j, name)] for j, name in enumerate(LAYER)}
-        layers.append(src if i < args.distinct_layers else {k: v.clone() for k, v in src.items()})
-    for layer in layers:
-        for t in layer.values():
-            t._gemm_tiling() if m > GEMV_UP_TO else t._tiling(m)
+        kind = "attn" if spec["gdn"] is None or i % spec["attn_every"] == spec["attn_every"] - 1 else "gdn"
+        d = used[kind] % prep.distinct[kind]
+        first = used[kind] < prep.distinct[kind]
+        used[kind] += 1
+        src = {name: base[(kind, d, name)] for name in spec[kind]}
+        layers.append((kind, src if first else {k: v.clone() for k, v in src.items()}))
+    vocab = None
+    if spec["vocab"]:
+        head = base[("vocab", 0, "vocab")]
+        vocab = {"embedding": head.clone(), "head": head}
+    everything = [t for _, layer in layers for t in layer.values()] + (list(vocab.values()) if vocab else [])
+    for t in everything:
+        t._gemm_tiling() if gemm else t._tiling(m)
     torch.cuda.synchronize()
-    frame_bytes = sum(t.frame_bytes for layer in layers for t in layer.values())
-    resident = sum(t.resident_bytes for layer in layers for t in layer.values())
-    dense = sum(2 * r * c for r, c in LAYER.values()) * args.layers
+    frame_bytes = 0
+    # frame bytes of the whole stack: every layer's frames (copies are the same frames again)
+    seen = {k: 0 for k in prep.distinct}
+    for kind, _ in layers:
+        d = seen[kind] % prep.distinct[kind]
+        seen[kind] += 1
+        frame_bytes += sum(frame_len[(kind, d, name)] for name in spec[kind])
+    if vocab:
+        frame_bytes += 2 * frame_len[("vocab", 0, "vocab")]
+    resident = sum(t.resident_bytes for t in everything)
+    dense = sum(2 * t.shape[0] * t.shape[1] for t in everything)
     log(f"{args.layers} layers resident: {dense} BF16 bytes as {frame_bytes} frame bytes, {resident} device bytes; "
         f"torch reports {torch.cuda.memory_allocated()} allocated")
 
     rng = np.random.default_rng(7)
-    x = {k: torch.from_numpy(bf16_words(rng.normal(0, 1, size=(m, k)))).view(torch.bfloat16).cuda()
-         for k in {c for _, c in LAYER.values()}}
+    widths = {t.shape[1] for t in everything}
+    x = {k: torch.from_numpy(bf16_words(rng.normal(0, 1, size=(m, k)))).view(torch.bfloat16).cuda() for k in widths}
+    ids = torch.from_numpy(rng.integers(0, spec["vocab"][0], size=m)).cuda() if vocab else None
 
-    # q, k, v read the same activations, gate and up too: each group is one launch
-    from georefine_amd.bitexact_context_gpu import HipLinearGroup
-    names = (("q", "k", "v"), ("o",), ("gate", "up"), ("down",))
     grouped = not args.no_groups
-    groups = [[HipLinearGroup([layer[n] for n in g]) if grouped and len(g) > 1 else None for g in names]
-              for layer in layers] if grouped else None
+    launches = []  # (label, members as tensors, callable) of one pass
+    if vocab:
+        launches.append(("embedding", [], lambda t=vocab["embedding"]: t.gather_rows(ids, check=False, validate=False)))
+    for kind, layer in layers:
+        rest = list(layer)
+        for sib in SHARED_INPUT:
+            if grouped and all(n_ in layer for n_ in sib):
+                g = HipLinearGroup([layer[n_] for n_ in sib])
+                launches.append(("+".join(sib), [layer[n_] for n_ in sib],
+                                 lambda g=g, w=layer[sib[0]].shape[1]: g.linear(x[w], batch_invariant=gemm)))
+                rest = [n_ for n_ in rest if n_ not in sib]
+        for name in rest:
+            launches.append((name, [layer[name]], lambda t=layer[name]: t.linear(x[t.shape[1]], batch_invariant=gemm)))
+    if vocab:
+        launches.append(("head", [vocab["head"]], lambda t=vocab["head"]: t.linear(x[t.shape[1]], batch_invariant=gemm)))
+    # (a pass in model order: the order above is by layer, siblings first -- every launch reads its own bytes,
+    # so the order changes nothing that is measured)
     torch.cuda.synchronize()
 
-    def step():
-        for i, layer in enumerate(layers):
-            for j, g in enumerate(names):
-                xin = x[LAYER[g[0]][1]]
-                if grouped and len(g) > 1:
-                    groups[i][j].linear(xin, batch_invariant=m > GEMV_UP_TO)
-                else:
-                    for name in g:
-                        layer[name].linear(xin, batch_invariant=m > GEMV_UP_TO)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # per-launch durations of the first layer's kernels, on the stream they run on
-    probes = {name: [] for name in LAYER}
-    wall0 = time.perf_counter()
-    for _ in range(args.steps):
-        for i, layer in enumerate(layers):
-            for name, t in layer.items():
-                if i == 0:
-                    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    a.record()
-                t.linear(x[LAYER[name][1]], batch_invariant=m > GEMV_UP_TO)
-                if i == 0:
-                    b.record()
-                    probes[name].append((a, b))
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - wall0
-    launch = "eager"
-    if args.graph:
-        try:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                step()
-            graph.replay()
-            torch.cuda.synchronize()
-        except Exception as exc:
-            log(f"graph capture failed ({exc}); reporting the eager steps")
+    ms_per_step, per_ms, launch, timing, clocks = time_launches(
+        torch, [launches], args.steps, args.warmup, args.graph,
+        lambda: sorted({label for label, members, _ in launches for t in members if t.error.item()}))
+    alg, count = {}, {}
+    for label, members, _ in launches:
+        if label == "embedding":  # the rows gathered: their share of both streams, written dense
+            t = vocab["embedding"]
+            total = int(m * (algorithmic_bytes(t, 0, gemm=False)["payload"] / t.shape[0] + 2 * t.shape[1]))
         else:
-            wall0 = time.perf_counter()
-            for _ in range(args.steps):
-                graph.replay()
-            torch.cuda.synchronize()
-            wall = time.perf_counter() - wall0
-            launch = "hip graph replay"
-    for layer in layers:
-        for name, t in layer.items():
-            if t.error.item():
-                sys.exit(f"bench.py: decoder error word set for {name}")
-    ms = {name: float(np.mean([a.elapsed_time(b) for a, b in ev])) for name, ev in probes.items()}
-    alg = {name: algorithmic_bytes(layers[0][name], m) for name in LAYER}
-    step_bytes = sum(algorithmic_bytes(t, m)["total"] for layer in layers[:args.distinct_layers] for t in layer.values())
-    step_bytes = step_bytes * args.layers // args.distinct_layers
-    ms_per_step = wall / args.steps * 1e3
+            total = sum(algorithmic_bytes(t, m, gemm=gemm)["total"] for t in members) - (len(members) - 1) * m * members[0].shape[1] * 2
+        alg[label] = alg.get(label, 0) + total
+        count[label] = count.get(label, 0) + 1
+    step_bytes = sum(alg.values())
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
-    dom = max(LAYER, key=lambda n_: ms[n_])
-    achieved = alg[dom]["total"] / (ms[dom] * 1e-3) / 1e9
-    kernel = kernel_name(False, m, False, 64)  # (of the ungrouped launch that took longest)
+    share = {label: per_ms[label] * count[label] for label in per_ms}  # ms of a pass spent in each kind of launch
+    dom = max((l_ for l_ in alg if l_ != "embedding"), key=lambda l_: alg[l_])  # the kind that moves most bytes
+    kernel = ("grf::fused_gemm_group_kernel<grf::SegmentWalkT<false>, MT, 1>" if "+" in dom else
+              "grf::fused_gemm_kernel<grf::SegmentWalkT<false>, MT, 1>") if gemm else kernel_name(False, m, "+" in dom, 64)
+    shapes_text = "; ".join(f"{k}: " + ", ".join(f"{n_} {c}->{r}" for n_, (r, c) in spec[k].items())
+                            for k in ("attn", "gdn") if spec[k])
     result = {
         "metric": "compressed-weight decode-GEMV GB/s", "value": round(value, 2), "unit": "GB/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "u32 rANS state / bf16 weights / fp32 accumulate",
         "data": "synthetic",
-        "config": {"workload": f"whole stack resident: {args.layers} layers x (q 5120->6144, k/v 5120->1024, o 6144->5120, "
-                               f"gate/up 5120->17408, down 17408->5120), one pass through every coded linear at batch {m}; "
-                               f"{dense / 1e9:.1f} GB of dense BF16 held as {frame_bytes / 1e9:.1f} GB of frames "
-                               f"(no embedding or head matrix in the stack)",
-                   "batch": m, "layers": args.layers, "distinct_layers": args.distinct_layers,
-                   "linears": args.layers * len(LAYER), "launch": launch,
-                   "launches": "q/k/v and gate/up grouped" if grouped else "one per linear"},
+        "config": {"workload": f"whole stack resident: {args.layers} layers ({prep.counts['attn']} attention, "
+                               f"{prep.counts['gdn']} linear-attention; {shapes_text})"
+                               + (f", embedding and head {spec['vocab'][0]}x{spec['vocab'][1]}" if vocab else "")
+                               + f"; one pass through every coded linear at batch {m} (the embedding: a gather of "
+                                 f"{m} rows); {dense / 1e9:.1f} GB of dense BF16 held as {frame_bytes / 1e9:.1f} GB of frames",
+                   "shapes": args.stack_shapes, "batch": m, "layers": args.layers,
+                   "distinct_layers": dict(prep.distinct), "linears": len(everything), "launches_per_pass": len(launches),
+                   "launch": launch, "launches": "siblings that take the same rows share a launch" if grouped else "one per linear",
+                   "per_kernel_timing": timing,
+                   "vocabulary_frame": "mode 0 (packed 6-bit residuals written directly); the embedding is a device "
+                                       "copy of the head's frame" if vocab else None},
         "dense_bf16_bytes": dense, "frame_bytes": frame_bytes, "resident_device_bytes": resident,
         "algorithmic_bytes_per_step": step_bytes,
         "effective_bf16_GBps": round(dense / (ms_per_step * 1e-3) / 1e9, 2),
         "tok_s_equiv": round(m / (ms_per_step * 1e-3), 1),
-        "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
-        "per_kernel": {n_: {"ms": round(ms[n_], 4), "alg_bytes": alg[n_]["total"],
-                            "GBps": round(alg[n_]["total"] / (ms[n_] * 1e-3) / 1e9, 2)} for n_ in LAYER},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None, "kernel": f"{kernel} on {dom}"},
+        "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2), **clocks,
+        "per_kernel": {l_: dict(launch_fields(alg[l_] / count[l_], per_ms[l_]), launches=count[l_],
+                                ms_of_pass=round(share[l_], 3)) for l_ in per_ms},
+        "roofline": roofline_fields(alg[dom] / count[dom], per_ms[dom], f"{kernel} on {dom} ({count[dom]} launches per pass)"),
     }
     if as_dict:  # as a key of the headline line: the fields that line carries itself are left out
         for key in ("metric", "unit", "n_gpus", "higher_is_better", "scaling", "vs_baseline", "dtype", "data"):
             result.pop(key)
-        layers.clear()
-        base.clear()
-        groups = graph = None
-        torch.cuda.empty_cache()
+    launches.clear()
+    layers.clear()
+    base.clear()
+    everything.clear()
+    vocab = None
+    torch.cuda.empty_cache()
+    if as_dict:
         return result
     print(json.dumps(result), flush=True)
 
@@ -501,21 +685,25 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 128 MiB read + 128 MiB write elementwise kernel three times, so that a "
                          "counter profile of this command holds a kernel of known traffic to scale by")
-    ap.add_argument("--workload", choices=("mlp", "stack", "ppcx", "decode"), default="mlp",
+    ap.add_argument("--workload", choices=("mlp", "stack", "ppcx", "decode", "attention"), default="mlp",
                     help="mlp: the three MLP matrices of one layer (the headline); stack: every coded linear of "
                          "--layers layers resident at once, one pass at batch 64 (or --batch); ppcx: a predictive "
-                         "frame against its dense reference, product with 96 rows (or --batch); decode: the "
-                         "three MLP matrices decoded to dense BF16 (decode(), the fused store sink)")
+                         "frame as served, products with 1 and 96 rows (or --batch); attention: q/k/v/o at batch "
+                         "1..128 through the batch-invariant GEMM; decode: the three MLP matrices decoded to dense "
+                         "BF16 (decode(), the fused store sink)")
+    ap.add_argument("--stack-shapes", choices=tuple(STACKS), default="qwen",
+                    help="stack: qwen = the linear shapes of the 27B model (16 attention and 48 linear-attention "
+                         "layers, embedding and head); baseline = 64 layers of q/k/v/o/gate/up/down")
     ap.add_argument("--layers", type=int, default=64)
     ap.add_argument("--no-groups", action="store_true",
                     help="one launch per linear instead of one for the matrices that take the same activations "
                          "(gate/up; in the stack also q/k/v)")
     ap.add_argument("--no-extras", action="store_true",
-                    help="mlp at batch 1: leave out the batch-64 step and the whole-stack pass that the default run "
-                         "adds to the line as `batch64` and `stack`")
+                    help="mlp at batch 1: leave out what the default run adds to the line: `batch64`, `attention`, "
+                         "`ppcx` and `stack`")
     ap.add_argument("--no-stack", action="store_true", help="mlp at batch 1: leave out the whole-stack pass only")
-    ap.add_argument("--distinct-layers", type=int, default=1,
-                    help="stack: layers encoded from their own seeds; the rest are device copies of these")
+    ap.add_argument("--distinct-layers", type=int, default=4,
+                    help="stack: layers of each kind encoded from their own seeds; the rest are device copies of these")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this decode path runs on one GPU; --gpus must be 1 (no multi-GPU figure exists)")
@@ -526,11 +714,21 @@ def main():
         args.batch, args.no_groups = 0, True  # no activations: rows = 0 selects the store sink's tiling
     if args.workload == "ppcx":
         return run_predictive(args)
+    if args.workload == "attention":
+        return run_attention(args)
     if args.workload == "stack":
         if not 1 <= args.distinct_layers <= args.layers:
             sys.exit("bench.py: --distinct-layers must be between 1 and --layers")
         return run_stack(args)
 
+    headline = args.workload == "mlp" and args.batch == 1 and not args.only and not args.no_extras
+    stack_args = prep = None
+    if headline and not args.no_stack:
+        # the stack's matrices are drawn, encoded and indexed in worker processes from now on (forked
+        # before this process touches the GPU), beside the GPU phases of the other workloads
+        stack_args = argparse.Namespace(**vars(args))
+        stack_args.batch, stack_args.steps, stack_args.warmup = 64, max(3, args.steps // 10), max(2, args.warmup // 10)
+        prep = StackPrep(stack_args)
     import torch
     from georefine_amd import bitexact_context_codec as codec
     from georefine_amd.bitexact_context_gpu import HipContextTensor
@@ -600,7 +798,7 @@ def main():
         units = per_layer[0]
         if pair is not None and not decode_only:
             log(f"batch {m} gate+up: one launch, tiling {pair._tiling('waves' if m <= GEMV_UP_TO else 'gemm')[0][3]}")
-        ms_per_step, per_kernel_ms, launch, timing = time_launches(
+        ms_per_step, per_kernel_ms, launch, timing, clocks = time_launches(
             torch, per_layer, args.steps, args.warmup, args.graph,
             lambda: sorted({n_ for ts, pr in layers for n_ in names if ts[n_].error.item()}
                            | {"gate+up" for ts, pr in layers if pr is not None and pr.error.item()}))
@@ -623,7 +821,8 @@ def main():
         value = step_bytes / (ms_per_step * 1e-3) / 1e9
         eff_bf16 = dense_bytes / (ms_per_step * 1e-3) / 1e9
         dom = max(per_kernel_ms, key=lambda n_: per_kernel_ms[n_])
-        kernel = kernel_name(decode_only, m, "+" in dom, tensors[names[0]].fused_plan["seg_len"])
+        kernel = kernel_name(decode_only, m, "+" in dom, tensors[names[0]].fused_plan["seg_len"],
+                             bool(tensors[names[0]].fused.raw_interleaved))
         traffic, traffic_source = recorded_traffic(decode_only, m, kernel)
         achieved = alg[dom]["total"] / (per_kernel_ms[dom] * 1e-3) / 1e9
         fields = {
@@ -638,6 +837,7 @@ def main():
                        "layer_copies": n_layers},
             "effective_bf16_GBps": round(eff_bf16, 2),
             "tok_s_equiv": round(eff_bf16 * 1e9 / MODEL_BF16_BYTES * m, 3) if m else None,
+            **clocks,
             "pct_hbm_roofline": round(100 * value / HBM_PEAK_GBPS, 2),
             "per_kernel": {n_: {"ms": round(per_kernel_ms[n_], 4), "alg_bytes": alg[n_]["total"],
                                 "payload_bytes": alg[n_]["payload"], "index_bytes": alg[n_]["index"],
@@ -668,31 +868,37 @@ def main():
     copy_rate = measured_copy_gbps(torch)
     result["hbm_copy_measured_GBps"] = round(copy_rate, 1)
     result["pct_of_measured_copy"] = round(100 * result["value"] / copy_rate, 2)
-    headline = args.workload == "mlp" and args.batch == 1 and not args.only and not args.no_extras
     if headline:
-        # the other two figures of the metric, timed in the same run: the MLP step at batch 64
-        # (fused GEMM on the matrix cores) and one pass through a whole resident stack
+        # the other figures of the metric, timed in the same run: the MLP step at batch 64 (fused
+        # GEMM on the matrix cores), the attention projections through the batch-invariant GEMM,
+        # a predictive frame, and one pass through a whole resident stack
         log("batch 64 ...")
         b64, _ = measure(64)
         b64.pop("config")
         result["batch64"] = b64
+        del tensors, pair, layers
+        torch.cuda.empty_cache()
+        log("attention ...")
+        result["attention"] = run_attention(args, as_dict=True)
+        log("ppcx ...")
+        result["ppcx"] = run_predictive(args, as_dict=True)
+    if prep is not None:
+        prep.wait()  # (before the CPU baseline takes the host's cores)
     if not args.no_cpu_baseline:
         log("timing the CPU oracle on whole frames ...")
         result["cpu_baseline"] = cpu_baseline(frames, words_of, x_words)
         result["cpu_baseline"]["host"] = host_description()
-    if headline and not args.no_stack:
-        del tensors, pair, layers
-        torch.cuda.empty_cache()
+    if prep is not None:
         log("whole stack ...")
-        stack_args = argparse.Namespace(**vars(args))
-        stack_args.batch, stack_args.steps, stack_args.warmup = 64, max(3, args.steps // 10), max(2, args.warmup // 10)
-        result["stack"] = run_stack(stack_args, as_dict=True)
+        result["stack"] = run_stack(stack_args, as_dict=True, prep=prep)
     print(json.dumps(result), flush=True)
 
 
-def kernel_name(decode_only, m, grouped, seg_len):
+def kernel_name(decode_only, m, grouped, seg_len, interleaved=True):
     """The kernel a launch of the workload runs (as rocprofv3 names it)."""
-    ahead = "true" if seg_len == 64 else "false"  # 64-symbol segments: the walker that reads a segment's residuals once
+    # the store sink reads a 64-symbol segment's residuals at once only from an array in the frame's
+    # own order; the resident array of a fused frame is in blocked order (raw_interleaved)
+    ahead = "true" if seg_len == 64 and not interleaved else "false"
     if decode_only:
         return f"grf::fused_walk_kernel<grf::SegmentWalkT<{ahead}>, 1, 1>"
     # (last template argument 1: the scan for frames without whole-range contexts, which these are)
@@ -714,19 +920,21 @@ def kernel_sources_sha256():
     return h.hexdigest()
 
 
-def recorded_traffic(decode_only, m, kernel):
+def recorded_traffic(decode_only, m, kernel, prefix=None):
     """HBM bytes per launch of `kernel` from the committed rocprofv3 FETCH_SIZE / WRITE_SIZE
     record (bench.py cannot read hardware counters itself), and where the figure comes from.
     The record names the kernels it measured and the digest of the device sources it was taken
     with; for another kernel or other sources the figure is withheld (None) and the reason given."""
-    name = ("fused_store_decode_qwen27b_mlp_traffic.json" if decode_only else
+    name = ((f"ppcx_gemv_m1_5120x17408_traffic.json" if m == 1 else f"ppcx_gemm_m{m}_5120x17408_traffic.json")
+            if prefix == "ppcx" else
+            "fused_store_decode_qwen27b_mlp_traffic.json" if decode_only else
             "fused_gemv_m1_qwen27b_mlp_traffic.json" if m == 1 else
             "fused_gemm_m64_qwen27b_mlp_traffic.json" if m == 64 else None)
     if name is None or not (ROOT / "profiles" / name).exists():
         return None, "no counter record for this workload"
     record = json.loads((ROOT / "profiles" / name).read_text())
     per_kernel = record.get("traffic_bytes_per_launch")
-    short = kernel.split("<")[0].split("::")[-1]
+    short = "product" if prefix == "ppcx" else kernel.split("<")[0].split("::")[-1]
     if not isinstance(per_kernel, dict) or short not in per_kernel:
         return None, f"profiles/{name} holds no figure for {short}"
     if record.get("kernel_sources_sha256") != kernel_sources_sha256():
@@ -734,18 +942,93 @@ def recorded_traffic(decode_only, m, kernel):
     return per_kernel[short], f"recorded: profiles/{name} (rocprofv3 --pmc, same kernel sources)"
 
 
-def time_launches(torch, per_layer, steps, warmup, graph, errors):
-    """(ms per step, {label: ms per launch}, how the step was launched, how launches were timed).
+class Stamps:
+    """Device timestamps between launches (grf_timestamp: a one-lane kernel that reads the device's
+    constant-rate counter and its shader-clock counter in stream order).  Events cannot be recorded
+    inside a captured HIP graph on this platform; these launches can, so a graph of steps with a
+    stamp after every launch gives each launch's duration in the very sequence that is timed."""
 
-    `per_layer[c]` holds the launches of a step on copy c of the layer's matrices; step i runs
-    on copy i mod len(per_layer), so no step finds its matrices in the caches.  After `warmup`
-    eager steps: each launch is captured twelve times into a HIP graph of its own, over the
-    copies in turn, and the replays are bracketed by events on the launch stream, which gives
-    the kernel's duration without the host's per-launch latency (eager events around single
-    launches where capture is not possible or --no-graph is given); then exactly `steps` steps,
-    replayed from graphs of up to 96 consecutive steps, are timed on the host clock between
-    synchronisations."""
+    def __init__(self, torch, count):
+        from georefine_amd import _native
+        self.torch, self.lib = torch, _native.hip()
+        self.khz = self.lib.grf_wall_clock_khz() or 100000
+        self.buf = torch.zeros((count, 3), dtype=torch.int64, device="cuda")
+        self.used = 0
+
+    def mark(self):
+        torch = self.torch
+        if self.lib.grf_timestamp(self.buf[self.used].data_ptr(), torch.cuda.current_stream().cuda_stream):
+            raise RuntimeError(self.lib.grf_last_error().decode(errors="replace"))
+        self.used += 1
+
+    def read(self):
+        """(milliseconds at every mark, shader clock in MHz between the two marks farthest apart
+        that ran on one compute unit -- the counters of different units do not share a zero)"""
+        host = self.buf[:self.used].cpu().numpy()
+        ms = host[:, 0].astype(np.float64) / self.khz
+        mhz, span = 0.0, 0.0
+        for unit in np.unique(host[:, 2]):
+            at = np.flatnonzero(host[:, 2] == unit)
+            if at.size > 1 and ms[at[-1]] - ms[at[0]] > span:
+                span = ms[at[-1]] - ms[at[0]]
+                mhz = float(host[at[-1], 1] - host[at[0], 1]) / (span * 1e3)
+        return ms, mhz
+
+
+class StampedGraph:
+    """`launches` (callables, in order) captured with a stamp after each, and two stamps back to
+    back first, whose distance is what a stamp itself adds to the sequence."""
+
+    def __init__(self, torch, launches):
+        self.torch = torch
+        self.stamps = Stamps(torch, len(launches) + 2)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.stamps.mark()
+            self.stamps.mark()
+            for run in launches:
+                run()
+                self.stamps.mark()
+
+    def durations(self, replays=2):
+        """(ms of every launch with the stamp's share taken off, the stamp's share in ms, shader
+        clock in MHz over the whole sequence, ms of the whole sequence), from the last replay."""
+        for _ in range(replays):
+            self.graph.replay()
+        self.torch.cuda.synchronize()
+        ms, mhz = self.stamps.read()
+        own = ms[1] - ms[0]
+        spans = np.diff(ms[1:]) - own
+        whole = ms[-1] - ms[1]
+        return spans, own, mhz, whole
+
+
+MAX_GRAPH_LAUNCHES = 4096  # kernel nodes per captured graph
+
+
+def time_launches(torch, per_layer, steps, warmup, graph, errors):
+    """(ms per step, {label: ms per launch}, how the step was launched, how launches were timed,
+    {shader clock, the step as the stamps see it, ...}).
+
+    `per_layer[c]` holds the launches of a step, (label, members, callable) each, on copy c of
+    the workload's matrices; step i runs on copy i mod len(per_layer), so no step finds its
+    matrices in the caches.  A label may occur several times in a step (the layers of a stack):
+    its figure is the mean over its launches.
+
+    Order of events: `warmup` eager steps (they also upload tilings and let the allocator
+    settle); every graph is captured -- the graphs of up to 96 consecutive steps that are timed,
+    and a graph of the same steps with a device timestamp after every launch (Stamps); the timed
+    graphs are replayed once more as they will be timed, untimed, so that the clocks are where
+    sustained work holds them (captures leave the GPU idle for tens of milliseconds, and the first
+    launches after such a gap run at a lower clock); synchronise; exactly `steps` steps are
+    replayed and timed on the host clock; synchronise.  Then the stamped graph gives the
+    per-launch durations: the same kernels in the same order on the same copies, so the
+    launches' sum and the step agree up to what the stamps add, which is measured and taken
+    off.  Without graphs (--no-graph, or a capture that fails): eager steps, and HIP events
+    around single launches."""
     copies = len(per_layer)
+    labels = [label for label, _, _ in per_layer[0]]
+    names = list(dict.fromkeys(labels))
 
     def step(i):
         return [run() for _, _, run in per_layer[i % copies]]
@@ -756,31 +1039,67 @@ def time_launches(torch, per_layer, steps, warmup, graph, errors):
     bad = errors()
     if bad:
         sys.exit(f"bench.py: decoder error word set for {bad}")
+    launch, wall, extra = "eager", None, {}
     per_kernel_ms = {}
-    timing = f"HIP events around 12 launches per graph replay, over {copies} device copies of the matrices in turn"
+    chunk = min(steps, 96, max(1, MAX_GRAPH_LAUNCHES // len(labels)))
+    chunk = chunk // copies * copies or chunk  # whole turns through the copies where a step is small
+    graphs, stamped = [], None
     if graph:
+        # consecutive steps captured once and replayed: the launches are submitted together, which
+        # takes the host's per-launch latency out of the gaps between kernels
         try:
-            for j, (label, _, _) in enumerate(per_layer[0]):
+            plan = [(chunk, steps // chunk)] + ([(steps % chunk, 1)] if steps % chunk else [])
+            for length, times in plan:
                 g = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(g):
-                    for i in range(12):
-                        per_layer[i % copies][j][2]()
+                    for i in range(length):
+                        step(i)
+                graphs.append((g, times))
+            torch.cuda.synchronize()
+        except Exception as exc:  # keep the eager figure
+            log(f"graph capture failed ({exc}); reporting the eager steps")
+            graphs = []
+        if graphs:
+            try:
+                stamped = StampedGraph(torch, [per_layer[i % copies][j][2] for i in range(chunk)
+                                               for j in range(len(labels))])
+            except Exception as exc:
+                log(f"stamped graph failed ({exc}); timing eager launches")
+    if graphs:
+        for g, times in graphs:  # untimed, as they will be timed
+            for _ in range(times):
                 g.replay()
-                torch.cuda.synchronize()
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                replays = max(2, steps // 10)
-                a.record()
-                for _ in range(replays):
-                    g.replay()
-                b.record()
-                torch.cuda.synchronize()
-                per_kernel_ms[label] = a.elapsed_time(b) / (12 * replays)
-        except Exception as exc:
-            log(f"graph capture failed ({exc}); timing eager launches")
-            per_kernel_ms = {}
+        torch.cuda.synchronize()
+        wall0 = time.perf_counter()
+        for g, times in graphs:
+            for _ in range(times):
+                g.replay()
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - wall0
+        launch = "hip graph replay"
+    else:
+        for i in range(max(warmup, 1)):
+            step(i)
+        torch.cuda.synchronize()
+        wall0 = time.perf_counter()
+        for i in range(steps):
+            step(i)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - wall0
+    if stamped is not None:
+        spans, own, mhz, whole = stamped.durations()
+        spans = spans.reshape(chunk, len(labels))
+        per_kernel_ms = {n_: float(np.mean([spans[:, j].mean() for j, l_ in enumerate(labels) if l_ == n_]))
+                         for n_ in names}
+        timing = (f"device timestamps after every launch inside a HIP graph of {chunk} consecutive steps (the "
+                  f"steps that are timed, plus the stamps), over {copies} device copies of the matrices in turn; a "
+                  f"stamp's own share ({own * 1e3:.1f} us) is taken off every launch")
+        extra = {"sclk_mhz": round(mhz, 1), "stamp_us": round(own * 1e3, 2),
+                 "step_ms_stamped_graph": round(whole / chunk, 4),
+                 "launches_sum_ms": round(float(spans.sum(axis=1).mean()), 4)}
     if not per_kernel_ms:
         timing = "HIP events around single eager launches"
-        n_units = len(per_layer[0])
+        n_units = len(labels)
         starts = [[torch.cuda.Event(enable_timing=True) for _ in range(n_units)] for _ in range(steps)]
         ends = [[torch.cuda.Event(enable_timing=True) for _ in range(n_units)] for _ in range(steps)]
         torch.cuda.synchronize()
@@ -790,46 +1109,12 @@ def time_launches(torch, per_layer, steps, warmup, graph, errors):
                 run()
                 ends[s_][j].record()
         torch.cuda.synchronize()
-        per_kernel_ms = {label: float(np.mean([starts[s_][j].elapsed_time(ends[s_][j]) for s_ in range(steps)]))
-                         for j, (label, _, _) in enumerate(per_layer[0])}
-    launch = "eager"
-    wall = None
-    if graph:
-        # consecutive steps captured once and replayed: the launches are submitted together, which
-        # takes the host's per-launch latency out of the gaps between kernels
-        try:
-            chunk = min(steps, 96) // copies * copies or steps  # whole turns through the copies
-            plan = [(chunk, steps // chunk)] + ([(steps % chunk, 1)] if steps % chunk else [])
-            graphs = []
-            for length, times in plan:
-                g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    for i in range(length):
-                        step(i)
-                g.replay()
-                graphs.append((g, times))
-            torch.cuda.synchronize()
-        except Exception as exc:  # keep the eager figure
-            log(f"graph capture failed ({exc}); reporting the eager steps")
-        else:
-            wall0 = time.perf_counter()
-            for g, times in graphs:
-                for _ in range(times):
-                    g.replay()
-            torch.cuda.synchronize()
-            wall = time.perf_counter() - wall0
-            launch = "hip graph replay"
-    if wall is None:
-        torch.cuda.synchronize()
-        wall0 = time.perf_counter()
-        for i in range(steps):
-            step(i)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - wall0
+        per_kernel_ms = {n_: float(np.mean([starts[s_][j].elapsed_time(ends[s_][j]) for s_ in range(steps)
+                                            for j, l_ in enumerate(labels) if l_ == n_])) for n_ in names}
     bad = errors()
     if bad:
         sys.exit(f"bench.py: decoder error word set for {bad}")
-    return wall / steps * 1e3, per_kernel_ms, launch, timing
+    return wall / steps * 1e3, per_kernel_ms, launch, timing, extra
 
 
 if __name__ == "__main__":

@@ -192,15 +192,12 @@ class HipContextTensor:
 
     GEMV_UP_TO, GEMM_TWO_ROWS_FROM, DENSE_ABOVE = GEMV_UP_TO, GEMM_TWO_ROWS_FROM, DENSE_ABOVE
 
-    def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None,
-                 m_invariant=False):
-        import torch
-        if not torch.cuda.is_available():
-            raise RuntimeError("a ROCm GPU is required")
-        self._lib = _native.hip()  # fails loudly when the device library is absent
-        # linear()'s default routing: True sends every row count to the matrix-core kernel, so
-        # that a row's output bits never depend on the rows it arrives with (route_rows)
-        self.m_invariant = bool(m_invariant)
+    @staticmethod
+    def host_prepare(frame: bytes, *, stride: int = 1024, fused=True, fused_segment=None):
+        """The host half of the constructor -- parse, validate and index the frame, lay out the
+        fused kernels' tables -- for callers that prepare frames on worker threads and construct
+        the device objects later (``HipContextTensor(frame, prepared=...)`` then only uploads).
+        Needs no GPU."""
         segment = None
         if fused:
             try:
@@ -209,6 +206,54 @@ class HipContextTensor:
             except _fused.FusedUnsupported:
                 segment = None
         indexed = index_frame(frame, stride, fused_segment=segment, raw6_residual=segment is not None)
+        plan, reason = None, "disabled" if not fused else "frame mode or geometry"
+        if "fused_states" in indexed:
+            try:
+                plan = _fused.FramePlan(indexed["shape"], indexed["nr"], indexed["nc"], indexed["rows"],
+                                        indexed["main_freq"], indexed.pop("fused_states"), indexed.pop("fused_offsets"),
+                                        len(indexed["main_stream"]), indexed["fused_segment"])
+            except _fused.FusedUnsupported as exc:
+                reason = str(exc)
+                indexed.pop("fused_states", None)
+                indexed.pop("fused_offsets", None)
+        main_bytes = len(indexed["main_stream"]) if "main_stream" in indexed else 0
+        raw6_segment = raw6_block = 0
+        if plan is not None:  # the fused kernels read 16-byte vectors: pad the stream's allocation
+            indexed["main_stream"] = np.concatenate((indexed["main_stream"], np.zeros(16, dtype=np.uint8)))
+            # The packed residuals in the order the tile walker reads them (a permutation of the
+            # 12-byte groups of 16 fields, no field is touched): rows by class as the tilings take
+            # them, in blocks of as many rows as a wave unit of the GEMV has; inside a block by
+            # position in the segment, then by segment, then by row.  The lanes of a unit walk
+            # neighbouring segments of the block's rows in step, so they read one run of bytes per
+            # visit and a 128-byte line is used in a single visit; in the frame's order a line came
+            # back from memory about twice per launch.
+            rows_, cols_ = indexed["shape"]
+            seg = indexed["fused_segment"]
+            raw = indexed["residual_stream"]
+            if raw.size == rows_ * cols_ * 3 // 4:
+                block, position, held = plan.residual_order()
+                indexed["residual_stream"] = _fused.order_residuals(raw, rows_, cols_, seg, block, position, held)
+                indexed["row_pos"] = position
+                raw6_segment, raw6_block = seg, block
+            indexed.update(fused_seg_state=plan.seg_state, fused_seg_offset=plan.seg_offset, fused_lut=plan.lut,
+                           fused_tab=plan.tab)
+        return {"indexed": indexed, "plan": plan, "reason": reason, "stride": stride, "fused": fused,
+                "main_bytes": main_bytes, "raw6_segment": raw6_segment, "raw6_block": raw6_block}
+
+    def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None,
+                 m_invariant=False, prepared=None):
+        import torch
+        if not torch.cuda.is_available():
+            raise RuntimeError("a ROCm GPU is required")
+        self._lib = _native.hip()  # fails loudly when the device library is absent
+        # linear()'s default routing: True sends every row count to the matrix-core kernel, so
+        # that a row's output bits never depend on the rows it arrives with (route_rows)
+        self.m_invariant = bool(m_invariant)
+        if prepared is None:
+            prepared = self.host_prepare(frame, stride=stride, fused=fused, fused_segment=fused_segment)
+        elif prepared["stride"] != stride or prepared["fused"] != fused:
+            raise ValueError("the frame was prepared with another stride or fused setting")
+        indexed, plan = prepared["indexed"], prepared["plan"]
         self.shape = indexed["shape"]
         self.n = math.prod(self.shape)
         self.stride = stride
@@ -221,38 +266,9 @@ class HipContextTensor:
         self.device = torch.device(device)
         self.buffers = {}
         self.fused = None
-        self.fused_reason = "disabled" if not fused else "frame mode or geometry"
-        plan = None
-        if "fused_states" in indexed:
-            try:
-                plan = _fused.FramePlan(self.shape, self.nr, self.nc, indexed["rows"], indexed["main_freq"],
-                                        indexed.pop("fused_states"), indexed.pop("fused_offsets"),
-                                        len(indexed["main_stream"]), indexed["fused_segment"])
-            except _fused.FusedUnsupported as exc:
-                self.fused_reason = str(exc)
-                indexed.pop("fused_states", None)
-                indexed.pop("fused_offsets", None)
-        self._main_bytes = len(indexed["main_stream"]) if "main_stream" in indexed else 0
-        self._raw6_segment, self._raw6_block = 0, 0
-        if plan is not None:  # the fused kernels read 16-byte vectors: pad the stream's allocation
-            indexed["main_stream"] = np.concatenate((indexed["main_stream"], np.zeros(16, dtype=np.uint8)))
-            # The packed residuals in the order the tile walker reads them (a permutation of the
-            # 12-byte groups of 16 fields, no field is touched): rows by class as the tilings take
-            # them, in blocks of as many rows as a wave unit of the GEMV has; inside a block by
-            # position in the segment, then by segment, then by row.  The lanes of a unit walk
-            # neighbouring segments of the block's rows in step, so they read one run of bytes per
-            # visit and a 128-byte line is used in a single visit; in the frame's order a line came
-            # back from memory about twice per launch.
-            rows_, cols_ = self.shape
-            seg = indexed["fused_segment"]
-            raw = indexed["residual_stream"]
-            if raw.size == rows_ * cols_ * 3 // 4:
-                block, position, held = plan.residual_order()
-                indexed["residual_stream"] = _fused.order_residuals(raw, rows_, cols_, seg, block, position, held)
-                indexed["row_pos"] = position
-                self._raw6_segment, self._raw6_block = seg, block
-            indexed.update(fused_seg_state=plan.seg_state, fused_seg_offset=plan.seg_offset, fused_lut=plan.lut,
-                           fused_tab=plan.tab)
+        self.fused_reason = prepared["reason"]
+        self._main_bytes = prepared["main_bytes"]
+        self._raw6_segment, self._raw6_block = prepared["raw6_segment"], prepared["raw6_block"]
         for name, array in indexed.items():
             if isinstance(array, np.ndarray):
                 self.buffers[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
@@ -513,17 +529,23 @@ class HipContextTensor:
             return self.gemm(x, bias, check=check)
         return self.gemv(x, bias, check=check)
 
-    def gather_rows(self, ids, *, check=True):
+    def gather_rows(self, ids, *, check=True, validate=True):
         """Rows ``ids`` (any shape) as BF16 [*ids.shape, cols]; IndexError for a row the matrix
         does not have (GCR/bitexact_context_gpu.py:159-168).  Frames the tile walker takes give
         every requested row a workgroup that walks all of its segments at once; others decode
-        the checkpoint blocks of the rows, one lane each."""
+        the checkpoint blocks of the rows, one lane each.  ``validate=False`` (with
+        ``check=False``) leaves out the range test, which reads a flag back from the device, for
+        callers that vouch for their ids and must not synchronise (a HIP graph capture); ids
+        outside the matrix are then clamped into it."""
         import torch
         ids = ids.to(device=self.device, dtype=torch.int64)
         if ids.numel() == 0:
             return torch.empty((*ids.shape, self.shape[1]), device=self.device, dtype=torch.bfloat16)
-        if torch.any((ids < 0) | (ids >= self.shape[0])).item():
-            raise IndexError("embedding row outside tensor")
+        if validate:
+            if torch.any((ids < 0) | (ids >= self.shape[0])).item():
+                raise IndexError("embedding row outside tensor")
+        else:
+            ids = ids.clamp(0, self.shape[0] - 1)
         if self.fused is not None and self._gather is not False:
             if self._gather is None:
                 try:

@@ -172,32 +172,7 @@ class HipPredictiveTensor:
                 self.buffers[name + "_bucket"] = torch.from_numpy(_tables.coarse_buckets(cum)).to(self.device)
         self.error = torch.zeros((), device=self.device, dtype=torch.int32)
         self._tilings = {}
-        self._frame = None
-        if self.mode != 2:
-            b = self.buffers
-            f = _hip_abi.GrfPpcxFrame()
-            f.main.bytes, f.main.n_bytes = b["main_stream"].data_ptr(), b["main_stream"].numel() - 16
-            f.main.vocab, f.main.nctx = codec.MAIN_VOCAB, codec.MAIN_CONTEXTS
-            f.main.cum, f.main.bucket = b["main_cum"].data_ptr(), b["main_bucket"].data_ptr()
-            f.main.states, f.main.offsets = b["main_states"].data_ptr(), b["main_offsets"].data_ptr()
-            if self.resident_mode == 0:
-                f.residual.bytes, f.residual.n_bytes = b["raw5"].data_ptr(), b["raw5"].numel() - 16
-            else:
-                f.residual.bytes, f.residual.n_bytes = b["residual_stream"].data_ptr(), b["residual_stream"].numel()
-                f.residual.vocab, f.residual.nctx = codec.RES_VOCAB, codec.RES_CONTEXTS
-                f.residual.cum, f.residual.bucket = b["residual_cum"].data_ptr(), b["residual_bucket"].data_ptr()
-                f.residual.states = b["residual_states"].data_ptr()
-                f.residual.offsets = b["residual_offsets"].data_ptr()
-            f.labels, f.flips, f.thresholds = b["labels"].data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr()
-            f.rows, f.cols = self.shape
-            f.mode, f.stride = self.resident_mode, stride
-            self._frame = f
-        self.fused = None
-        if self._plan is not None:
-            try:
-                self._prepare_fused()
-            except _fused.FusedUnsupported as exc:
-                self.fused, self.fused_reason = None, str(exc)
+        self._bind()
         # What the tile walker needs of the reference is the 4-bit bin of every word (the
         # decoded word itself comes from the frame's symbols alone), and the reference is given
         # here, once.  Keeping that plane, half a byte per weight, takes the reference out of
@@ -217,6 +192,48 @@ class HipPredictiveTensor:
             self.has_contexts = True
             del ref
 
+    def _bind(self):
+        """Descriptors over this object's device buffers (their addresses go into the structures
+        the kernels take)."""
+        self._frame = None
+        if self.mode != 2:
+            b = self.buffers
+            f = _hip_abi.GrfPpcxFrame()
+            f.main.bytes, f.main.n_bytes = b["main_stream"].data_ptr(), b["main_stream"].numel() - 16
+            f.main.vocab, f.main.nctx = codec.MAIN_VOCAB, codec.MAIN_CONTEXTS
+            f.main.cum, f.main.bucket = b["main_cum"].data_ptr(), b["main_bucket"].data_ptr()
+            f.main.states, f.main.offsets = b["main_states"].data_ptr(), b["main_offsets"].data_ptr()
+            if self.resident_mode == 0:
+                f.residual.bytes, f.residual.n_bytes = b["raw5"].data_ptr(), b["raw5"].numel() - 16
+            else:
+                f.residual.bytes, f.residual.n_bytes = b["residual_stream"].data_ptr(), b["residual_stream"].numel()
+                f.residual.vocab, f.residual.nctx = codec.RES_VOCAB, codec.RES_CONTEXTS
+                f.residual.cum, f.residual.bucket = b["residual_cum"].data_ptr(), b["residual_bucket"].data_ptr()
+                f.residual.states = b["residual_states"].data_ptr()
+                f.residual.offsets = b["residual_offsets"].data_ptr()
+            f.labels, f.flips, f.thresholds = b["labels"].data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr()
+            f.rows, f.cols = self.shape
+            f.mode, f.stride = self.resident_mode, self.stride
+            self._frame = f
+        self.fused = None
+        if self._plan is not None:
+            try:
+                self._prepare_fused()
+            except _fused.FusedUnsupported as exc:
+                self.fused, self.fused_reason = None, str(exc)
+
+    def clone(self):
+        """A second resident copy of the same coded matrix: every device buffer is duplicated
+        (nothing is decoded or indexed again)."""
+        import copy
+        import torch
+        other = copy.copy(self)
+        other.buffers = {k: v.clone() for k, v in self.buffers.items()}
+        other.error = torch.zeros_like(self.error)
+        other._tilings = {}
+        other._bind()
+        return other
+
     @property
     def resident_bytes(self):
         """Every device allocation this tensor holds: buffers, tilings made so far, the error word."""
@@ -230,7 +247,8 @@ class HipPredictiveTensor:
         plan, b = self._plan, self.buffers
         for name, array in (("fused_seg_state", plan.seg_state), ("fused_seg_offset", plan.seg_offset),
                             ("fused_lut", plan.lut), ("fused_tab", plan.tab.view(np.int64))):
-            b[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
+            if name not in b:  # (a clone already holds its copies)
+                b[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
         f = _hip_abi.GrfPpcxFused()
         f.main_bytes, f.raw5 = b["main_stream"].data_ptr(), b["raw5"].data_ptr()
         f.seg_state, f.seg_offset = b["fused_seg_state"].data_ptr(), b["fused_seg_offset"].data_ptr()

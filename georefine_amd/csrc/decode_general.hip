@@ -177,10 +177,38 @@ int launch_status(const char *what) {
 
 }  // namespace
 
+namespace grf {
+// One lane writes the two device counters -- the constant-rate one and the shader clock's --
+// and where it ran: shader-clock counters of different parts of the chip do not share a zero,
+// so only two readings taken at one place may be subtracted.
+__global__ void timestamp_kernel(uint64_t *slot) {
+  if (threadIdx.x == 0) {
+    slot[0] = wall_clock64();
+    slot[1] = clock64();
+    slot[2] = __smid();
+  }
+}
+}  // namespace grf
+
 extern "C" {
 
 const char *grf_last_error(void) { return grf::g_error.c_str(); }
-int grf_abi_version(void) { return 2; }
+int grf_abi_version(void) { return 3; }
+
+int grf_wall_clock_khz(void) {
+  int dev = 0, khz = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return 0;
+  if (hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) return 0;
+  return khz;
+}
+
+int grf_timestamp(uint64_t *slot, void *hip_stream) {
+  if (!slot) return fail(GRF_BAD_ARGUMENT, "grf_timestamp: null argument");
+  hipLaunchKernelGGL(grf::timestamp_kernel, dim3(1), dim3(64), 0, (hipStream_t)hip_stream, slot);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(GRF_LAUNCH_FAILED, std::string("grf_timestamp: ") + hipGetErrorString(e));
+  return GRF_OK;
+}
 
 int grf_bctx_decode(const grf_bctx_frame *frame, const int64_t *block_ids, uint32_t count, uint16_t *out,
                     int32_t *error, void *hip_stream) {

@@ -411,6 +411,18 @@ int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, c
                   uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
                   size_t workspace_bytes, int32_t *error, void *hip_stream);
 
+/* A one-lane kernel that writes slot[0] = the device's constant-rate counter
+ * (grf_wall_clock_khz), slot[1] = its shader-clock counter and slot[2] = the identifier of the
+ * compute unit it ran on, all read when the kernel runs, i.e. in stream order after the work
+ * launched before it.  Two of them around launches give their duration on the device where
+ * events cannot be recorded (inside a captured HIP graph); two that ran on the same compute
+ * unit (shader-clock counters of different parts of the chip do not share a zero) also give
+ * the shader clock the work between them ran at.  slot: device memory, three 64-bit words.
+ * No reference counterpart; it allocates nothing and can be captured. */
+int grf_timestamp(uint64_t *slot, void *hip_stream);
+/* Rate of the constant counter of the current device in kHz (0 if the runtime does not say). */
+int grf_wall_clock_khz(void);
+
 const char *grf_last_error(void);
 int grf_abi_version(void);
 

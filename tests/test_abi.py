@@ -32,7 +32,7 @@ def test_header_functions_are_exported():
 def test_device_library_reports_its_abi_version_without_a_gpu():
     lib = ctypes.CDLL(str(_native.HIP_LIB))
     lib.grf_abi_version.restype = ctypes.c_int
-    assert lib.grf_abi_version() == 2
+    assert lib.grf_abi_version() == 3
 
 
 def test_struct_mirrors_match_the_header_field_order():
