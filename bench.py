@@ -248,6 +248,16 @@ def cpu_baseline(frames, words_of, x_words, min_seconds=8.0, max_frames=12):
     return result
 
 
+def calibration_copy(torch):
+    """A plain 128 MiB read + 128 MiB write elementwise kernel, three times: a kernel of known
+    traffic for a counter profile of this command to scale its FETCH_SIZE / WRITE_SIZE by."""
+    src = torch.ones(32 * 1024 * 1024, dtype=torch.int32, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        torch.add(src, 1, out=dst)
+    torch.cuda.synchronize()
+
+
 def launch_fields(alg_total, ms):
     gbps = alg_total / (ms * 1e-3) / 1e9
     return {"ms": round(ms, 4), "alg_bytes": int(alg_total), "GBps": round(gbps, 2),
@@ -337,6 +347,8 @@ def run_attention(args, as_dict=False):
         batches[str(m)], timing = one(m, True)
         log(f"attention batch {m}: {batches[str(m)]['ms_per_pass']} ms per pass")
     default1, _ = one(1, False)
+    if args.calibrate_copy:
+        calibration_copy(torch)
     result = {
         "config": {"workload": "attention projections q 5120->6144, k/v 5120->1024, o 6144->5120 (BCTX (16,4) frames), "
                                "q/k/v in one launch, o in another; every batch through the matrix-core GEMM "
@@ -387,7 +399,9 @@ def run_predictive(args, as_dict=False):
     t = HipPredictiveTensor(frame, ref, stride=1024, device="cuda:0")
     if t.fused is None:
         sys.exit(f"bench.py: the frame is not eligible for the fused kernels: {t.fused_reason}")
-    log(f"PPCX frame {len(frame)} B ({8 * len(frame) / target.size:.3f} bit/weight) mode {t.mode}; setup {time.perf_counter() - t0:.1f}s")
+    log(f"PPCX frame {len(frame)} B ({8 * len(frame) / target.size:.3f} bit/weight) mode {t.mode}; setup {time.perf_counter() - t0:.1f}s; "
+        f"rows per label {np.bincount(t.buffers['labels'].cpu().numpy(), minlength=16).tolist()}; GEMV tiling "
+        f"{t._tiling_for('waves')[3]}; GEMM tiling {t._tiling_for('gemm')[3]}")
     copies = [t, t.clone(), t.clone()]  # three targets in rotation: more bytes than the caches hold
     steps, warmup = (args.steps, args.warmup) if not as_dict else (max(10, args.steps // 2), max(4, args.warmup // 4))
     x_all = torch.from_numpy(bf16_words(np.random.default_rng(7).normal(0, 1, size=(max(batches), cols)))).view(torch.bfloat16).cuda()
@@ -417,6 +431,8 @@ def run_predictive(args, as_dict=False):
                        "algorithmic_bytes_per_product": alg,
                        "roofline": roofline_fields(alg, per_ms["product"], kernel + " (all launches of a product)", traffic, source)}
         log(f"ppcx batch {m}: {ms_step:.4f} ms per product")
+    if args.calibrate_copy:
+        calibration_copy(torch)
     n = target.size
     result = {
         "config": {"workload": "PPCX target 5120x17408 coded against a reference (target + N(0, 0.002)), products as "
@@ -803,11 +819,7 @@ def main():
             lambda: sorted({n_ for ts, pr in layers for n_ in names if ts[n_].error.item()}
                            | {"gate+up" for ts, pr in layers if pr is not None and pr.error.item()}))
         if args.calibrate_copy:
-            src = torch.ones(32 * 1024 * 1024, dtype=torch.int32, device="cuda")
-            dst = torch.empty_like(src)
-            for _ in range(3):
-                torch.add(src, 1, out=dst)
-            torch.cuda.synchronize()
+            calibration_copy(torch)
         alg = {}
         for label, members, _ in units:
             parts = [algorithmic_bytes(tensors[n_], m) for n_ in members]

@@ -400,6 +400,49 @@ def build_tiles(row_class, nr, r):
     return np.concatenate(tiles), np.asarray(classes, dtype=np.uint8)
 
 
+def build_balanced_tiles(row_class, nr, unit_rows, slots, max_rows):
+    """Rows grouped by class (index order inside a class) into at most ``slots`` tiles whose
+    heights are as equal as the classes allow: every class gets tiles in proportion to its
+    rows -- one at least -- and cuts its rows into them evenly, in whole units of ``unit_rows``
+    rows.  A launch is as long as its tallest tile; cut at one height for all classes, a frame
+    whose classes differ widely in size (the row labels of a predictive frame) leaves workgroup
+    slots empty or pays a second round for a few tiles.  Returns (tile_rows with stride R,
+    tile_class, R) or None when no cut within ``slots`` tiles and ``max_rows`` rows exists."""
+    order = np.argsort(row_class, kind="stable").astype(np.uint32)
+    counts = np.bincount(row_class, minlength=nr)
+    live = [rho for rho in range(nr) if counts[rho]]
+    if not live or len(live) > slots:
+        return None
+    units = {rho: -(-int(counts[rho]) // unit_rows) for rho in live}
+    tiles = {rho: 1 for rho in live}
+    height = lambda rho: -(-units[rho] // tiles[rho])
+    for _ in range(slots - len(live)):  # the next tile to the class whose tiles are tallest
+        rho = max(live, key=lambda c: (height(c), units[c]))
+        if height(rho) <= 1:
+            break
+        tiles[rho] += 1
+    tallest = max(height(rho) for rho in live) * unit_rows
+    if tallest > max_rows:
+        return None
+    out_rows, out_class = [], []
+    first = np.concatenate(([0], np.cumsum(counts)[:-1]))
+    for rho in live:
+        rows_of_class = order[first[rho]:first[rho] + counts[rho]]
+        n, u = tiles[rho], units[rho]
+        at = 0
+        for k in range(n):  # units per tile differ by at most one
+            take = (u // n + (1 if k < u % n else 0)) * unit_rows
+            chunk = rows_of_class[at:at + take]
+            at += take
+            if chunk.size == 0:
+                continue
+            slot = np.full(tallest, 0xFFFFFFFF, dtype=np.uint32)
+            slot[:chunk.size] = chunk
+            out_rows.append(slot)
+            out_class.append(rho)
+    return np.concatenate(out_rows), np.asarray(out_class, dtype=np.uint8), tallest
+
+
 class FramePlan:
     """Frame-level derived arrays (shared by every tiling) and a tiling factory."""
 
@@ -479,6 +522,17 @@ class FramePlan:
                 seg_len=self.seg_len, table_bytes=self.table_bytes())
         tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)
         assert len(tile_class) == n_tiles
+        if waves and m and not os.environ.get("GEOREFINE_FUSED_WAVE_TILING"):
+            # classes of very different sizes: the same workgroup slots, cut so that no tile is
+            # taller than it has to be (the kernel walks a tile's real height)
+            nwaves, rpw = threads // 64, 64 // p
+            per_cu = max(1, min(24 // nwaves, (MAX_LDS - 1024) // lds))
+            slots = -(-n_tiles // (256 * per_cu)) * 256 * per_cu
+            even = build_balanced_tiles(self.row_class, self.nr, rpw, slots, r)
+            if even is not None and (even[2] < r or (even[2] == r and len(even[1]) > n_tiles)):
+                tile_rows, tile_class, r = even
+                n_tiles = len(tile_class)
+                lds = lds_bytes_waves(self.nc, self.lognb, self.tabn, WAVE_ROWS_PER_PASS, threads, p, r, n_slabs, cap)
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
                                  n_tiles=n_tiles, piece_cap=cap,

@@ -338,9 +338,18 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
   float *sub = reinterpret_cast<float *>(lds + L.sub);
   uint32_t *rows = reinterpret_cast<uint32_t *>(lds + L.rows);
   const uint32_t piece_off = L.stream + (wave * rpw + rl) * g.piece_cap;
-  const uint32_t groups = (R + rpw - 1) / rpw, units = groups * g.n_slabs;
+  // The tile's real height: the slots up to its last row.  A tile with fewer rows than R --
+  // the tail of a row class, or a tiling that gives the tiles of a small class fewer rows --
+  // has that many row groups fewer to walk (its empty slots, kNoRow, are at the end).
+  uint32_t r_real = 0;
+  for (uint32_t i0 = 0; i0 < R; i0 += 64) {  // uniform
+    const uint32_t i = i0 + lane;
+    const uint64_t has = __ballot(i < R && g.tile_rows[tile * R + min(i, R - 1)] < f.rows);
+    if (has) r_real = i0 + 64 - (uint32_t)__builtin_clzll(has);
+  }
+  const uint32_t groups = (r_real + rpw - 1) / rpw, units = groups * g.n_slabs;
   const bool by_slab = K * 2u * M > kUnitsBySlabBytes;
-  const uint32_t n_minor = by_slab ? groups : g.n_slabs;
+  const uint32_t n_minor = max(1u, by_slab ? groups : g.n_slabs);
   const uint32_t step_major = nwaves / n_minor, step_minor = nwaves % n_minor;
   uint32_t bad = 0;
 
@@ -928,8 +937,10 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     __syncthreads();  // tables and stream bytes (or the previous chunk's sums) are done with
 #pragma unroll
     for (int jj = 0; jj < CT; ++jj)
+      if (c0 + jj < MT) {  // (six tiles: the second round holds two)
 #pragma unroll
-      for (int v = 0; v < 4; ++v) sums[((wave * CT + jj) * 4 + v) * 64 + lane2] = acc[c0 + jj][v];
+        for (int v = 0; v < 4; ++v) sums[((wave * CT + jj) * 4 + v) * 64 + lane2] = acc[c0 + jj][v];
+      }
     __syncthreads();
     const uint32_t per_block = CT * 256;  // values of one row block: [tile jj][v][lane]
     for (uint32_t i = tid2; i < shape.row_blocks * per_block; i += nthreads) {
@@ -937,7 +948,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
       const uint32_t jj = within / 256, v = (within / 64) % 4, ln = within % 64;
       const uint32_t n_local = blk * 16 + ln % 16, m = (c0 + jj) * 16 + (ln / 16) * 4 + v;
       const uint32_t orow = n_local < R ? g.tile_rows[tile * R + n_local] : grf::kNoRow;
-      if (orow >= f.rows || m >= m_rows) continue;  // empty slot, no such row, or a padding row
+      if (orow >= f.rows || m >= m_rows || c0 + jj >= (uint32_t)MT) continue;  // empty slot, no such row, a padding row
       // wave index of (quad, block) is quad * row_blocks + block
       float sum = sums[(blk * CT) * 256 + within];
       for (uint32_t qd = 1; qd < shape.quads; ++qd) sum += sums[((qd * shape.row_blocks + blk) * CT) * 256 + within];
