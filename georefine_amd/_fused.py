@@ -381,6 +381,20 @@ def order_residuals(raw, rows, cols, seg_len, block, position, held):
     return np.ascontiguousarray(ordered).reshape(-1)
 
 
+def order_records(raw, rows, cols, seg_len, block, position, held, record_symbols, record_bytes):
+    """``order_residuals`` for records of another size: ``record_symbols`` consecutive symbols of a
+    row in ``record_bytes`` bytes (the predictive codec's 32 five-bit residuals in 20 bytes, or
+    the 32 four-bit reference bins in 16).  Record t of segment s of position q goes to
+    (((q // block * U + t) * spr + s) * block + q % block) * record_bytes, U = seg_len //
+    record_symbols; positions that no row has hold zeros."""
+    spr, per_seg = cols // seg_len, seg_len // record_symbols
+    ordered = np.zeros((held, per_seg, spr, record_bytes), dtype=np.uint8)
+    ordered[position] = np.asarray(raw)[:rows * spr * per_seg * record_bytes].reshape(
+        rows, spr, per_seg, record_bytes).transpose(0, 2, 1, 3)
+    ordered = ordered.reshape(held // block, block, per_seg, spr, record_bytes).transpose(0, 2, 3, 1, 4)
+    return np.ascontiguousarray(ordered).reshape(-1)
+
+
 def build_tiles(row_class, nr, r):
     """Rows grouped by class (index order inside a class), cut into tiles of r rows."""
     order = np.argsort(row_class, kind="stable").astype(np.uint32)

@@ -22,7 +22,9 @@ class GrfBctxFrame(ctypes.Structure):
 class GrfPpcxFrame(ctypes.Structure):
     _fields_ = [("main", GrfStream), ("residual", GrfStream), ("labels", ctypes.c_void_p),
                 ("flips", ctypes.c_void_p), ("thresholds", ctypes.c_void_p), ("rows", ctypes.c_uint32),
-                ("cols", ctypes.c_uint32), ("mode", ctypes.c_uint32), ("stride", ctypes.c_uint32)]
+                ("cols", ctypes.c_uint32), ("mode", ctypes.c_uint32), ("stride", ctypes.c_uint32),
+                ("raw5_row_pos", ctypes.c_void_p), ("raw5_segment", ctypes.c_uint32),
+                ("raw5_block_rows", ctypes.c_uint32)]
 
 
 class GrfBctxFused(ctypes.Structure):
@@ -42,16 +44,16 @@ class GrfFusedTiling(ctypes.Structure):
 
 class GrfPpcxFused(ctypes.Structure):
     _fields_ = [(name, ctypes.c_void_p) for name in (
-        "main_bytes", "raw5", "seg_state", "seg_offset", "lut", "tab")] + [
+        "main_bytes", "raw5", "seg_state", "seg_offset", "lut", "tab", "row_pos")] + [
         (name, ctypes.c_uint32) for name in (
             "main_n_bytes", "rows", "cols", "n_labels", "seg_len", "segs_per_row", "shift", "lognb", "tabn",
-            "whole_range")]
+            "whole_range", "raw_interleaved")]
 
 
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
                   "grf_bctx_fused_decode", "grf_bctx_fused_gather", "grf_bctx_fused_validate_host", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
                   "grf_gemm_workspace_bytes", "grf_gemm_workspace_bytes_split", "grf_bctx_gemm_noalloc", "grf_gemm_noalloc_limit_bytes", "grf_pack_activations", "grf_bctx_gemv_group", "grf_bctx_gemm_group",
-                  "grf_ppcx_bins", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_last_error",
+                  "grf_ppcx_bins", "grf_ppcx_bins_ordered", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_last_error",
                   "grf_abi_version", "grf_timestamp", "grf_wall_clock_khz")
 
 
@@ -95,6 +97,8 @@ def declare(L):
     L.grf_bctx_fused_lds_bytes.restype = u32
     L.grf_ppcx_bins.argtypes = [vp, vp, vp, u32, u32, vp, vp]
     L.grf_ppcx_bins.restype = i
+    L.grf_ppcx_bins_ordered.argtypes = [vp, vp, vp, u32, u32, u32, u32, vp, vp, vp]
+    L.grf_ppcx_bins_ordered.restype = i
     L.grf_ppcx_fused_decode.argtypes = [ctypes.POINTER(GrfPpcxFused), tiling, vp, vp, vp, vp]
     L.grf_ppcx_fused_decode.restype = i
     L.grf_ppcx_gemv.argtypes = [ctypes.POINTER(GrfPpcxFused), tiling, vp, vp, u32, u32, vp, u32, vp, vp, vp]

@@ -160,6 +160,19 @@ class HipPredictiveTensor:
         for key in ("source_sha256", "target_sha256", "reference_sha256", "frame_sha256", "frame_bytes"):
             setattr(self, key, ix[key])
         self.buffers = {}
+        # The packed residuals -- and the plane of reference bins made below -- in the order the
+        # tile walker reads them: records of 32 symbols (20 and 16 bytes), rows by label as the
+        # tilings take them, in blocks of as many rows as a wave unit of the GEMV has; inside a
+        # block by position in the segment, then by segment, then by row (the order the context
+        # codec's tensors give their 12-byte groups, for the same reason: the lanes of a unit then
+        # read one run of bytes per visit and a 128-byte line is not visited four times).
+        self._raw5_segment = self._raw5_block = self._rows_held = 0
+        if self._plan is not None and "raw5" in ix and self.resident_mode == 0:
+            block, position, held = self._plan.residual_order()
+            rows_, cols_ = self.shape
+            ix["raw5"] = _fused.order_records(ix["raw5"], rows_, cols_, self._plan.seg_len, block, position, held, 32, 20)
+            ix["row_pos"] = position
+            self._raw5_segment, self._raw5_block, self._rows_held = self._plan.seg_len, block, held
         for name, array in ix.items():
             if isinstance(array, np.ndarray) and name != "residual_symbols":
                 if name in ("raw5", "main_stream"):  # the kernels read whole dwords / 16-byte chunks at the end
@@ -205,6 +218,8 @@ class HipPredictiveTensor:
             f.main.states, f.main.offsets = b["main_states"].data_ptr(), b["main_offsets"].data_ptr()
             if self.resident_mode == 0:
                 f.residual.bytes, f.residual.n_bytes = b["raw5"].data_ptr(), b["raw5"].numel() - 16
+                f.raw5_segment, f.raw5_block_rows = self._raw5_segment, self._raw5_block
+                f.raw5_row_pos = b["row_pos"].data_ptr() if self._raw5_segment else None
             else:
                 f.residual.bytes, f.residual.n_bytes = b["residual_stream"].data_ptr(), b["residual_stream"].numel()
                 f.residual.vocab, f.residual.nctx = codec.RES_VOCAB, codec.RES_CONTEXTS
@@ -260,6 +275,8 @@ class HipPredictiveTensor:
         f.seg_len, f.segs_per_row, f.shift, f.lognb, f.tabn = (sc["seg_len"], sc["segs_per_row"], sc["shift"],
                                                                 sc["lognb"], sc["tabn"])
         f.whole_range = sc["whole_range"]
+        f.raw_interleaved = self._raw5_block if self._raw5_segment else 0
+        f.row_pos = b["row_pos"].data_ptr() if self._raw5_segment else None
         self.fused = f
         store = self._tiling_for(0)
         self.fused_plan = dict(sc, **store[3])
@@ -283,11 +300,17 @@ class HipPredictiveTensor:
     def _bins(self, ref):
         """Transient plane of 4-bit bins of the reference words (one launch)."""
         import torch
-        bins = torch.empty(self.n // 8, device=self.device, dtype=torch.int32)
         b = self.buffers
-        status = self._lib.grf_ppcx_bins(ref.data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr(),
-                                         self.shape[0], self.shape[1], bins.data_ptr(),
-                                         torch.cuda.current_stream(self.device).cuda_stream)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        if self._raw5_segment:  # in the residuals' blocked order (dwords of positions no row has stay unwritten, unread)
+            bins = torch.empty(self._rows_held * self.shape[1] // 8, device=self.device, dtype=torch.int32)
+            status = self._lib.grf_ppcx_bins_ordered(ref.data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr(),
+                                                     self.shape[0], self.shape[1], self._raw5_segment, self._raw5_block,
+                                                     b["row_pos"].data_ptr(), bins.data_ptr(), stream)
+        else:
+            bins = torch.empty(self.n // 8, device=self.device, dtype=torch.int32)
+            status = self._lib.grf_ppcx_bins(ref.data_ptr(), b["flips"].data_ptr(), b["thresholds"].data_ptr(),
+                                             self.shape[0], self.shape[1], bins.data_ptr(), stream)
         return bins, status
 
     def _contexts(self, reference_bf16_device):

@@ -88,6 +88,17 @@ __global__ __launch_bounds__(kThreads) void bctx_decode_kernel(grf_bctx_frame f,
   if (bad) atomicOr(error, (int)bad);
 }
 
+// Index of element (row, col) among the packed 5-bit fields: the frame's own order, or, for a
+// tensor that keeps them for the fused kernels, records of 32 in blocks of rows, ordered by their
+// position in the segment, the segment's number and the row inside the block.
+__device__ __forceinline__ uint64_t raw5_index(const grf_ppcx_frame &f, uint32_t row, uint32_t col) {
+  if (!f.raw5_segment) return (uint64_t)row * f.cols + col;
+  const uint32_t S = f.raw5_segment, spr = f.cols / S, B = f.raw5_block_rows ? f.raw5_block_rows : 1;
+  const uint32_t q = f.raw5_row_pos ? f.raw5_row_pos[row] : row, within = q % B;
+  const uint64_t record = (uint64_t)(q - within) * (f.cols / 32) + ((uint64_t)((col % S) / 32) * spr + col / S) * B + within;
+  return record * 32 + col % 32;
+}
+
 // MODE1: residual is a second rANS stream (vocab 32) whose context is the main symbol.
 template <bool MODE1>
 __global__ __launch_bounds__(kThreads) void ppcx_decode_kernel(grf_ppcx_frame f, const uint16_t *reference,
@@ -121,7 +132,7 @@ __global__ __launch_bounds__(kThreads) void ppcx_decode_kernel(grf_ppcx_frame f,
       r = grf::rans_step_global(rstate, rip, f.residual.bytes, f.residual.n_bytes,
                                 f.residual.cum + (size_t)m * 33, f.residual.bucket + (size_t)m * 256, bad);
     else
-      r = grf::packed_field<5>(f.residual.bytes, f.residual.n_bytes, start + t);
+      r = grf::packed_field<5>(f.residual.bytes, f.residual.n_bytes, raw5_index(f, row, col));
     dst[t] = (uint16_t)grf::ppcx_word(m, r);
     if (++col == f.cols) {
       col = 0;
@@ -249,8 +260,12 @@ int grf_ppcx_decode(const grf_ppcx_frame *frame, const uint16_t *reference, uint
   if (!stream_ok(f.main, true) || !stream_ok(f.residual, f.mode == 1))
     return fail(GRF_BAD_ARGUMENT, "grf_ppcx_decode: incomplete stream descriptor");
   const uint64_t n = (uint64_t)f.rows * f.cols;
-  if (f.mode == 0 && f.residual.n_bytes != (n * 5 + 7) / 8)
+  if (f.mode == 0 && (f.raw5_segment ? f.residual.n_bytes < (n * 5 + 7) / 8 : f.residual.n_bytes != (n * 5 + 7) / 8))
     return fail(GRF_BAD_ARGUMENT, "grf_ppcx_decode: packed residual length mismatch");
+  if (f.mode == 0 && f.raw5_segment &&
+      (f.raw5_segment % 32 || f.cols % f.raw5_segment || f.raw5_block_rows > 16 ||
+       (f.raw5_block_rows & (f.raw5_block_rows - 1))))
+    return fail(GRF_BAD_ARGUMENT, "grf_ppcx_decode: residual order (segment length, block rows)");
   const uint64_t segments = (n + f.stride - 1) / f.stride;
   const dim3 grid((unsigned)((segments + kThreads - 1) / kThreads)), block(kThreads);
   hipStream_t s = (hipStream_t)hip_stream;

@@ -28,9 +28,24 @@ namespace {
 // 4-bit bins out (element i of the matrix in bits 4*(i%8) of dword i/8).
 constexpr uint32_t kBinsThreads = 1024;
 
+// Where the two dwords of the group of 16 elements that starts at element `at` go: the frame's
+// order, or (block != 0) the blocked order of records of 32 elements (four dwords each).
+struct BinsOrder {
+  uint32_t cols, seg_len, segs_per_row, block;
+  const uint32_t *row_pos;
+  __device__ __forceinline__ uint64_t dword_of(uint64_t at) const {
+    if (!block) return at / 8;
+    const uint32_t row = (uint32_t)(at / cols), col = (uint32_t)(at % cols);
+    const uint32_t q = row_pos ? row_pos[row] : row, within = q % block;
+    const uint64_t record = (uint64_t)(q - within) * (cols / 32) +
+                            ((uint64_t)((col % seg_len) / 32) * segs_per_row + col / seg_len) * block + within;
+    return record * 4 + (col % 32) / 8;
+  }
+};
+
 __global__ __launch_bounds__(kBinsThreads) void ppcx_bins_kernel(const uint16_t *reference, const uint8_t *flips,
                                                                   const uint16_t *thresholds, uint32_t cols,
-                                                                  uint64_t n, uint32_t *bins) {
+                                                                  uint64_t n, uint32_t *bins, BinsOrder order) {
   extern __shared__ __align__(16) uint8_t table[];  // bin of the sign-aligned word
   __shared__ uint16_t th[16];
   if (threadIdx.x < 15) th[threadIdx.x] = thresholds[threadIdx.x];
@@ -67,7 +82,7 @@ __global__ __launch_bounds__(kBinsThreads) void ppcx_bins_kernel(const uint16_t 
         const uint32_t a = (i % 2) ? (w[i / 2] >> 16) : (w[i / 2] & 0xFFFFu);
         packed[i / 8] |= (uint32_t)table[a] << (4 * (i % 8));
       }
-      *reinterpret_cast<uint2 *>(bins + at[c] / 8) = make_uint2(packed[0], packed[1]);
+      *reinterpret_cast<uint2 *>(bins + order.dword_of(at[c])) = make_uint2(packed[0], packed[1]);
     }
   }
 }
@@ -104,29 +119,53 @@ struct PpcxWalk {
   grf::Cursor c;
   uint32_t gofs, eofs;        // byte offsets of this segment's and the next segment's checkpoints
   uint32_t end_state, end_jb;  // what the walk must end on: the next checkpoint's state, and its offset as an LDS cursor
-  const uint8_t *rawp;    // the segment's first residual byte (5 * S / 8 bytes per segment)
-  const uint2 *binp;      // the segment's bins, 8 bytes per 16 symbols
+  const uint8_t *rawp;    // the residual array (uniform)
+  const uint2 *binp;      // the bins plane (uniform)
   uint32_t n0, n1, n2;
   uint2 nb;
   Raw5x16 rr;      // the group being decoded
   uint32_t bw[2];
 
-  __device__ __forceinline__ static const uint32_t *group_dwords(const uint8_t *rawp, uint32_t g) {
-    return reinterpret_cast<const uint32_t *>(rawp + ((10 * g) & ~3u));
+  // The residuals and bins of the group of 16 symbols g of the segment: in the frame's order a
+  // segment's bytes are one run (10 and 8 bytes a group); in the blocked order a record of two
+  // groups (20 and 16 bytes) is followed by the same record of the block's next row.  Either
+  // way the second group of a record starts two bytes into its third dword.
+  uint32_t raw_off, bin_off;        // byte offsets of the segment's first record in the two arrays
+  uint32_t raw_stride, bin_stride;  // bytes from a record to the segment's next record
+  __device__ __forceinline__ const uint32_t *group_dwords(uint32_t g) const {
+    return reinterpret_cast<const uint32_t *>(rawp + (raw_off + (g >> 1) * raw_stride + (g & 1u) * 8u));
+  }
+  __device__ __forceinline__ uint2 group_bins(uint32_t g) const {
+    return *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint8_t *>(binp) +
+                                            (bin_off + (g >> 1) * bin_stride + (g & 1u) * 8u));
   }
   // global reads of the segment, issued before the wait for the slab's stream bytes
-  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t, uint32_t, uint32_t) {
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t,
+                                           uint32_t seg_in_row, uint32_t rpos) {
     gofs = grf::fused_index_entry(f.seg_offset, seg_);
     eofs = grf::fused_index_entry(f.seg_offset, seg_ + 1);
     c.state = grf::fused_index_entry(f.seg_state, seg_);
     end_state = grf::fused_index_entry(f.seg_state, seg_ + 1);
-    rawp = f.raw6 + elem0 / 8 * 5;
-    binp = reinterpret_cast<const uint2 *>(f.col_class) + elem0 / 16;
-    const uint32_t *d = group_dwords(rawp, 0);
+    rawp = f.raw6;
+    binp = reinterpret_cast<const uint2 *>(f.col_class);
+    if (f.raw_interleaved) {
+      const uint32_t B = f.raw_interleaved, within = rpos & (B - 1);
+      const uint32_t record = (rpos - within) * (f.cols / 32) + seg_in_row * B + within;  // (once per segment)
+      raw_off = record * 20;
+      bin_off = record * 16;
+      raw_stride = f.segs_per_row * B * 20;
+      bin_stride = f.segs_per_row * B * 16;
+    } else {
+      raw_off = elem0 / 8 * 5;
+      bin_off = elem0 / 2;
+      raw_stride = 20;
+      bin_stride = 16;
+    }
+    const uint32_t *d = group_dwords(0);
     n0 = d[0];
     n1 = d[1];
     n2 = d[2];
-    nb = binp[0];
+    nb = group_bins(0);
   }
   __device__ __forceinline__ void start(uint32_t piece_off, uint32_t a0) {
     c.jb = (piece_off + (gofs - a0)) << 3;
@@ -139,11 +178,11 @@ struct PpcxWalk {
     bw[1] = nb.y;
     // the last group loads itself again rather than branch around the loads
     const uint32_t next = min(t / 16 + 1, S / 16 - 1);
-    const uint32_t *d = group_dwords(rawp, next);
+    const uint32_t *d = group_dwords(next);
     n0 = d[0];
     n1 = d[1];
     n2 = d[2];
-    nb = binp[next];
+    nb = group_bins(next);
   }
   template <int H, int SCAN = grf::kScanAny>
   __device__ __forceinline__ void half(const grf::FusedParams &q, uint32_t (&pair)[4]) {
@@ -198,6 +237,8 @@ int walker_frame(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, co
   f.lognb = frame->lognb;
   f.tabn = frame->tabn;
   f.whole_range = frame->whole_range;
+  f.raw_interleaved = frame->raw_interleaved;
+  f.row_pos = frame->row_pos;
   if (int rc = grf::check_fused_frame(f, *tiling, who, use)) return rc;
   if (f.seg_len % 32)  // a segment's residual bytes must start on a dword
     return grf::set_error(GRF_UNSUPPORTED, std::string(who) + ": segment length must be a multiple of 32");
@@ -208,22 +249,32 @@ int walker_frame(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, co
 
 extern "C" {
 
-int grf_ppcx_bins(const uint16_t *reference, const uint8_t *flips, const uint16_t *thresholds, uint32_t rows,
-                  uint32_t cols, uint32_t *bins, void *hip_stream) {
+int grf_ppcx_bins_ordered(const uint16_t *reference, const uint8_t *flips, const uint16_t *thresholds, uint32_t rows,
+                          uint32_t cols, uint32_t seg_len, uint32_t block_rows, const uint32_t *row_pos,
+                          uint32_t *bins, void *hip_stream) {
   if (!reference || !flips || !thresholds || !bins)
     return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_bins: null argument");
   if (!rows || !cols || cols % 16 || ((uintptr_t)reference & 15) || ((uintptr_t)bins & 7))
     return grf::set_error(GRF_BAD_ARGUMENT,
                           "grf_ppcx_bins: row length must be a multiple of 16, reference 16-byte and bins 8-byte aligned");
+  if (block_rows && (block_rows > 16 || (block_rows & (block_rows - 1)) || !seg_len || seg_len % 32 || cols % seg_len))
+    return grf::set_error(GRF_BAD_ARGUMENT,
+                          "grf_ppcx_bins_ordered: blocks of 1, 2, 4, 8 or 16 rows, segments a multiple of 32 that divides the row");
   const uint64_t n = (uint64_t)rows * cols;
   if (n > 0xFFFFFFFFull) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_bins: matrix too large");
   const uint64_t chunks = (n / 16 + kBinsThreads - 1) / kBinsThreads;
   const uint32_t blocks = (uint32_t)(chunks < 512 ? chunks : 512);  // two workgroups per CU amortise the table
+  const BinsOrder order{cols, seg_len, seg_len ? cols / seg_len : 0, block_rows, row_pos};
   hipLaunchKernelGGL(ppcx_bins_kernel, dim3(blocks), dim3(kBinsThreads), 65536, (hipStream_t)hip_stream, reference,
-                     flips, thresholds, cols, n, bins);
+                     flips, thresholds, cols, n, bins, order);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return grf::set_error(GRF_LAUNCH_FAILED, std::string("bins kernel: ") + hipGetErrorString(e));
   return GRF_OK;
+}
+
+int grf_ppcx_bins(const uint16_t *reference, const uint8_t *flips, const uint16_t *thresholds, uint32_t rows,
+                  uint32_t cols, uint32_t *bins, void *hip_stream) {
+  return grf_ppcx_bins_ordered(reference, flips, thresholds, rows, cols, 0, 0, nullptr, bins, hip_stream);
 }
 
 int grf_ppcx_fused_decode(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, const uint32_t *bins,

@@ -146,6 +146,12 @@ typedef struct grf_ppcx_frame {
   uint32_t rows, cols;
   uint32_t mode;
   uint32_t stride;
+  /* mode 0 only: the order of the packed 5-bit fields.  raw5_segment == 0: the frame's own
+   * order.  Otherwise the blocked order grf_ppcx_fused describes (records of 32 fields, segments
+   * of raw5_segment symbols, blocks of raw5_block_rows rows at the positions raw5_row_pos gives,
+   * NULL = the row itself), so that one resident array serves this kernel and the tile walker. */
+  const uint32_t *raw5_row_pos;
+  uint32_t raw5_segment, raw5_block_rows;
 } grf_ppcx_frame;
 
 /* Replaces the Triton launch of the predictive decode_words
@@ -368,7 +374,15 @@ uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_t
  *   lut  u8 [n_labels][16 << lognb], tab u64 [n_labels][16][tabn+1]   as in grf_bctx_fused:
  *        low32 = start | (freq & 0xFFFF)<<16, high32 = the symbol's bits in the BF16 word
  *        (sign, exponent, mantissa bits 6..5) in place of symbol<<5
- * seg_len must be a multiple of 32.  Tilings are built over row labels. */
+ * seg_len must be a multiple of 32.  Tilings are built over row labels.
+ * raw_interleaved: 0 = raw5, and the bins plane given with every call, in the frame's order
+ * (element i of the matrix: field i of raw5; bits 4*(i%8) of bins[i/8]).  B = 1, 2, 4, 8 or 16 =
+ * both in records of 32 consecutive symbols of a row (20 bytes of raw5, 16 of bins), in blocks
+ * of B rows: with q the row's position (row_pos[r], or r when row_pos is null) and U =
+ * seg_len / 32, record t of segment s lies at index ((q / B * U + t) * segs_per_row + s) * B +
+ * q % B -- the order grf_bctx_fused gives its 12-byte groups, for the same reason: the lanes of
+ * a wave unit then read one run of bytes per visit.  grf_ppcx_bins_ordered writes a plane in
+ * that order. */
 typedef struct grf_ppcx_fused {
   const uint8_t *main_bytes;
   const uint8_t *raw5;
@@ -376,12 +390,14 @@ typedef struct grf_ppcx_fused {
   const uint32_t *seg_offset;
   const uint8_t *lut;
   const uint64_t *tab;
+  const uint32_t *row_pos;
   uint32_t main_n_bytes;
   uint32_t rows, cols;
   uint32_t n_labels;
   uint32_t seg_len, segs_per_row;
   uint32_t shift, lognb, tabn;
   uint32_t whole_range; /* as in grf_bctx_fused */
+  uint32_t raw_interleaved;
 } grf_ppcx_fused;
 
 /* The bin of every reference word (GCR/bitexact_predictive_codec.py:106-110, device form
@@ -391,6 +407,14 @@ typedef struct grf_ppcx_fused {
  * flips u8 [rows]; thresholds u16 [15]; bins u32 [rows*cols/8]. */
 int grf_ppcx_bins(const uint16_t *reference, const uint8_t *flips, const uint16_t *thresholds, uint32_t rows,
                   uint32_t cols, uint32_t *bins, void *hip_stream);
+/* The same plane in the blocked order of a grf_ppcx_fused with raw_interleaved = block_rows
+ * (seg_len, row_pos as there; cols % 32 == 0, seg_len % 32 == 0): bins u32 [rows_held * cols / 8]
+ * with rows_held the rows the order holds (a multiple of block_rows above the largest
+ * position); dwords of positions no row has are not written.  block_rows == 0 is
+ * grf_ppcx_bins. */
+int grf_ppcx_bins_ordered(const uint16_t *reference, const uint8_t *flips, const uint16_t *thresholds, uint32_t rows,
+                          uint32_t cols, uint32_t seg_len, uint32_t block_rows, const uint32_t *row_pos,
+                          uint32_t *bins, void *hip_stream);
 
 /* Decode a prepared PPCX frame to dense BF16 words given the bins of its reference (replaces
  * the Triton launch of CudaPredictiveTensor.decode, GCR/bitexact_predictive_gpu.py:160-174,

@@ -112,7 +112,9 @@ def test_ppcx_wrong_reference_on_device_sets_error(oracle):
         t.decode(None)
     # a tensor that keeps its context plane (the default) needs no reference after construction
     kept = HipPredictiveTensor(frame, ref, stride=64)
-    assert kept.has_contexts and kept.resident_bytes == t.resident_bytes + target.size // 2
+    plane = kept.buffers["context_bins"].numel() * 4  # half a byte per weight (+ the rows the blocked order pads a label to)
+    assert kept.has_contexts and kept.resident_bytes == t.resident_bytes + plane
+    assert target.size // 2 <= plane <= (target.shape[0] + 16 * 16) * target.shape[1] // 2
     assert np.array_equal(kept.decode(None).view(torch.uint16).cpu().numpy(), target)
     x = torch.from_numpy(bf16_words(np.random.default_rng(5).normal(0, 1, size=(3, target.shape[1])))).view(torch.bfloat16).cuda()
     ref_dev = torch.from_numpy(ref).view(torch.bfloat16).cuda()
