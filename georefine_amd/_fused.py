@@ -479,15 +479,21 @@ class FramePlan:
         self.class_rows = np.bincount(self.row_class, minlength=nr)
         self._caps = {}
 
-    def residual_order(self):
+    def residual_order(self, block=None):
         """(block rows B, row positions u32[rows], rows of the array) of the resident residual
         order: the rows by class, index order inside a class, as every tiling takes them, each
         class starting on a multiple of 16; B = the rows of a wave unit of the GEMV (1 where
-        the GEMV has no wave tiling), so that a unit's rows are the rows of one block."""
-        try:
-            block = 64 // self.tiling(1, waves=True)["scalars"]["lanes_per_row"]
-        except FusedUnsupported:
-            block = 1
+        the GEMV has no wave tiling), so that a unit's rows are the rows of one block -- or the
+        ``block`` asked for (1, 2, 4, 8, 16): 16 makes a wave of the matrix-core kernel, which
+        holds sixteen rows, read whole lines, for matrices that are served in batches."""
+        if block is not None:
+            if block not in (1, 2, 4, 8, 16):
+                raise FusedUnsupported("residual blocks have 1, 2, 4, 8 or 16 rows")
+        else:
+            try:
+                block = 64 // self.tiling(1, waves=True)["scalars"]["lanes_per_row"]
+            except FusedUnsupported:
+                block = 1
         order = np.argsort(self.row_class, kind="stable")
         starts = np.zeros(self.nr + 1, dtype=np.int64)
         for rho in range(self.nr):

@@ -193,7 +193,7 @@ class HipContextTensor:
     GEMV_UP_TO, GEMM_TWO_ROWS_FROM, DENSE_ABOVE = GEMV_UP_TO, GEMM_TWO_ROWS_FROM, DENSE_ABOVE
 
     @staticmethod
-    def host_prepare(frame: bytes, *, stride: int = 1024, fused=True, fused_segment=None):
+    def host_prepare(frame: bytes, *, stride: int = 1024, fused=True, fused_segment=None, residual_block=None):
         """The host half of the constructor -- parse, validate and index the frame, lay out the
         fused kernels' tables -- for callers that prepare frames on worker threads and construct
         the device objects later (``HipContextTensor(frame, prepared=...)`` then only uploads).
@@ -231,7 +231,7 @@ class HipContextTensor:
             seg = indexed["fused_segment"]
             raw = indexed["residual_stream"]
             if raw.size == rows_ * cols_ * 3 // 4:
-                block, position, held = plan.residual_order()
+                block, position, held = plan.residual_order(residual_block)
                 indexed["residual_stream"] = _fused.order_residuals(raw, rows_, cols_, seg, block, position, held)
                 indexed["row_pos"] = position
                 raw6_segment, raw6_block = seg, block
@@ -241,7 +241,7 @@ class HipContextTensor:
                 "main_bytes": main_bytes, "raw6_segment": raw6_segment, "raw6_block": raw6_block}
 
     def __init__(self, frame: bytes, *, stride: int = 1024, device="cuda:0", fused=True, fused_segment=None,
-                 m_invariant=False, prepared=None):
+                 m_invariant=False, prepared=None, residual_block=None):
         import torch
         if not torch.cuda.is_available():
             raise RuntimeError("a ROCm GPU is required")
@@ -250,7 +250,8 @@ class HipContextTensor:
         # that a row's output bits never depend on the rows it arrives with (route_rows)
         self.m_invariant = bool(m_invariant)
         if prepared is None:
-            prepared = self.host_prepare(frame, stride=stride, fused=fused, fused_segment=fused_segment)
+            prepared = self.host_prepare(frame, stride=stride, fused=fused, fused_segment=fused_segment,
+                                         residual_block=residual_block)
         elif prepared["stride"] != stride or prepared["fused"] != fused:
             raise ValueError("the frame was prepared with another stride or fused setting")
         indexed, plan = prepared["indexed"], prepared["plan"]
@@ -330,14 +331,27 @@ class HipContextTensor:
             except _fused.FusedUnsupported:
                 pass  # reported by the call that needs it
 
-    def clone(self):
+    def clone(self, residual_block=None):
         """A second resident copy of the same coded matrix: every device buffer is duplicated
         (nothing is decoded or indexed again), so a stack of layers with equal weights can be
-        laid out in device memory at the cost of one device-to-device copy each."""
+        laid out in device memory at the cost of one device-to-device copy each.
+        ``residual_block``: the copy keeps its packed residuals in blocks of that many rows (1,
+        2, 4, 8 or 16; see ``host_prepare``), re-ordered on the device: a permutation of the
+        12-byte groups, no field is touched."""
         import copy
         import torch
         other = copy.copy(self)
         other.buffers = {k: v.clone() for k, v in self.buffers.items()}
+        if residual_block is not None and self._raw6_segment and residual_block != self._raw6_block:
+            if residual_block not in (1, 2, 4, 8, 16):
+                raise ValueError("residual blocks have 1, 2, 4, 8 or 16 rows")
+            old, groups, spr = self._raw6_block, self._raw6_segment // 16, self.shape[1] // self._raw6_segment
+            raw = other.buffers["residual_stream"]
+            held = raw.numel() // (groups * spr * 12)  # a multiple of 16: every class starts on one
+            by_row = raw[:held * groups * spr * 12].view(held // old, groups, spr, old, 12).permute(0, 3, 1, 2, 4)
+            by_row = by_row.reshape(held // residual_block, residual_block, groups, spr, 12)
+            other.buffers["residual_stream"] = by_row.permute(0, 2, 3, 1, 4).contiguous().view(-1)
+            other._raw6_block = residual_block
         other.error = torch.zeros_like(self.error)
         other.resident_bytes = int(sum(t.numel() * t.element_size() for t in other.buffers.values())
                                    + other.error.numel() * other.error.element_size())

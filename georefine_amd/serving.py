@@ -20,12 +20,16 @@ class ContextServingError(RuntimeError):
     """Malformed or incomplete coded-weight module."""
 
 
-def hip_tensor_factory(frame, *, stride=1024, device="cuda:0", fused_segment=None):
+def hip_tensor_factory(frame, *, stride=1024, device="cuda:0", fused_segment=None, residual_block=None):
     """The ``tensor_factory`` to hand to ``load_bctx_model`` (GCR/bitexact_context_serving.py:416,560).
     ``fused_segment`` fixes the segment length of the fused index (matrices that are to share a
-    launch need one length); the loader passes it to factories that take it."""
+    launch need one length); the loader passes it to factories that take it.  ``residual_block``
+    (``functools.partial(hip_tensor_factory, residual_block=16)``): the rows per block of the
+    resident residual order; 16 suits matrices that are served in batches (the matrix-core
+    kernel's waves hold sixteen rows), the default the one-row GEMV."""
     from .bitexact_context_gpu import HipContextTensor
-    return HipContextTensor(frame, stride=stride, device=device, fused_segment=fused_segment)
+    return HipContextTensor(frame, stride=stride, device=device, fused_segment=fused_segment,
+                            residual_block=residual_block)
 
 
 def hip_predictive_factory(frame, reference_uint16_numpy, stride=1024, device="cuda:0"):
@@ -150,11 +154,16 @@ class PredictiveContextTensor:
     """PPCX weight that resolves its reference tensors when decoded
     (GCR/bitexact_predictive_serving.py:490-523): one reference is used as is, two are mixed
     by ``predictor(up, gate, coefficients)``; ``transform == "target transpose"`` stores the
-    frame transposed."""
+    frame transposed.
+
+    ``row_major``: a coded tensor of the weight in the model's own orientation, made at load from
+    the decoded frame (``reframe`` below); products, decodes and row gathers then go to it and
+    the predictive frame's device buffers are released."""
 
     def __init__(self, native, references, *, predictor=None, coefficients=None, transform=None, shape,
                  source_sha256, frame_sha256, resident_bytes):
         self.native = native
+        self.row_major = None
         self.references = tuple(references)
         self.predictor = predictor
         self.coefficients = coefficients
@@ -170,7 +179,33 @@ class PredictiveContextTensor:
         walker: nothing of the references is then read after load."""
         return not (getattr(self.native, "has_contexts", False) and getattr(self.native, "fused", None) is not None)
 
+    def reframe(self, tensor_factory, *, stride, device, encoder=None):
+        """A frame stored transposed holds W^T row by row: the walk produces words along the
+        product's K axis, which no sink of the tile walker can contract.  The reference's shipped
+        servers re-frame their Context weights at start-up (GS/predictive_tbe.py:1-15); this does
+        the same for such targets, once: the frame is decoded on the device (the index builder has
+        already checked it against its digests), turned, encoded row-major with the context
+        codec's encoder, and the new frame is indexed like any other -- the decoded words of the
+        result must hash to the receipt's ``source_sha256`` of the tensor.  Every later product is
+        then one fused launch and ``decode()`` a fused decode; the predictive frame's device
+        buffers are released.  Returns the new tensor."""
+        import numpy as np
+        if encoder is None:
+            from .bitexact_context_codec import encode as encoder
+        with self._decode_lock:
+            words = self.decode(check=True).view(torch.uint16).cpu().numpy()
+            tensor = tensor_factory(encoder(np.ascontiguousarray(words)), stride=stride, device=device)
+            if tuple(tensor.shape) != tuple(words.shape) or tensor.source_sha256 != self.source_sha256:
+                raise ContextServingError("re-framed tensor does not reproduce the decoded source")
+            self.row_major = tensor
+            self.resident_bytes = int(tensor.resident_bytes)
+            self.native = None  # its device buffers go with it
+            self.references = ()
+        return tensor
+
     def decode(self, *, check=True):
+        if self.row_major is not None:
+            return self.row_major.decode(check=check)
         with self._decode_lock:
             value = self.native.decode(self._reference(check) if self._needs_reference() else None, check=check)
             if self.transform == "target transpose":
@@ -178,6 +213,8 @@ class PredictiveContextTensor:
             return value
 
     def gather_rows(self, ids, *, check=True):
+        if self.row_major is not None:
+            return self.row_major.gather_rows(ids, check=check)
         return self.decode(check=check)[ids]
 
     def _reference(self, check):
@@ -194,7 +231,13 @@ class PredictiveContextTensor:
         product: one launch that decodes and contracts, with the contexts of the reference read
         from the plane kept at load (a native tensor without that plane gets the reference
         decoded first); a transposed frame holds W^T row by row, so it is decoded and multiplied
-        densely."""
+        densely -- unless it was re-framed at load (``reframe``), in which case the row-major tensor's
+        fused product runs."""
+        if self.row_major is not None:
+            fused = getattr(self.row_major, "linear", None)
+            if fused is None:  # a tensor class without a fused product
+                return torch.nn.functional.linear(x, self.row_major.decode(check=check), bias)
+            return fused(x, bias, check=check, batch_invariant=batch_invariant)
         fused = getattr(self.native, "linear", None)
         if fused is None or self.transform == "target transpose":
             return torch.nn.functional.linear(x, self.decode(check=check), bias)
@@ -227,7 +270,7 @@ def _runtime_dtype(model, name, parameter, requested):
 def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
                     tensor_factory=None, predictive_factory=None, mix_predictor=None, host_decoder=None,
                     loader_workers=1, batch_invariant=False, log=print, progress_callback=None,
-                    share_launches=()):
+                    share_launches=(), reframe_transposed=True):
     """Build ``model_factory()`` on the meta device and fill it from a BCTX package without
     ever holding a dense checkpoint: returns ``(model, receipt)``.
 
@@ -246,7 +289,14 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
     stride=, device=)`` indexes the frame against the reference words (for ``mixbf16`` the
     row-wise mix of two references with the candidate's coefficients, whose digest is
     checked), and the module receives a ``PredictiveContextTensor`` that resolves the
-    references when it decodes.  ``share_launches`` names sibling linears that are applied to
+    references when it decodes.  A candidate stored transposed (``target transpose``: the real
+    model's down projections, GCR/bitexact_predictive_serving.py:909-933) cannot be contracted by
+    the tile walker as it lies; with ``reframe_transposed`` (the default) it is decoded once at load,
+    turned and encoded row-major with the context codec, and that frame stays resident instead
+    (``PredictiveContextTensor.reframe``; the receipt lists such tensors under
+    ``reframed_tensors`` and counts them as transcoded), so its products are fused launches with
+    no dense transient; off, it is decoded to a dense transient and multiplied by the library
+    on every call, which is what the reference does with every frame.  ``share_launches`` names sibling linears that are applied to
     one tensor, e.g. ``[("q_proj", "k_proj", "v_proj"), ("gate_proj", "up_proj")]``: wherever a
     module has all the children of a tuple as coded linears of one input width (and the device
     tensors support it), they are indexed with one segment length and multiplied in one
@@ -462,6 +512,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
             raise ContextServingError(f"derived reference checksum mismatch: {name}")
         return derived
 
+    reframed = []
     for name in order:
         if name not in selected:
             continue
@@ -486,6 +537,15 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
             predictor=mix_predictor if c["mode"] == "mixbf16" else None, coefficients=coefficients,
             transform=c["transform"], shape=pkg.frame_shape(row["shape"]), source_sha256=row["source_sha256"],
             frame_sha256=c["frame_sha256"], resident_bytes=own)
+        if reframe_transposed and c["transform"] == "target transpose" and hasattr(native, "decode"):
+            try:
+                wrapped.reframe(tensor_factory, stride=stride, device=device)
+                own = wrapped.resident_bytes
+                reframed.append(name)
+            except ContextServingError:
+                raise
+            except Exception as exc:  # the frame stays as it is: decode + dense product per call
+                log(f"[bctx] {name}: not re-framed ({exc})")
         accept(name, (wrapped, own))
     host_words.clear()
 
@@ -493,7 +553,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         """What the device holds of a coded tensor, where the backend says so: the frame's mode,
         the mode of the resident form (a frame whose conditional residual stream was re-packed
         into 6-bit fields at load is resident in mode 0), and whether the fused kernels take it."""
-        native = getattr(context, "native", context)
+        native = getattr(context, "row_major", None) or getattr(context, "native", context)
         if not hasattr(native, "resident_mode"):
             return {}
         fused = getattr(native, "fused", None) is not None
@@ -569,7 +629,9 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         "consumed_tensors": consumed, "restored_bf16_control": False,
         # true when a frame's residual stream is resident in another form than the frame's own
         # (re-packed 6-bit fields); the main stream and the decoded words are never altered
-        "transcoded": any(r.get("residual_repacked") for r in consumed.values()),
+        "transcoded": any(r.get("residual_repacked") for r in consumed.values()) or bool(reframed),
+        # predictive frames stored transposed that were decoded, turned and encoded row-major at load
+        "reframed_tensors": sorted(reframed),
         "residual_repacked_tensors": sorted(n for n, r in consumed.items() if r.get("residual_repacked")),
         "general_kernel_tensors": sorted(n for n, r in consumed.items()
                                          if r.get("fused") is False and r.get("frame_mode") != 1),
@@ -582,7 +644,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
 def load_predictive_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
                           tensor_factory=None, context_factory=None, predictive_factory=None, mix_predictor=None,
                           host_decoder=None, loader_workers=1, batch_invariant=False, log=print,
-                          progress_callback=None, share_launches=()):
+                          progress_callback=None, share_launches=(), reframe_transposed=True):
     """The predictive-package loader under the reference's name and keywords
     (GCR/bitexact_predictive_serving.py:596-619): ``context_factory`` makes the BCTX tensors
     (``tensor_factory`` is accepted as its older spelling), ``predictive_factory`` the PPCX ones,
@@ -599,5 +661,5 @@ def load_predictive_model(package, *, model_factory, device="cuda:0", dtype=torc
                            tensor_factory=context_factory or tensor_factory, predictive_factory=predictive_factory,
                            mix_predictor=mix_predictor, host_decoder=host_decoder, loader_workers=loader_workers,
                            batch_invariant=batch_invariant, log=log, progress_callback=progress_callback,
-                           share_launches=share_launches)
+                           share_launches=share_launches, reframe_transposed=reframe_transposed)
 

@@ -98,6 +98,31 @@ def test_package_with_predictive_candidates_on_device(tmp_path):
             dict(dense.named_parameters())[name].copy_(torch.from_numpy(words).view(torch.bfloat16).cuda())
     x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(6, 256)))).view(torch.bfloat16).cuda()
     assert torch.allclose(model(x).float(), dense(x).float(), rtol=2e-2, atol=2e-2)
+    # The down projection is stored transposed: by default the loader decodes it once, turns it
+    # and keeps a row-major coded tensor, so its products are fused launches and no dense weight
+    # is ever materialised by a forward; the receipt says so.
+    assert receipt["reframed_tensors"] == ["down.weight"] and receipt["transcoded"]
+    down = model.down.context_weight
+    assert isinstance(down, serving.PredictiveContextTensor) and down.native is None
+    assert down.row_major.fused is not None and down.row_major.source_sha256 == down.source_sha256
+    assert down.resident_bytes == down.row_major.resident_bytes
+    assert receipt["consumed_tensors"]["down.weight"]["fused"] is True
+    before = model.down.weight_materializations
+    for rows in (1, 6):
+        model.down(x[:rows, :1].expand(rows, 384).contiguous())
+    model(x)
+    assert model.down.weight_materializations == before and model.down.forward_calls >= 3
+    h = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(5, 384)))).view(torch.bfloat16).cuda()
+    want = torch.nn.functional.linear(h.float(), torch.from_numpy(tensors["down.weight"]).view(torch.bfloat16).cuda().float())
+    assert torch.allclose(model.down(h).float(), want, rtol=2e-2, atol=2e-2)
+    assert torch.equal(model.down(h[:1]).view(torch.uint16), down.row_major.gemv(h[:1]).view(torch.uint16))
+    # without the re-frame the frame stays predictive: decoded and multiplied densely per call
+    kept, receipt2 = serving.load_bctx_model(path, model_factory=Gated, device="cuda:0", log=lambda _: None,
+                                             reframe_transposed=False)
+    assert receipt2["reframed_tensors"] == [] and kept.down.context_weight.row_major is None
+    assert kept.down.context_weight.native is not None
+    assert torch.allclose(kept(x).float(), dense(x).float(), rtol=2e-2, atol=2e-2)
+    assert np.array_equal(kept.down.weight.view(torch.uint16).cpu().numpy(), tensors["down.weight"])
 
 
 def test_sibling_projections_share_a_launch(tmp_path):

@@ -363,7 +363,7 @@ def test_loader_resolves_predictive_candidates(tmp_path):
     selected = pkg.read_candidates(path, manifest, entries)
     assert selected["down.weight"]["mode"] == "mixbf16" and selected["twin.weight"]["mode"] == "single"
     assert pkg.read_coefficients(path, selected["down.weight"]).shape == (16, 3)
-    model, receipt = _load(path, model_factory=GatedNet, predictive_factory=HostPredictive)
+    model, receipt = _load(path, model_factory=GatedNet, predictive_factory=HostPredictive, reframe_transposed=False)
     assert isinstance(model.down.context_weight, serving.PredictiveContextTensor)
     assert model.down.context_weight.transform == "target transpose" and model.down.context_weight.shape == (32, 16)
     for name, words in tensors.items():
@@ -378,6 +378,17 @@ def test_loader_resolves_predictive_candidates(tmp_path):
     assert receipt["compressed_tensor_count"] == 4
     assert receipt["consumed_tensors"]["down.weight"]["frame_sha256"] == selected["down.weight"]["frame_sha256"]
     assert receipt["resident_context_bytes"] == 37 + 37 + (11 + 16 * 3 * 2) + 11
+    assert receipt["reframed_tensors"] == [] and model.down.context_weight.row_major is None
+    # by default the target stored transposed is decoded once at load, turned and encoded
+    # row-major with the context codec: the tensor factory's object replaces the predictive one
+    turned, receipt = _load(path, model_factory=GatedNet, predictive_factory=HostPredictive)
+    down = turned.down.context_weight
+    assert receipt["reframed_tensors"] == ["down.weight"] and receipt["transcoded"] is True
+    assert isinstance(down.row_major, HostContext) and down.native is None and down.references == ()
+    assert down.row_major.source_sha256 == entries["down.weight"]["source_sha256"]
+    assert receipt["resident_context_bytes"] == 37 + 37 + 37 + 11
+    assert np.array_equal(turned.down.weight.view(torch.uint16).numpy(), tensors["down.weight"])
+    assert torch.equal(turned(x), dense(x))
 
 
 @pytest.mark.parametrize("edit,message", [
