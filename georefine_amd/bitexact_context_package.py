@@ -11,7 +11,9 @@ bytes against their pinned size and SHA-256.
 The writer covers what tests and small deployments need (every tensor coded with one
 (row classes, column classes) setting, optional sidecar files pinned by size and digest);
 the reference's package builder, with its per-tensor configuration search and archive of
-model assets, is outside this library.
+model assets, is outside this library.  What that builder writes is read in full:
+``verify_inventory`` checks the self-sized ``files`` inventory and ``restore`` rebuilds the
+source safetensors shards byte for byte from the retained headers and the decoded frames.
 
 Predictive candidates.  A manifest may carry ``selected_candidates``: tensors whose frame is
 a PPCX frame coded against one other tensor of the package (``mode`` "single") or against
@@ -281,6 +283,129 @@ def read_metadata(package, manifest):
             raise PackageError("package holds neither a metadata archive nor sidecar files")
         return {}
     return members if members is not None else physical
+
+
+# ------------------------------------------------------------------ whole-package inventory
+
+def _sha_file(path):
+    h = hashlib.sha256()
+    with open(path, "rb") as f:
+        for chunk in iter(lambda: f.read(8 << 20), b""):
+            h.update(chunk)
+    return h.hexdigest()
+
+
+def verify_inventory(package, manifest, *, absent=()):
+    """Check a builder-written package against its own ``files`` inventory
+    (GCR/bitexact_context_package.py:595-612): every listed path is safe and unique, exactly
+    the listed files exist, each has its pinned size and SHA-256 (the manifest pins its own
+    size only), and ``package_bytes`` is the sum of the listed sizes.
+
+    ``absent`` names inventory paths (or prefixes ending in "/") that the holder of the
+    package has dropped on purpose, such as the ``decoder/`` copies of the encoder's sources:
+    they are neither required nor allowed on disk.  Returns the number of files checked."""
+    package = Path(package)
+    files = manifest.get("files")
+    if not isinstance(files, list):
+        raise PackageError("manifest files must be a list")
+    expected = {}
+    for row in files:
+        if not isinstance(row, dict) or not isinstance(row.get("path"), str) or row["path"] in expected:
+            raise PackageError("malformed or duplicate package file inventory")
+        rel = PurePosixPath(row["path"])
+        if rel.is_absolute() or not rel.parts or ".." in rel.parts:
+            raise PackageError("unsafe package inventory path")
+        if type(row.get("bytes")) is not int or row["bytes"] < 0:
+            raise PackageError(f"invalid inventory size: {row['path']}")
+        if (row.get("sha256") is None) != (row["path"] == "manifest.json"):
+            raise PackageError("only the self-sized manifest may omit its own digest")
+        if row.get("sha256") is not None and not _is_digest(row["sha256"]):
+            raise PackageError(f"invalid inventory digest: {row['path']}")
+        expected[row["path"]] = row
+    if any(p.is_symlink() for p in package.rglob("*")):
+        raise PackageError("package must contain regular files, not symlinks")
+    dropped = lambda rel: any(rel == a or (a.endswith("/") and rel.startswith(a)) for a in absent)
+    required = {rel for rel in expected if not dropped(rel)}
+    actual = {p.relative_to(package).as_posix() for p in package.rglob("*") if p.is_file()}
+    if actual != required:
+        odd = sorted(actual ^ required)
+        raise PackageError(f"package file inventory mismatch: {odd[:4]}")
+    for rel in sorted(required):
+        row, path = expected[rel], package.joinpath(*PurePosixPath(rel).parts)
+        if path.stat().st_size != row["bytes"] or (row["sha256"] is not None and _sha_file(path) != row["sha256"]):
+            raise PackageError(f"package file integrity mismatch: {rel}")
+    if manifest.get("package_bytes") != sum(row["bytes"] for row in files):
+        raise PackageError("whole-package byte accounting mismatch")
+    return len(required)
+
+
+def _shard_layout(package, manifest, entries):
+    """Per source shard: (retained header bytes, receipts in file order), with the receipts
+    checked against the header they came from (GCR/bitexact_context_package.py:647-681)."""
+    import struct
+    headers, source = manifest.get("headers"), manifest.get("source") or {}
+    shards = source.get("shards")
+    if not isinstance(headers, dict) or not isinstance(shards, dict) or set(headers) != set(shards):
+        raise PackageError("original safetensors header coverage differs from shard set")
+    by_shard = {}
+    for row in entries.values():
+        by_shard.setdefault(row.get("source_shard"), []).append(row)
+    if set(by_shard) - set(headers):
+        raise PackageError("tensor receipt names a shard without a retained header")
+    layout = {}
+    for shard, pin in headers.items():
+        if PurePosixPath(shard).name != shard:
+            raise PackageError("unsafe source shard name")
+        raw = _inside(package, pin.get("path"), "header").read_bytes()
+        if len(raw) != pin.get("bytes") or hashlib.sha256(raw).hexdigest() != pin.get("sha256"):
+            raise PackageError(f"safetensors header identity mismatch: {shard}")
+        if len(raw) < 8 or struct.unpack("<Q", raw[:8])[0] != len(raw) - 8:
+            raise PackageError(f"original header length mismatch: {shard}")
+        described = json.loads(raw[8:], object_pairs_hook=_unique)
+        rows = sorted(by_shard.get(shard, []), key=lambda row: row["offsets"][0])
+        if set(described) - {"__metadata__"} != {row["name"] for row in rows}:
+            raise PackageError(f"header tensor set differs from receipts: {shard}")
+        at = 0
+        for row in rows:
+            d = described[row["name"]]
+            if d.get("dtype") != row["dtype"] or d.get("shape") != row["shape"] or d.get("data_offsets") != row["offsets"]:
+                raise PackageError(f"receipt differs from original header: {row['name']}")
+            if row["offsets"][0] != at or row["offsets"][1] - at != row["source_bytes"]:
+                raise PackageError(f"original shard ranges are incomplete: {shard}")
+            at = row["offsets"][1]
+        if at + len(raw) != shards[shard].get("bytes"):
+            raise PackageError(f"original shard ranges are incomplete: {shard}")
+        layout[shard] = (raw, rows)
+    return layout
+
+
+def restore(package, destination, decoder=codec.decode):
+    """Rebuild the source checkpoint of a builder-written package: every safetensors shard from
+    its retained header and the decoded frames, byte for byte (checked against the shard's
+    pinned SHA-256), and the sidecars from the metadata archive
+    (GCR/bitexact_context_package.py:699-763).  ``destination`` must be new or empty."""
+    package, destination = Path(package), Path(destination)
+    manifest, entries = read_manifest(package)
+    layout = _shard_layout(package, manifest, entries)
+    sidecars = read_metadata(package, manifest)
+    if destination.exists() and any(destination.iterdir()):
+        raise PackageError("restore destination must be new or empty")
+    destination.mkdir(parents=True, exist_ok=True)
+    for shard, (header, rows) in layout.items():
+        digest = hashlib.sha256(header)
+        with open(destination / shard, "wb") as out:
+            out.write(header)
+            for row in rows:
+                raw = decode_tensor(package, row, decoder).astype("<u2", copy=False).tobytes()
+                digest.update(raw)
+                out.write(raw)
+        if digest.hexdigest() != manifest["source"]["shards"][shard].get("sha256"):
+            raise PackageError(f"restored shard differs byte-for-byte: {shard}")
+    for name, payload in sidecars.items():
+        target = destination.joinpath(*PurePosixPath(name).parts[1:])
+        target.parent.mkdir(parents=True, exist_ok=True)
+        target.write_bytes(payload)
+    return {"tensors": len(entries), "shards": len(layout), "assets": len(sidecars)}
 
 
 # ------------------------------------------------------------------ predictive candidates
