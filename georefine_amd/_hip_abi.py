@@ -53,7 +53,7 @@ class GrfPpcxFused(ctypes.Structure):
 DEVICE_SYMBOLS = ("grf_bctx_decode", "grf_ppcx_decode", "grf_mix_predict", "grf_bctx_gemv",
                   "grf_bctx_fused_decode", "grf_bctx_fused_gather", "grf_bctx_fused_validate_host", "grf_bctx_fused_lds_bytes", "grf_bctx_gemm", "grf_bctx_gemm_lds_bytes",
                   "grf_gemm_workspace_bytes", "grf_gemm_workspace_bytes_split", "grf_bctx_gemm_noalloc", "grf_gemm_noalloc_limit_bytes", "grf_pack_activations", "grf_bctx_gemv_group", "grf_bctx_gemm_group",
-                  "grf_ppcx_bins", "grf_ppcx_bins_ordered", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_last_error",
+                  "grf_ppcx_bins", "grf_ppcx_bins_ordered", "grf_ppcx_fused_decode", "grf_ppcx_gemv", "grf_ppcx_gemm", "grf_ppcx_gemv_group", "grf_ppcx_gemm_group", "grf_last_error",
                   "grf_abi_version", "grf_timestamp", "grf_wall_clock_khz")
 
 
@@ -106,6 +106,10 @@ def declare(L):
     L.grf_ppcx_gemm.argtypes = [ctypes.POINTER(GrfPpcxFused), tiling, vp, vp, u32, u32, vp, u32, vp, vp,
                                 ctypes.c_size_t, vp, vp]
     L.grf_ppcx_gemm.restype = i
+    L.grf_ppcx_gemv_group.argtypes = [u32, vp, vp, vp, vp, u32, u32, vp, vp, vp, vp, vp]
+    L.grf_ppcx_gemv_group.restype = i
+    L.grf_ppcx_gemm_group.argtypes = [u32, vp, vp, vp, vp, u32, u32, vp, vp, vp, vp, ctypes.c_size_t, vp, vp]
+    L.grf_ppcx_gemm_group.restype = i
     L.grf_timestamp.argtypes = [vp, vp]
     L.grf_timestamp.restype = i
     L.grf_wall_clock_khz.argtypes = []

@@ -446,4 +446,118 @@ class HipPredictiveTensor:
         return out[:self.n].view(torch.bfloat16).reshape(self.shape)
 
 
+class HipPredictiveGroup:
+    """PPCX-coded matrices of one width that take the same activations, multiplied in one launch
+    (``grf_ppcx_gemv_group`` / ``grf_ppcx_gemm_group``): what ``HipLinearGroup`` is for tensors
+    of the context codec.  The members keep their context planes resident (no reference is
+    passed at call time), share one segment length and stay usable on their own; a member's
+    rows get the kernel family, and with it the bits, of its own ``linear``."""
+
+    def __init__(self, tensors, *, m_invariant=None):
+        import torch
+        self.tensors = list(tensors)
+        if not 1 <= len(self.tensors) <= 4:
+            raise ValueError("a group has 1..4 members")
+        first = self.tensors[0]
+        for t in self.tensors:
+            if t.fused is None:
+                raise codec.CodecError("frame is not eligible for the fused kernels: " + str(t.fused_reason))
+            if not t.has_contexts:
+                raise ValueError("group members keep their context planes resident (resident_contexts=True)")
+            if t.shape[1] != first.shape[1] or t.device != first.device:
+                raise ValueError("group members need one width and one device")
+        self.device, self._lib = first.device, first._lib
+        self.m_invariant = any(t.m_invariant for t in self.tensors) if m_invariant is None else bool(m_invariant)
+        self.error = torch.zeros((), device=self.device, dtype=torch.int32)
+        self._tilings, self._pointer_arrays = {}, {}
+        for key in ("waves", "gemm"):
+            self._tiling(key)  # raises FusedUnsupported when the members cannot share a tiling
+
+    def _tiling(self, key):
+        import torch
+        if key not in self._tilings:
+            plans = [t._plan for t in self.tensors]
+            hosts = (_fused.plan_group(plans, gemm=True) if key == "gemm"
+                     else _fused.plan_group(plans, m=_fused.WAVE_ROWS_PER_PASS, waves=True))
+            made = []
+            for host in hosts:
+                rows = torch.from_numpy(host["tile_rows"].view(np.int32)).to(self.device)
+                classes = torch.from_numpy(host["tile_class"]).to(self.device)
+                g = _hip_abi.GrfFusedTiling()
+                g.tile_rows, g.tile_class = rows.data_ptr(), classes.data_ptr()
+                for name, value in host["scalars"].items():
+                    setattr(g, name, value)
+                made.append((g, rows, classes, dict(host["scalars"], lds=host["lds"])))
+            self._tilings[key] = made
+        return self._tilings[key]
+
+    def _arrays(self, key, outs, biases):
+        n = len(self.tensors)
+        if key not in self._pointer_arrays:  # frames, tilings and planes do not change between calls
+            self._pointer_arrays[key] = (
+                (ctypes.POINTER(_hip_abi.GrfPpcxFused) * n)(*[ctypes.pointer(t.fused) for t in self.tensors]),
+                (ctypes.POINTER(_hip_abi.GrfFusedTiling) * n)(*[ctypes.pointer(g[0]) for g in self._tiling(key)]),
+                (ctypes.c_void_p * n)(*[t.buffers["context_bins"].data_ptr() for t in self.tensors]))
+        frames, tiles, bins = self._pointer_arrays[key]
+        ys = (ctypes.c_void_p * n)(*[y.data_ptr() for y in outs])
+        ldy = (ctypes.c_uint32 * n)(*[y.stride(0) for y in outs])
+        bias = (ctypes.c_void_p * n)(*[b.data_ptr() if b is not None else None for b in biases])
+        return frames, tiles, bins, ys, ldy, bias
+
+    def linear(self, x, biases=None, *, check=False, batch_invariant=None):
+        """[x @ W.T (+ bias) for every member]; x is BF16 [..., K] or ``PackedActivations``.
+        One activation row goes to the vector-ALU kernel, up to 128 to the matrix cores (every
+        row count under ``batch_invariant``), more than that to the members' own ``linear``."""
+        import torch
+        from .bitexact_context_gpu import PackedActivations
+        n = len(self.tensors)
+        biases = list(biases) if biases is not None else [None] * n
+        if len(biases) != n:
+            raise ValueError("one bias (or None) per member")
+        packed = x if isinstance(x, PackedActivations) else None
+        m = packed.rows if packed else math.prod(x.shape[:-1])
+        lead = packed.lead if packed else tuple(x.shape[:-1])
+        cols = self.tensors[0].shape[1]
+        if batch_invariant is None:
+            batch_invariant = self.m_invariant
+        first = self.tensors[0]
+        if packed is None and m > first.DENSE_ABOVE and not batch_invariant:
+            return [t.linear(None, x, b, check=check, batch_invariant=False) for t, b in zip(self.tensors, biases)]
+        use_gemm = packed is not None or batch_invariant or m > first.GEMV_UP_TO
+        if packed is not None:
+            if packed.cols != cols or packed.buffer.device != self.device:
+                raise ValueError("packed activations of another width or device")
+            x2 = None
+        else:
+            if x.dtype != torch.bfloat16 or x.shape[-1] != cols:
+                raise ValueError("activation must be bfloat16 with the weights' input width")
+            x2 = x.reshape(-1, cols).to(self.device)
+            if x2.stride(-1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+                x2 = x2.clone(memory_format=torch.contiguous_format)
+        biases = [b.to(device=self.device, dtype=torch.bfloat16).contiguous() if b is not None else None for b in biases]
+        outs = [torch.empty((m, t.shape[0]), device=self.device, dtype=torch.bfloat16) for t in self.tensors]
+        if m:
+            if check:
+                self.error.zero_()
+            with torch.cuda.device(self.device):
+                stream = torch.cuda.current_stream(self.device).cuda_stream
+                xp, ldx = (x2.data_ptr(), x2.stride(0)) if x2 is not None else (None, 0)
+                if use_gemm:
+                    a = self._arrays("gemm", outs, biases)
+                    space = packed.buffer if packed else torch.empty(
+                        self._lib.grf_gemm_workspace_bytes(cols, m), device=self.device, dtype=torch.uint8)
+                    status = self._lib.grf_ppcx_gemm_group(n, a[0], a[1], a[2], xp, ldx, m, a[3], a[4], a[5],
+                                                           space.data_ptr(), space.numel(), self.error.data_ptr(), stream)
+                else:
+                    a = self._arrays("waves", outs, biases)
+                    status = self._lib.grf_ppcx_gemv_group(n, a[0], a[1], a[2], xp, ldx, m, a[3], a[4], a[5],
+                                                           self.error.data_ptr(), stream)
+            if status:
+                raise codec.CodecError(f"device launch failed ({status}): "
+                                       + self._lib.grf_last_error().decode(errors="replace"))
+            if check and self.error.item() != 0:
+                raise codec.CodecError("HIP PPCX checkpoint/context mismatch")
+        return [y.reshape(*lead, t.shape[0]) for y, t in zip(outs, self.tensors)]
+
+
 CudaPredictiveTensor = HipPredictiveTensor

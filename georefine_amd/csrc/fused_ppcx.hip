@@ -306,4 +306,52 @@ int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, c
                                     workspace_bytes, error, (hipStream_t)hip_stream);
 }
 
+
+}  // extern "C"
+
+namespace {
+
+// The members of a grouped PPCX launch in the walker's frame structure.
+struct PpcxMembers {
+  grf_bctx_fused frames[grf::kMaxGroup];
+  const grf_bctx_fused *pointers[grf::kMaxGroup];
+  int fill(const char *who, uint32_t n, const grf_ppcx_fused *const *members, const grf_fused_tiling *const *tilings,
+           const uint32_t *const *bins, grf::TilingUse use) {
+    if (n < 1 || n > grf::kMaxGroup) return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": a group has 1..4 members");
+    if (!members || !tilings || !bins) return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": null argument");
+    for (uint32_t i = 0; i < n; ++i) {
+      if (int rc = walker_frame(members[i], tilings[i], bins[i], who, frames[i], use)) return rc;
+      pointers[i] = &frames[i];
+    }
+    return GRF_OK;
+  }
+};
+
+}  // namespace
+
+extern "C" {
+
+int grf_ppcx_gemv_group(uint32_t n, const grf_ppcx_fused *const *frames, const grf_fused_tiling *const *tilings,
+                        const uint32_t *const *bins, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
+                        uint16_t *const *y, const uint32_t *ldy, const uint16_t *const *bias, int32_t *error,
+                        void *hip_stream) {
+  if (!error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemv_group: null argument");
+  PpcxMembers members;
+  if (int rc = members.fill("grf_ppcx_gemv_group", n, frames, tilings, bins, grf::kGemvTiling)) return rc;
+  const grf::GroupSpec spec{n, members.pointers, tilings, y, ldy, bias};
+  return grf::launch_gemv_group<PpcxWalk>("grf_ppcx_gemv_group", spec, x, ldx, m_rows, error, (hipStream_t)hip_stream);
+}
+
+int grf_ppcx_gemm_group(uint32_t n, const grf_ppcx_fused *const *frames, const grf_fused_tiling *const *tilings,
+                        const uint32_t *const *bins, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
+                        uint16_t *const *y, const uint32_t *ldy, const uint16_t *const *bias, void *workspace,
+                        size_t workspace_bytes, int32_t *error, void *hip_stream) {
+  if (!error) return grf::set_error(GRF_BAD_ARGUMENT, "grf_ppcx_gemm_group: null argument");
+  PpcxMembers members;
+  if (int rc = members.fill("grf_ppcx_gemm_group", n, frames, tilings, bins, grf::kGemmTiling)) return rc;
+  const grf::GroupSpec spec{n, members.pointers, tilings, y, ldy, bias};
+  return grf::launch_gemm_group<PpcxWalk>("grf_ppcx_gemm_group", spec, x, ldx, m_rows, workspace, workspace_bytes,
+                                          error, (hipStream_t)hip_stream);
+}
+
 }  // extern "C"

@@ -32,10 +32,12 @@ def hip_tensor_factory(frame, *, stride=1024, device="cuda:0", fused_segment=Non
                             residual_block=residual_block)
 
 
-def hip_predictive_factory(frame, reference_uint16_numpy, stride=1024, device="cuda:0"):
-    """The ``predictive_factory`` of ``load_predictive_model`` (GCR/bitexact_predictive_serving.py:918-924)."""
+def hip_predictive_factory(frame, reference_uint16_numpy, stride=1024, device="cuda:0", *, fused_segment=None):
+    """The ``predictive_factory`` of ``load_predictive_model`` (GCR/bitexact_predictive_serving.py:918-924).
+    ``fused_segment``: the tile walker's segment length, given by the loader to siblings that
+    are to share launches (they need one length)."""
     from .bitexact_predictive_gpu import HipPredictiveTensor
-    return HipPredictiveTensor(frame, reference_uint16_numpy, stride=stride, device=device)
+    return HipPredictiveTensor(frame, reference_uint16_numpy, stride=stride, device=device, fused_segment=fused_segment)
 
 
 class SharedProducts:
@@ -246,6 +248,22 @@ class PredictiveContextTensor:
                          batch_invariant=batch_invariant)
 
 
+def _launch_group(weights):
+    """One grouped launch for sibling weights, or None when they do not all take the same
+    walker: tensors of the context codec (a predictive weight re-framed at load counts as its
+    row-major tensor) share ``HipLinearGroup``; predictive weights stored untransposed whose
+    native tensors keep their context planes share ``HipPredictiveGroup``."""
+    from .bitexact_context_gpu import HipContextTensor, HipLinearGroup
+    effective = [getattr(w, "row_major", None) or w for w in weights]
+    if all(isinstance(w, HipContextTensor) for w in effective):
+        return HipLinearGroup(effective)
+    from .bitexact_predictive_gpu import HipPredictiveGroup, HipPredictiveTensor
+    if all(isinstance(w, PredictiveContextTensor) and w.transform != "target transpose"
+           and isinstance(w.native, HipPredictiveTensor) and not w._needs_reference() for w in effective):
+        return HipPredictiveGroup([w.native for w in effective])
+    return None
+
+
 # ----------------------------------------------------------------------------- loader
 
 def _parent_and_attr(model, dotted):
@@ -414,8 +432,14 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         takes_segment = "fused_segment" in inspect.signature(tensor_factory).parameters
     except (TypeError, ValueError):
         takes_segment = False
+    try:
+        predictive_takes_segment = "fused_segment" in inspect.signature(predictive_factory).parameters
+    except (TypeError, ValueError):
+        predictive_takes_segment = False
+    # (predictive candidates too: siblings that are all coded against references, or all re-framed
+    # at load, share launches like plain frames; mixed groups keep separate launches)
     coded_linears = {module_name: (module, weight_name) for module_name, module, weight_name in coded
-                     if isinstance(module, nn.Linear) and weight_name not in selected}
+                     if isinstance(module, nn.Linear)}
     sibling_groups, shared_segment = [], {}
     for names in share_launches or ():
         names = tuple(names)
@@ -429,7 +453,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
             if all(m in coded_linears for m in members) and \
                     len({coded_linears[m][0].in_features for m in members}) == 1:
                 sibling_groups.append(members)
-                if takes_segment:
+                if takes_segment or predictive_takes_segment:
                     from . import _fused
                     cols = coded_linears[members[0]][0].in_features
                     try:
@@ -517,7 +541,8 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         if name not in selected:
             continue
         c, row = selected[name], entries[name]
-        native = predictive_factory(candidate_frame(name), reference_words(name), stride=stride, device=device)
+        extra = {"fused_segment": shared_segment[name]} if name in shared_segment and predictive_takes_segment else {}
+        native = predictive_factory(candidate_frame(name), reference_words(name), stride=stride, device=device, **extra)
         geometry = pkg.frame_shape(row["shape"])
         if c["transform"] == "target transpose":
             geometry = geometry[::-1]
@@ -586,11 +611,10 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
     for members in sibling_groups:
         modules = [replacements[m] for m in members]
         try:
-            from .bitexact_context_gpu import HipContextTensor, HipLinearGroup
-            if not all(isinstance(m.context_weight, HipContextTensor) for m in modules):
+            group = _launch_group([m.context_weight for m in modules])
+            if group is None:
                 continue
-            products = SharedProducts(HipLinearGroup([m.context_weight for m in modules]), [m.bias for m in modules],
-                                      batch_invariant=batch_invariant)
+            products = SharedProducts(group, [m.bias for m in modules], batch_invariant=batch_invariant)
         except Exception as exc:  # the members stay separate launches
             log(f"[bctx] {members} keep separate launches: {exc}")
             continue

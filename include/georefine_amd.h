@@ -435,6 +435,20 @@ int grf_ppcx_gemm(const grf_ppcx_fused *frame, const grf_fused_tiling *tiling, c
                   uint32_t ldx, uint32_t m_rows, uint16_t *y, uint32_t ldy, const uint16_t *bias, void *workspace,
                   size_t workspace_bytes, int32_t *error, void *hip_stream);
 
+/* Up to four prepared PPCX frames of one width that take the same activations in one launch,
+ * as grf_bctx_gemv_group / grf_bctx_gemm_group do for BCTX frames (same grid of the members'
+ * tiles, same restrictions on the tilings, a member's rows bit-equal to grf_ppcx_gemv /
+ * grf_ppcx_gemm with that tiling); bins[i] is the bins plane of member i's reference.  The
+ * reference multiplies every such weight on its own (GCR/bitexact_predictive_serving.py:490-523). */
+int grf_ppcx_gemv_group(uint32_t n, const grf_ppcx_fused *const *frames, const grf_fused_tiling *const *tilings,
+                        const uint32_t *const *bins, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
+                        uint16_t *const *y, const uint32_t *ldy, const uint16_t *const *bias, int32_t *error,
+                        void *hip_stream);
+int grf_ppcx_gemm_group(uint32_t n, const grf_ppcx_fused *const *frames, const grf_fused_tiling *const *tilings,
+                        const uint32_t *const *bins, const uint16_t *x, uint32_t ldx, uint32_t m_rows,
+                        uint16_t *const *y, const uint32_t *ldy, const uint16_t *const *bias, void *workspace,
+                        size_t workspace_bytes, int32_t *error, void *hip_stream);
+
 /* A one-lane kernel that writes slot[0] = the device's constant-rate counter
  * (grf_wall_clock_khz), slot[1] = its shader-clock counter and slot[2] = the identifier of the
  * compute unit it ran on, all read when the kernel runs, i.e. in stream order after the work

@@ -89,3 +89,56 @@ def test_group_reports_a_member_that_misses_its_checkpoints_and_rejects_mismatch
         HipLinearGroup([tensors[0], coarse[0]])
     with pytest.raises(ValueError):
         HipLinearGroup([])
+
+
+def test_predictive_group_products():
+    """PPCX members of one width in one launch: one row gives each member the bits of its own
+    vector-ALU launch; the matrix-core rows agree with the dense product of the decoded target
+    within 1e-2 and do not depend on the batch; a member that misses its checkpoints is
+    reported."""
+    import torch
+    from georefine_amd import bitexact_predictive_codec as ppcx
+    from georefine_amd.bitexact_context_gpu import PackedActivations
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveGroup, HipPredictiveTensor
+    rng = np.random.default_rng(77)
+    cols, members, targets = 1280, [], []
+    for rows in (200, 72, 330):
+        target = weight_like(rng, rows, cols)
+        tf = (target.astype(np.uint32) << 16).view(np.float32)
+        ref = bf16_words(tf + rng.normal(0, 0.003, target.shape).astype(np.float32))
+        t = HipPredictiveTensor(ppcx.encode(target, ref), ref, stride=1024, device="cuda:0", fused_segment=64)
+        assert t.fused is not None and t.has_contexts, t.fused_reason
+        members.append(t)
+        targets.append(torch.from_numpy(target).view(torch.bfloat16).cuda().float())
+    group = HipPredictiveGroup(members)
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(140, cols)))).view(torch.bfloat16).cuda()
+    biases = [torch.from_numpy(bf16_words(rng.normal(0, 1, size=200))).view(torch.bfloat16).cuda(), None, None]
+
+    def close(y, i, rows):
+        b = biases[i].float() if biases[i] is not None else None
+        want = torch.nn.functional.linear(x[:rows].float(), targets[i], b)
+        scale = torch.nn.functional.linear(x[:rows].float().abs(), targets[i].abs(), b.abs() if b is not None else None)
+        return bool((y.float() - want).abs().le(1e-2 * want.abs().clamp_min(1e-3 * scale) + 1e-30).all())
+
+    ys = group.linear(x[:1], biases, check=True)
+    for i, (y, t) in enumerate(zip(ys, members)):
+        assert y.shape == (1, t.shape[0])
+        assert torch.equal(y.view(torch.uint16), t.gemv(None, x[:1], biases[i]).view(torch.uint16)), i
+    full = group.linear(x[:128], biases, check=True, batch_invariant=True)
+    for i, y in enumerate(full):
+        assert close(y, i, 128), i
+    for rows in (1, 3, 17, 64, 100):
+        for y, f in zip(group.linear(x[:rows], biases, batch_invariant=True), full):
+            assert torch.equal(y.view(torch.uint16), f[:rows].view(torch.uint16)), rows
+    for y, f in zip(group.linear(x[:40], biases), full):  # the default route at 40 rows is the same kernel
+        assert torch.equal(y.view(torch.uint16), f[:40].view(torch.uint16))
+    for y, f in zip(group.linear(PackedActivations(x[:40]), biases), full):
+        assert torch.equal(y.view(torch.uint16), f[:40].view(torch.uint16))
+    for i, y in enumerate(group.linear(x, biases, check=True)):  # above 128 rows: the members' own route
+        assert close(y, i, 140), i
+    assert group.linear(x[:0], biases)[1].shape == (0, 72)
+    members[1].buffers["fused_seg_state"].view(torch.int32)[3] += 1  # forced from the host; kernels finish normally
+    with pytest.raises(ppcx.CodecError):
+        group.linear(x[:1], biases, check=True)
+    with pytest.raises(ppcx.CodecError):
+        group.linear(x[:5], biases, check=True)

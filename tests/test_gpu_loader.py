@@ -211,3 +211,55 @@ def test_sibling_projections_share_a_launch(tmp_path):
             assert row["fused"] == (row["frame_mode"] != 1) and row["residual_repacked"] == (row["frame_mode"] == 128)
     assert receipt["transcoded"] == bool(receipt["residual_repacked_tensors"])
     assert serving.decode_errors(shared) == [] and serving.decode_errors(plain) == []
+
+
+def test_predictive_siblings_share_a_launch(tmp_path):
+    """gate and up of a block both coded against another tensor (PPCX, stored untransposed):
+    with share_launches they run as one grouped launch of the predictive walker, and one row
+    gives the bits of the same model loaded without sharing."""
+    import torch
+    from torch import nn
+    from conftest import words_to_float
+    from georefine_amd import bitexact_context_package as pkg
+    from georefine_amd import serving
+    from georefine_amd.bitexact_predictive_gpu import HipPredictiveGroup
+
+    class Gated(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.base = nn.Linear(256, 384, bias=False)
+            self.gate = nn.Linear(256, 384, bias=False)
+            self.up = nn.Linear(256, 384, bias=True)
+            self.down = nn.Linear(384, 256, bias=False)
+
+        def forward(self, x):
+            return self.down(torch.nn.functional.silu(self.gate(x)) * self.up(x) + self.base(x))
+
+    rng = np.random.default_rng(31)
+    base = weight_like(rng, 384, 256)
+    near = lambda: bf16_words(words_to_float(base) + rng.normal(0, 2e-4, (384, 256)))
+    tensors = {"base.weight": base, "gate.weight": near(), "up.weight": near(),
+               "up.bias": bf16_words(rng.normal(0, 0.1, size=384)), "down.weight": weight_like(rng, 256, 384)}
+    path = tmp_path / "package"
+    pkg.write_package(path, tensors)
+    for name in ("gate.weight", "up.weight"):
+        pkg.add_candidate(path, name, references=["base.weight"])
+    shared, receipt = serving.load_bctx_model(path, model_factory=Gated, device="cuda:0", log=lambda _: None,
+                                              share_launches=[("gate", "up")])
+    plain, _ = serving.load_bctx_model(path, model_factory=Gated, device="cuda:0", log=lambda _: None)
+    assert receipt["shared_launches"] == [["gate.weight", "up.weight"]]
+    products = shared.gate.shared[0]
+    assert products is shared.up.shared[0] and isinstance(products.group, HipPredictiveGroup)
+    dense = Gated().to(torch.bfloat16).cuda()
+    with torch.no_grad():
+        for name, words in tensors.items():
+            dict(dense.named_parameters())[name].copy_(torch.from_numpy(words).view(torch.bfloat16).cuda())
+    for rows in (1, 6, 70):
+        x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(rows, 256)))).view(torch.bfloat16).cuda()
+        with torch.no_grad():
+            got, want = shared(x), dense(x)
+        assert float((got.float() - want.float()).abs().max()) <= 3e-2 * float(want.float().abs().max())
+        if rows == 1:
+            assert torch.equal(got.view(torch.uint16), plain(x).view(torch.uint16))
+    assert products.launches == 3 and shared.gate.weight_materializations == 0
+    assert serving.decode_errors(shared) == []
