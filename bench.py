@@ -16,7 +16,8 @@ CPU baseline (the CPU oracle's decode + matvec on the host cores).
 The K timed steps are replays of HIP graphs of consecutive steps (--no-graph times eager
 steps instead); the per-launch durations come from device timestamps inside a graph of the
 same steps.  The default run adds the other configurations of the metric to the same line:
-`batch64` (the MLP step at batch 64, fused GEMM), `attention` (q/k/v/o at batch 1..128 through
+`m_invariant_policy` (the down projection at 1 and 6 rows under the batch-invariant route, beside
+the default route), `batch64` (the MLP step at batch 64, fused GEMM), `attention` (q/k/v/o at batch 1..128 through
 the batch-invariant GEMM), `ppcx` (a predictive frame, products with 1 and 96 rows) and `stack`
 (every coded linear of a 64-layer model resident at once, one pass at batch 64).
 """
@@ -694,6 +695,8 @@ def main():
                                                          "some milliseconds of work to come up)")
     ap.add_argument("--batch", type=int, default=None, help="activation rows (default 1 for mlp, the headline figure, and 64 for stack); 1..2 run the fused GEMV, more the fused GEMM")
     ap.add_argument("--segment", type=int, default=0, help="fused segment length (0 = automatic)")
+    ap.add_argument("--residual-block", type=int, default=0,
+                    help="mlp: rows per block of the resident residual order (0 = by batch: 16 above 2 rows, else the GEMV unit's)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", dest="graph", action="store_false",
                     help="time K eager steps; by default the K timed steps are replays of one captured HIP graph "
@@ -757,6 +760,9 @@ def main():
     names = [s for s in args.only.split(",") if s] or list(SHAPES)
     tensors, frames, words_of = {}, {}, {}
     t_setup = time.perf_counter()
+    # matrices that are served in batches keep their packed residuals in blocks of sixteen rows,
+    # the matrix-core kernel's unit; the others in blocks of the vector-ALU kernel's unit
+    residual_block = args.residual_block or (16 if args.batch > GEMV_UP_TO else None)
     for i, name in enumerate(SHAPES):
         if name not in names:
             continue
@@ -765,8 +771,8 @@ def main():
         t0 = time.perf_counter()
         frame = codec.encode(w)
         t1 = time.perf_counter()
-        tensors[name] = HipContextTensor(frame, stride=1024, device="cuda:0",
-                                         fused_segment=args.segment or None)
+        tensors[name] = HipContextTensor(frame, stride=1024, device="cuda:0", fused_segment=args.segment or None,
+                                         residual_block=residual_block)
         t2 = time.perf_counter()
         if tensors[name].fused is None:
             sys.exit(f"bench.py: {name} is not eligible for the fused kernel: {tensors[name].fused_reason}")
@@ -886,6 +892,21 @@ def main():
         # the other figures of the metric, timed in the same run: the MLP step at batch 64 (fused
         # GEMM on the matrix cores), the attention projections through the batch-invariant GEMM,
         # a predictive frame, and one pass through a whole resident stack
+        # what the M-invariant policy (HipContextTensor(..., m_invariant=True), the MTP head's and
+        # BctxLinear(batch_invariant=True)'s route: every row count through the matrix-core kernel,
+        # so a row's bits do not depend on the batch) costs on the down projection at 1 and 6 rows,
+        # beside the default route (1 row: the vector-ALU kernel; 6 rows: the same matrix-core kernel)
+        log("M-invariant policy on down ...")
+        rng6 = np.random.default_rng(11)
+        x6 = torch.from_numpy(bf16_words(rng6.normal(0, 1, size=(6, SHAPES["down"][1])))).view(torch.bfloat16).cuda()
+        policy = {"matrix": "down %dx%d" % SHAPES["down"], "m1_default_ms": result["per_kernel"]["down"]["ms"]}
+        for key, rows_, inv in (("m1_invariant_ms", 1, True), ("m6_default_ms", 6, False), ("m6_invariant_ms", 6, True)):
+            per_layer = [[("down", ["down"], lambda t=ts["down"], r=rows_, i=inv: t.linear(x6[:r], batch_invariant=i))]
+                         for ts, _ in layers]
+            _, per, _, _, _ = time_launches(torch, per_layer, min(args.steps, 40), min(args.warmup, 10), args.graph,
+                                            lambda: sorted({"down" for ts, _ in layers if ts["down"].error.item()}))
+            policy[key] = round(per["down"], 4)
+        result["m_invariant_policy"] = policy
         log("batch 64 ...")
         # matrices that are served in batches keep their packed residuals in blocks of sixteen rows
         # (a load-time choice: HipContextTensor(..., residual_block=16)); here the copies are
