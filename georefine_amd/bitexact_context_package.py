@@ -19,7 +19,11 @@ Predictive candidates.  A manifest may carry ``selected_candidates``: tensors wh
 a PPCX frame coded against one other tensor of the package (``mode`` "single") or against
 the row-wise mix of two (``"mixbf16"``, with a ``[rows, 3]`` BF16 coefficient file), possibly
 stored transposed.  The fields and their checks follow the reference's predictive package
-(GCR/bitexact_predictive_package.py:433-537; coefficient files :59-86).
+(GCR/bitexact_predictive_package.py:433-537; coefficient files :59-86).  That builder's own
+packages (schema ``bitexact-predictive-context-package-v1``) keep the tensor receipts in the
+manifest of the context package they were made from, stored compressed beside the manifest and
+pinned by size and digest; ``read_manifest`` reads both layouts and returns the receipts either
+way, ``TensorResolver`` decodes any tensor on the host through its candidate and references.
 """
 from __future__ import annotations
 
@@ -34,6 +38,11 @@ import numpy as np
 from . import bitexact_context_codec as codec
 
 SCHEMA = "bitexact-context-package-v1"
+# A predictive package (GCR/bitexact_predictive_package.py:11-13): a context package in which the
+# frames of some tensors are replaced by PPCX frames (``selected_candidates``); the context
+# package's manifest, with every tensor's receipt, is kept beside it, compressed and pinned.
+PREDICTIVE_SCHEMA = "bitexact-predictive-context-package-v1"
+CANDIDATE_SCHEMA = "ppcx-reference-conditioned-bf16-v1"
 
 
 class PackageError(ValueError):
@@ -77,8 +86,11 @@ def read_manifest(package):
         manifest = json.loads(path.read_text(encoding="utf-8"), object_pairs_hook=_unique)
     except (OSError, json.JSONDecodeError) as exc:
         raise PackageError(f"cannot read BCTX manifest: {exc}") from exc
-    if not isinstance(manifest, dict) or manifest.get("schema") != SCHEMA or manifest.get("complete") is not True:
+    if (not isinstance(manifest, dict) or manifest.get("schema") not in (SCHEMA, PREDICTIVE_SCHEMA)
+            or manifest.get("complete") is not True):
         raise PackageError("unsupported or incomplete BCTX package manifest")
+    if manifest["schema"] == PREDICTIVE_SCHEMA:
+        manifest = dict(manifest, tensors=_parent_receipts(package, manifest))
     rows = manifest.get("tensors")
     if not isinstance(rows, list):
         raise PackageError("manifest tensors must be a list")
@@ -105,6 +117,74 @@ def read_manifest(package):
     return manifest, entries
 
 
+def _parent_receipts(package, manifest):
+    """The tensor receipts of a predictive package: they live in the manifest of the context
+    package it was made from, stored as ``baseline-manifest.json.xz`` (or plain, in older
+    packages) and pinned by size and SHA-256 (GCR/bitexact_predictive_package.py:47-57,
+    446-450).  ``verify_on_load`` must be set, as the reference's reader demands of this schema."""
+    import lzma
+    package = Path(package)
+    if manifest.get("verify_on_load") is not True:
+        raise PackageError("predictive package lacks stable verification metadata")
+    plain, packed = package / "baseline-manifest.json", package / "baseline-manifest.json.xz"
+    if plain.is_file() == packed.is_file():
+        raise PackageError("baseline tensor manifest missing or ambiguous")
+    try:
+        raw = plain.read_bytes() if plain.is_file() else lzma.decompress(packed.read_bytes())
+    except (OSError, lzma.LZMAError) as exc:
+        raise PackageError("baseline manifest is unreadable or corrupt") from exc
+    if hashlib.sha256(raw).hexdigest() != manifest.get("baseline_manifest_sha256"):
+        raise PackageError("baseline manifest checksum mismatch")
+    if manifest.get("baseline_manifest_bytes") is not None and manifest["baseline_manifest_bytes"] != len(raw):
+        raise PackageError("baseline manifest byte count mismatch")
+    try:
+        parent = json.loads(raw, object_pairs_hook=_unique)
+    except json.JSONDecodeError as exc:
+        raise PackageError("baseline manifest is not JSON") from exc
+    if not isinstance(parent, dict) or parent.get("schema") != SCHEMA or parent.get("complete") is not True:
+        raise PackageError("baseline manifest is not a complete context-package manifest")
+    return parent.get("tensors")
+
+
+def verify_receipt_archive(package, manifest):
+    """The archive of the parent package's per-tensor receipts that a predictive package keeps
+    (``baseline_receipts``: path, size, SHA-256 and the same per member;
+    GCR/bitexact_predictive_package.py:236-249).  Returns the number of members (0: the package
+    pins none)."""
+    import io
+    import lzma
+    import tarfile
+    pin = manifest.get("baseline_receipts")
+    if pin is None:
+        return 0
+    if not isinstance(pin, dict) or not isinstance(pin.get("members"), list):
+        raise PackageError("baseline receipt archive pin is malformed")
+    raw = _inside(package, pin.get("path"), "receipt archive").read_bytes()
+    if len(raw) != pin.get("bytes") or hashlib.sha256(raw).hexdigest() != pin.get("sha256"):
+        raise PackageError("baseline receipt archive checksum mismatch")
+    want = {row.get("path"): row for row in pin["members"] if isinstance(row, dict)}
+    if len(want) != len(pin["members"]):
+        raise PackageError("duplicate baseline receipt member metadata")
+    seen = set()
+    try:
+        with tarfile.open(fileobj=io.BytesIO(raw), mode="r:xz") as tf:
+            for member in tf.getmembers():
+                rel = PurePosixPath(member.name)
+                name = rel.as_posix()
+                if (not member.isfile() or rel.is_absolute() or ".." in rel.parts or not name.startswith("receipts/")
+                        or name in seen or name not in want):
+                    raise PackageError("unsafe or unexpected baseline receipt member")
+                payload = tf.extractfile(member).read()
+                if len(payload) != want[name].get("bytes") or hashlib.sha256(payload).hexdigest() != want[name].get("sha256"):
+                    raise PackageError("baseline receipt raw content mismatch")
+                seen.add(name)
+    except (tarfile.TarError, lzma.LZMAError) as exc:
+        raise PackageError("invalid xz receipt archive") from exc
+    if seen != set(want):
+        raise PackageError("baseline receipt archive is incomplete")
+    return len(seen)
+
+
 def read_frame(package, row):
     """The frame bytes of one receipt, checked against the pinned size and digest."""
     name = row["name"]
@@ -127,16 +207,72 @@ def decode_tensor(package, row, decoder=codec.decode):
     return words.reshape(row["shape"])
 
 
+class TensorResolver:
+    """Host decode of any tensor of a package, through its predictive candidate where it has
+    one: the candidate's references are decoded first (recursively), two of them mixed with the
+    stored coefficients, the PPCX frame decoded against the result and turned back if it was
+    stored transposed; every step is checked against its digest
+    (GCR/bitexact_predictive_package.py:497-522).  Decoded tensors are kept while they may still
+    be needed as references."""
+
+    def __init__(self, package, manifest=None, entries=None, decoder=codec.decode):
+        if manifest is None:
+            manifest, entries = read_manifest(package)
+        self.package, self.manifest, self.entries, self.decoder = Path(package), manifest, entries, decoder
+        self.selected = read_candidates(package, manifest, entries)
+        self._needed = {ref["name"] for c in self.selected.values() for ref in c["references"]}
+        self._kept = {}
+
+    def words(self, name):
+        """BF16 words of ``name`` in its own shape."""
+        if name in self._kept:
+            return self._kept[name]
+        row = self.entries[name]
+        c = self.selected.get(name)
+        if c is None:
+            out = decode_tensor(self.package, row, self.decoder)
+        else:
+            from . import bitexact_predictive_codec as ppcx
+            refs = [self.words(ref["name"]) for ref in c["references"]]
+            refs = [r.reshape(frame_shape(self.entries[ref["name"]]["shape"])) for r, ref in zip(refs, c["references"])]
+            reference = refs[0]
+            if c["mode"] == "mixbf16":
+                from . import bitexact_predictive_mix as mix
+                reference = np.ascontiguousarray(mix.predict(refs[0], refs[1], read_coefficients(self.package, c)))
+                if hashlib.sha256(reference.astype("<u2", copy=False).tobytes()).hexdigest() != c["derived_reference_sha256"]:
+                    raise PackageError(f"derived reference checksum mismatch: {name}")
+            decoded = np.ascontiguousarray(ppcx.decode(read_candidate_frame(self.package, c), reference))
+            if c["transform"] == "target transpose":
+                decoded = np.ascontiguousarray(decoded.T)
+            if (decoded.dtype != np.uint16 or decoded.size * 2 != row["source_bytes"]
+                    or hashlib.sha256(decoded.astype("<u2", copy=False).tobytes()).hexdigest() != row["source_sha256"]):
+                raise PackageError(f"tensor decode/source SHA mismatch: {name}")
+            out = decoded.reshape(row["shape"])
+        if name in self._needed:
+            self._kept[name] = out
+        return out
+
+    def coded_bytes(self, name):
+        """Bytes the package holds for ``name``: its frame, or its candidate's frame and coefficients."""
+        c = self.selected.get(name)
+        if c is None:
+            return self.entries[name]["frame_bytes"]
+        return c["frame_bytes"] + (c["coefficients"]["bytes"] if c["mode"] == "mixbf16" else 0)
+
+
 def verify(package, decoder=codec.decode):
-    """Decode every frame on the host and check every pin; returns totals."""
+    """Decode every tensor on the host -- predictive candidates through their references -- and
+    check every pin; returns totals."""
     manifest, entries = read_manifest(package)
+    resolver = TensorResolver(package, manifest, entries, decoder)
     source = coded = 0
-    for row in entries.values():
-        decode_tensor(package, row, decoder)
+    for name, row in entries.items():
+        resolver.words(name)
         source += row["source_bytes"]
-        coded += row["frame_bytes"]
+        coded += resolver.coded_bytes(name)
     sidecars = read_metadata(package, manifest) if ("metadata_assets" in manifest or "files" in manifest) else {}
-    return {"tensors": len(entries), "source_bytes": source, "frame_bytes": coded, "metadata_assets": len(sidecars)}
+    return {"tensors": len(entries), "source_bytes": source, "frame_bytes": coded, "metadata_assets": len(sidecars),
+            "predictive_candidates": len(resolver.selected), "receipt_members": verify_receipt_archive(package, manifest)}
 
 
 def _words(tensor):
@@ -388,6 +524,7 @@ def restore(package, destination, decoder=codec.decode):
     manifest, entries = read_manifest(package)
     layout = _shard_layout(package, manifest, entries)
     sidecars = read_metadata(package, manifest)
+    resolver = TensorResolver(package, manifest, entries, decoder)
     if destination.exists() and any(destination.iterdir()):
         raise PackageError("restore destination must be new or empty")
     destination.mkdir(parents=True, exist_ok=True)
@@ -396,7 +533,7 @@ def restore(package, destination, decoder=codec.decode):
         with open(destination / shard, "wb") as out:
             out.write(header)
             for row in rows:
-                raw = decode_tensor(package, row, decoder).astype("<u2", copy=False).tobytes()
+                raw = resolver.words(row["name"]).astype("<u2", copy=False).tobytes()
                 digest.update(raw)
                 out.write(raw)
         if digest.hexdigest() != manifest["source"]["shards"][shard].get("sha256"):
@@ -429,7 +566,7 @@ def read_candidates(package, manifest, entries):
     frames = set()
     for name, c in selected.items():
         row = entries.get(name)
-        if row is None or not isinstance(c, dict) or c.get("name") != name:
+        if row is None or not isinstance(c, dict) or c.get("name") != name or c.get("schema") != CANDIDATE_SCHEMA:
             raise PackageError(f"candidate schema/name mismatch: {name}")
         refs = c.get("references")
         wanted = {"single": 1, "mixbf16": 2}.get(c.get("mode"))
@@ -523,7 +660,8 @@ def add_candidate(package, name, *, references, transform="identity", coefficien
     target = decode_tensor(package, row).reshape(frame_shape(row["shape"]))
     if transform == "target transpose":
         target = np.ascontiguousarray(target.T)
-    candidate = {"name": name, "mode": "single" if len(references) == 1 else "mixbf16", "transform": transform,
+    candidate = {"schema": CANDIDATE_SCHEMA, "name": name, "mode": "single" if len(references) == 1 else "mixbf16",
+                 "transform": transform,
                  "references": [{"name": r, "sha256": entries[r]["source_sha256"]} for r in references],
                  "shape": row["shape"], "source_sha256": row["source_sha256"], "source_bytes": row["source_bytes"]}
     reference = words[0]

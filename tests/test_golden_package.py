@@ -163,3 +163,143 @@ def test_loader_serves_the_builders_package_on_the_device():
     rows = model.emb(torch.tensor([7, 95], device="cuda")).view(torch.uint16).cpu().numpy()
     assert np.array_equal(rows, source["emb.weight"][[7, 95]])
     assert model.up.weight_materializations == 0
+
+
+# ------------------------------------------------------------------ a predictive package of the reference's builder
+
+PREDICTIVE = Path(__file__).resolve().parent / "golden" / "reference_predictive_package"
+UP, GATE, DOWN = (f"model.layers.0.mlp.{n}_proj.weight" for n in ("up", "gate", "down"))
+
+
+class Block(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.gate_proj = nn.Linear(256, 384, bias=False)
+        self.up_proj = nn.Linear(256, 384, bias=False)
+        self.down_proj = nn.Linear(384, 256, bias=False)
+
+
+class Layer(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.input_layernorm = nn.LayerNorm(256, bias=False)
+        self.mlp = Block()
+
+
+class Inner(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.embed_tokens = nn.Embedding(64, 256)
+        self.layers = nn.ModuleList([Layer()])
+
+
+class Causal(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.model = Inner()
+
+    def forward(self, ids):
+        layer = self.model.layers[0]
+        h = layer.input_layernorm(self.model.embed_tokens(ids))
+        return layer.mlp.down_proj(torch.nn.functional.silu(layer.mlp.gate_proj(h)) * layer.mlp.up_proj(h))
+
+
+def _predictive_source():
+    with np.load(PREDICTIVE / "source_words.npz") as z:
+        return {name: z[name] for name in z.files}
+
+
+def _predictive_package(tmp_path):
+    target = tmp_path / "predictive"
+    shutil.copytree(PREDICTIVE, target, ignore=shutil.ignore_patterns("source_words.npz"))
+    return target
+
+
+def test_predictive_manifest_of_the_builder_is_read_and_every_tensor_resolves(tmp_path):
+    """The reference's predictive builder (GCR/bitexact_predictive_package.py:138-394, run by
+    tests/golden/make_golden_predictive_package.py) kept up as a single-reference candidate and
+    down as a mixed-reference candidate stored transposed, with deflated coefficients: the
+    reader takes the receipts from the compressed parent manifest, the candidates resolve on
+    the host to the source words -- the mix predictor's output hashing to the builder's
+    ``derived_reference_sha256`` on the way -- and the inventory, the receipt archive and the
+    restored shard check out."""
+    package = _predictive_package(tmp_path)
+    manifest, entries = pkg.read_manifest(package)
+    source = _predictive_source()
+    assert manifest["schema"] == pkg.PREDICTIVE_SCHEMA and set(entries) == set(source)
+    selected = pkg.read_candidates(package, manifest, entries)
+    assert set(selected) == {UP, DOWN}
+    assert selected[UP]["mode"] == "single" and selected[UP]["transform"] == "identity"
+    assert [r["name"] for r in selected[UP]["references"]] == [GATE]
+    assert selected[DOWN]["mode"] == "mixbf16" and selected[DOWN]["transform"] == "target transpose"
+    assert [r["name"] for r in selected[DOWN]["references"]] == [UP, GATE]
+    assert selected[DOWN]["coefficients"]["encoding"] == "zlib"
+    for name in (UP, DOWN):  # the builder removes the context frames it replaced
+        assert not pkg.frame_path(package, entries[name]["frame"]).exists()
+    resolver = pkg.TensorResolver(package, manifest, entries)
+    for name, words in source.items():
+        assert np.array_equal(resolver.words(name), words), name
+    totals = pkg.verify(package)
+    assert totals["tensors"] == 5 and totals["predictive_candidates"] == 2 and totals["receipt_members"] == 5
+    assert totals["frame_bytes"] == sum(entries[n]["frame_bytes"] for n in entries) - sum(
+        c["physical_saved_bytes"] for c in selected.values())
+    assert pkg.verify_inventory(package, manifest, absent=DROPPED) == len(manifest["files"]) - len(manifest["decoder_files"])
+    done = pkg.restore(package, tmp_path / "restored")
+    assert done == {"tensors": 5, "shards": 1, "assets": 13}
+    shard = tmp_path / "restored" / "model-00001-of-00018.safetensors"
+    assert hashlib.sha256(shard.read_bytes()).hexdigest() == manifest["source"]["shards"][shard.name]["sha256"]
+    # tampering: the parent manifest, a candidate frame, the coefficient file
+    packed = package / "baseline-manifest.json.xz"
+    good = packed.read_bytes()
+    import lzma
+    packed.write_bytes(lzma.compress(lzma.decompress(good).replace(b'"BF16"', b'"BF17"', 1), format=lzma.FORMAT_XZ))
+    with pytest.raises(pkg.PackageError, match="baseline manifest checksum mismatch"):
+        pkg.read_manifest(package)
+    packed.write_bytes(good)
+    frame = package / selected[UP]["frame"]
+    data = bytearray(frame.read_bytes())
+    data[200] ^= 1
+    frame.write_bytes(bytes(data))
+    with pytest.raises(pkg.PackageError, match="candidate frame integrity mismatch"):
+        pkg.verify(package)
+    data[200] ^= 1
+    frame.write_bytes(bytes(data))
+    coeff = package / selected[DOWN]["coefficients"]["path"]
+    coeff.write_bytes(coeff.read_bytes()[:-1] + b"\0")
+    with pytest.raises(pkg.PackageError, match="mixed coefficient checksum mismatch"):
+        pkg.verify(package)
+
+
+def _causal_dense(device="cpu"):
+    dense = Causal().to(torch.bfloat16).to(device)
+    with torch.no_grad():
+        for name, words in _predictive_source().items():
+            dict(dense.named_parameters())[name].copy_(torch.from_numpy(words).view(torch.bfloat16).to(device))
+    return dense
+
+
+@pytest.mark.gpu
+def test_loader_serves_the_builders_predictive_package_on_the_device():
+    """The same package through the loader and the device factories: up stays a PPCX tensor with
+    its context plane resident (fused products, no reference at run time), down -- stored
+    transposed against the mix of up and gate -- is re-framed row-major at load; weights are
+    bit-exact and the forward matches the dense model."""
+    model, receipt = serving.load_predictive_model(PREDICTIVE, model_factory=Causal, device="cuda:0", log=lambda _: None)
+    source = _predictive_source()
+    mlp = model.model.layers[0].mlp
+    assert receipt["status"] == "ok" and receipt["compressed_tensor_count"] == 4
+    assert receipt["reframed_tensors"] == [DOWN] and len(receipt["verified_metadata_assets"]) == 13
+    for layer, name in ((mlp.up_proj, UP), (mlp.gate_proj, GATE), (mlp.down_proj, DOWN)):
+        assert isinstance(layer, serving.BctxLinear)
+        assert np.array_equal(layer.weight.view(torch.uint16).cpu().numpy(), source[name]), name
+    up = mlp.up_proj.context_weight
+    assert isinstance(up, serving.PredictiveContextTensor) and up.native.fused is not None and up.native.has_contexts
+    assert mlp.down_proj.context_weight.row_major.fused is not None
+    dense = _causal_dense("cuda:0")
+    for shape in ((1,), (3, 5), (40,)):
+        ids = torch.from_numpy(np.random.default_rng(9).integers(0, 64, size=shape)).cuda()
+        with torch.no_grad():
+            got, want = model(ids), dense(ids)
+        assert float((got.float() - want.float()).abs().max()) <= 3e-2 * float(want.float().abs().max())
+    assert mlp.up_proj.weight_materializations == 1 and mlp.down_proj.weight_materializations == 1  # the two .weight reads above
+    assert serving.decode_errors(model) == []
