@@ -155,8 +155,12 @@ def load_bctx_mtp(manifest_path, frame_root, text_config, *, device="cuda:0", te
     if tensor_cls is None:
         from .bitexact_context_gpu import HipContextTensor
         tensor_cls = HipContextTensor
-    manifest_path, frame_root = Path(manifest_path), Path(frame_root)
-    listed = json.loads(manifest_path.read_text()).get("tensors", [])
+    frame_root = Path(frame_root)
+    if isinstance(manifest_path, dict):  # a manifest already read (and checked) by the caller
+        listed, manifest_path = manifest_path.get("tensors", []), manifest_path.get("path", "<manifest>")
+    else:
+        manifest_path = Path(manifest_path)
+        listed = json.loads(manifest_path.read_text()).get("tensors", [])
     entries = {t["name"]: t for t in listed if t.get("name", "").startswith("mtp.")}
     if set(entries) != set(MTP_SHAPES):
         raise ValueError(f"MTP manifest keys differ: missing={sorted(set(MTP_SHAPES) - set(entries))}, "
@@ -215,6 +219,42 @@ def load_bctx_mtp(manifest_path, frame_root, text_config, *, device="cuda:0", te
         "m_invariant": bool(m_invariant),
     }
     return mtp
+
+
+def load_predictive_mtp(package, model=None, *, device="cuda:0", checkpoint_stride=1024, tensor_cls=None,
+                        skeleton=None, m_invariant=True, check_inventory=None, optional=("decoder/",)):
+    """The MTP head of a predictive package (GCR/bitexact_predictive_serving.py:997-1079): its
+    fifteen tensors must be unchanged context frames -- a predictive candidate that replaces one
+    is refused -- listed in the package's pinned parent manifest, with their frames intact.
+    ``model`` gives the text configuration the default skeleton needs (``model.config.text_config``
+    or ``model.config``; not needed with ``skeleton``).  A package whose manifest says
+    ``verify_on_load`` has its file inventory and receipt archive checked first
+    (``check_inventory``: None follows the manifest; ``optional``: inventory paths that may be
+    absent, by default the ``decoder/`` copies of the builder's sources, which this library
+    does not use).  Returns ``(head, None, receipt)``: the reference returns its speculator in
+    the middle, which is generation control and is not part of this library."""
+    from . import bitexact_context_package as pkg
+    package = Path(package).resolve()
+    manifest, entries = pkg.read_manifest(package)
+    if check_inventory is None:
+        check_inventory = manifest.get("verify_on_load") is True
+    if check_inventory:
+        pkg.verify_inventory(package, manifest, optional=optional)
+        pkg.verify_receipt_archive(package, manifest)
+    selected = pkg.read_candidates(package, manifest, entries)
+    if set(MTP_SHAPES) - set(entries):
+        raise ValueError("predictive baseline manifest lacks unchanged MTP tensors")
+    for name in MTP_SHAPES:
+        if name in selected:
+            raise ValueError(f"MTP tensor is not an unchanged BCTX frame: {name}")
+        pkg.read_frame(package, entries[name])  # present, regular, of the pinned size and digest
+    config = getattr(getattr(model, "config", None), "text_config", None) or getattr(model, "config", None)
+    if config is None and skeleton is None:
+        raise ValueError("predictive model has no text configuration for MTP")
+    head = load_bctx_mtp({"tensors": [entries[name] for name in MTP_SHAPES], "path": str(package / "manifest.json")},
+                         package, config, device=device, tensor_cls=tensor_cls, checkpoint_stride=checkpoint_stride,
+                         skeleton=skeleton, m_invariant=m_invariant)
+    return head, None, dict(head._bctx_receipt)
 
 
 def bctx_mtp_receipt(mtp, *, require_consumed=False):

@@ -431,7 +431,7 @@ def _sha_file(path):
     return h.hexdigest()
 
 
-def verify_inventory(package, manifest, *, absent=()):
+def verify_inventory(package, manifest, *, absent=(), optional=()):
     """Check a builder-written package against its own ``files`` inventory
     (GCR/bitexact_context_package.py:595-612): every listed path is safe and unique, exactly
     the listed files exist, each has its pinned size and SHA-256 (the manifest pins its own
@@ -439,7 +439,8 @@ def verify_inventory(package, manifest, *, absent=()):
 
     ``absent`` names inventory paths (or prefixes ending in "/") that the holder of the
     package has dropped on purpose, such as the ``decoder/`` copies of the encoder's sources:
-    they are neither required nor allowed on disk.  Returns the number of files checked."""
+    they are neither required nor allowed on disk.  ``optional`` names paths (or prefixes) that
+    may be missing but are checked when present.  Returns the number of files checked."""
     package = Path(package)
     files = manifest.get("files")
     if not isinstance(files, list):
@@ -460,12 +461,14 @@ def verify_inventory(package, manifest, *, absent=()):
         expected[row["path"]] = row
     if any(p.is_symlink() for p in package.rglob("*")):
         raise PackageError("package must contain regular files, not symlinks")
-    dropped = lambda rel: any(rel == a or (a.endswith("/") and rel.startswith(a)) for a in absent)
-    required = {rel for rel in expected if not dropped(rel)}
+    named = lambda rel, names: any(rel == a or (a.endswith("/") and rel.startswith(a)) for a in names)
+    allowed = {rel for rel in expected if not named(rel, absent)}
+    required = {rel for rel in allowed if not named(rel, optional)}
     actual = {p.relative_to(package).as_posix() for p in package.rglob("*") if p.is_file()}
-    if actual != required:
-        odd = sorted(actual ^ required)
+    if not required <= actual <= allowed:
+        odd = sorted((required - actual) | (actual - allowed))
         raise PackageError(f"package file inventory mismatch: {odd[:4]}")
+    required = actual
     for rel in sorted(required):
         row, path = expected[rel], package.joinpath(*PurePosixPath(rel).parts)
         if path.stat().st_size != row["bytes"] or (row["sha256"] is not None and _sha_file(path) != row["sha256"]):

@@ -288,7 +288,7 @@ def _runtime_dtype(model, name, parameter, requested):
 def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
                     tensor_factory=None, predictive_factory=None, mix_predictor=None, host_decoder=None,
                     loader_workers=1, batch_invariant=False, log=print, progress_callback=None,
-                    share_launches=(), reframe_transposed=True):
+                    share_launches=(), reframe_transposed=True, check_inventory=None, optional_files=("decoder/",)):
     """Build ``model_factory()`` on the meta device and fill it from a BCTX package without
     ever holding a dense checkpoint: returns ``(model, receipt)``.
 
@@ -323,7 +323,12 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
     through the matrix-core kernel, so a verify pass over k + 1 rows reproduces the one-row
     decode steps bit for bit (GS/miv_gemv.py:1-9); the default lets the row count pick the
     fastest kernel, and rows are then bit-equal only between calls of the same kernel family
-    (``bitexact_context_gpu.route_rows``).  The receipt records the choice.  What this loader leaves to the caller is the model
+    (``bitexact_context_gpu.route_rows``).  The receipt records the choice.  ``check_inventory``: check
+    every file of the package against the manifest's ``files`` inventory (and the archive of the
+    parent package's receipts) before anything is served; None does so when the manifest says
+    ``verify_on_load``, as the reference's predictive packages do; ``optional_files`` names
+    inventory paths that may be absent (the ``decoder/`` copies of the builder's sources, which
+    this library does not use).  What this loader leaves to the caller is the model
     construction itself (the reference reads a Transformers config and generation config
     from the package's sidecars): ``model_factory`` returns the module to fill."""
     import hashlib
@@ -342,6 +347,13 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         manifest, entries = pkg.read_manifest(package)
         # the model's configuration sidecars are checked against their pins before any weight is read
         sidecars = pkg.read_metadata(package, manifest) if ("metadata_assets" in manifest or "files" in manifest) else {}
+        # a package that asks for it is checked file by file before anything is served from it
+        # (the reference's predictive loader runs its package verifier at load,
+        # GCR/bitexact_predictive_serving.py:727-731)
+        inventory_checked = manifest.get("verify_on_load") is True if check_inventory is None else bool(check_inventory)
+        if inventory_checked:
+            pkg.verify_inventory(package, manifest, optional=optional_files)
+            pkg.verify_receipt_archive(package, manifest)
     except pkg.PackageError as exc:
         raise ContextServingError(str(exc)) from exc
     if tensor_factory is None:
@@ -656,6 +668,7 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
         "transcoded": any(r.get("residual_repacked") for r in consumed.values()) or bool(reframed),
         # predictive frames stored transposed that were decoded, turned and encoded row-major at load
         "reframed_tensors": sorted(reframed),
+        "package_inventory_checked": inventory_checked,
         "residual_repacked_tensors": sorted(n for n, r in consumed.items() if r.get("residual_repacked")),
         "general_kernel_tensors": sorted(n for n, r in consumed.items()
                                          if r.get("fused") is False and r.get("frame_mode") != 1),
@@ -668,7 +681,8 @@ def load_bctx_model(package, *, model_factory, device="cuda:0", dtype=torch.bflo
 def load_predictive_model(package, *, model_factory, device="cuda:0", dtype=torch.bfloat16, stride=1024,
                           tensor_factory=None, context_factory=None, predictive_factory=None, mix_predictor=None,
                           host_decoder=None, loader_workers=1, batch_invariant=False, log=print,
-                          progress_callback=None, share_launches=(), reframe_transposed=True):
+                          progress_callback=None, share_launches=(), reframe_transposed=True, check_inventory=None,
+                          optional_files=("decoder/",)):
     """The predictive-package loader under the reference's name and keywords
     (GCR/bitexact_predictive_serving.py:596-619): ``context_factory`` makes the BCTX tensors
     (``tensor_factory`` is accepted as its older spelling), ``predictive_factory`` the PPCX ones,
@@ -685,5 +699,6 @@ def load_predictive_model(package, *, model_factory, device="cuda:0", dtype=torc
                            tensor_factory=context_factory or tensor_factory, predictive_factory=predictive_factory,
                            mix_predictor=mix_predictor, host_decoder=host_decoder, loader_workers=loader_workers,
                            batch_invariant=batch_invariant, log=log, progress_callback=progress_callback,
-                           share_launches=share_launches, reframe_transposed=reframe_transposed)
+                           share_launches=share_launches, reframe_transposed=reframe_transposed,
+                           check_inventory=check_inventory, optional_files=optional_files)
 

@@ -279,16 +279,21 @@ def _causal_dense(device="cpu"):
 
 
 @pytest.mark.gpu
-def test_loader_serves_the_builders_predictive_package_on_the_device():
+def test_loader_serves_the_builders_predictive_package_on_the_device(tmp_path):
     """The same package through the loader and the device factories: up stays a PPCX tensor with
     its context plane resident (fused products, no reference at run time), down -- stored
     transposed against the mix of up and gate -- is re-framed row-major at load; weights are
     bit-exact and the forward matches the dense model."""
-    model, receipt = serving.load_predictive_model(PREDICTIVE, model_factory=Causal, device="cuda:0", log=lambda _: None)
+    package = _predictive_package(tmp_path)
+    model, receipt = serving.load_predictive_model(package, model_factory=Causal, device="cuda:0", log=lambda _: None)
     source = _predictive_source()
+    (package / "stray.bin").write_bytes(b"x")
+    with pytest.raises(serving.ContextServingError, match="inventory mismatch"):
+        serving.load_predictive_model(package, model_factory=Causal, device="cuda:0", log=lambda _: None)
     mlp = model.model.layers[0].mlp
     assert receipt["status"] == "ok" and receipt["compressed_tensor_count"] == 4
     assert receipt["reframed_tensors"] == [DOWN] and len(receipt["verified_metadata_assets"]) == 13
+    assert receipt["package_inventory_checked"] is True  # the manifest says verify_on_load
     for layer, name in ((mlp.up_proj, UP), (mlp.gate_proj, GATE), (mlp.down_proj, DOWN)):
         assert isinstance(layer, serving.BctxLinear)
         assert np.array_equal(layer.weight.view(torch.uint16).cpu().numpy(), source[name]), name

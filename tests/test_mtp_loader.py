@@ -186,3 +186,69 @@ def test_frame_geometry_and_path_guard(tmp_path):
     assert _safe_frame_path(tmp_path, "frames/a.bctx") == (tmp_path / "frames" / "a.bctx").resolve()
     with pytest.raises(ValueError, match="escapes frame_root"):
         _safe_frame_path(tmp_path, "../outside.bctx")
+
+
+def test_head_of_a_predictive_package(tmp_path):
+    """load_predictive_mtp: the fifteen tensors come from the pinned parent manifest of a
+    predictive package and must be unchanged context frames; the inventory is checked when the
+    manifest says ``verify_on_load``; a candidate that replaces an MTP tensor, a frame that was
+    touched and a stray file are refused."""
+    import lzma
+    from georefine_amd import bitexact_context_package as pkg
+    from georefine_amd.bitexact_context_mtp import load_predictive_mtp
+    package = tmp_path / "package"
+    package.mkdir()
+    parent = _package(package)
+    parent["tensors"][0].update(frame="frames/head.bctx", frame_bytes=4, frame_sha256=hashlib.sha256(b"head").hexdigest(),
+                                source_sha256="2" * 64, source_bytes=8, complete=True)
+    (package / "frames" / "head.bctx").write_bytes(b"head")
+    for row in parent["tensors"][1:]:
+        row.update(complete=True, source_bytes=2 * int(torch.tensor(row["shape"]).prod()))
+    parent.update(schema=pkg.SCHEMA, complete=True)
+    raw = json.dumps(parent).encode()
+    (package / "baseline-manifest.json.xz").write_bytes(lzma.compress(raw, format=lzma.FORMAT_XZ))
+
+    def write(selected=None):
+        manifest = {"schema": pkg.PREDICTIVE_SCHEMA, "complete": True, "verify_on_load": True,
+                    "baseline_manifest_sha256": hashlib.sha256(raw).hexdigest(), "baseline_manifest_bytes": len(raw),
+                    "baseline_manifest_encoding": "xz", "selected_candidates": selected or {}, "metadata_assets": {}}
+        files = [{"path": p.relative_to(package).as_posix(), "bytes": p.stat().st_size,
+                  "sha256": hashlib.sha256(p.read_bytes()).hexdigest()}
+                 for p in sorted(package.rglob("*")) if p.is_file() and p.name != "manifest.json"]
+        manifest["files"] = files + [{"path": "manifest.json", "bytes": 0, "sha256": None}]
+        for _ in range(5):
+            size = len(json.dumps(manifest).encode())
+            manifest["files"][-1]["bytes"] = size
+            manifest["package_bytes"] = sum(f["bytes"] for f in manifest["files"])
+        (package / "manifest.json").write_text(json.dumps(manifest))
+
+    write()
+    fake = _fake_tensor_class(parent, package)
+    load = lambda: load_predictive_mtp(package, None, device="cpu", tensor_cls=fake, skeleton=lambda _c: TinyMTP())
+    head, speculator, receipt = load()
+    assert speculator is None and receipt["tensor_count"] == 15 and receipt["m_invariant"] is True
+    assert isinstance(head.fc, BCTXLinear) and receipt["manifest"].endswith("manifest.json")
+    (package / "stray.bin").write_bytes(b"x")
+    with pytest.raises(ValueError, match="inventory mismatch"):
+        load()
+    (package / "stray.bin").unlink()
+    frame = package / "frames" / "f03.bctx"
+    good = frame.read_bytes()
+    frame.write_bytes(good[:-1] + b"?")
+    with pytest.raises(ValueError, match="integrity mismatch"):
+        load()
+    frame.write_bytes(good)
+    name = "mtp.fc.weight"
+    row = next(r for r in parent["tensors"] if r["name"] == name)
+    (package / "predictive-frames").mkdir()
+    (package / "predictive-frames" / "x.ppcx").write_bytes(b"ppcx")
+    write({name: {"schema": pkg.CANDIDATE_SCHEMA, "name": name, "mode": "single", "transform": "identity",
+                  "references": [{"name": "mtp.norm.weight", "sha256": next(
+                      r for r in parent["tensors"] if r["name"] == "mtp.norm.weight")["source_sha256"]}],
+                  "shape": row["shape"], "source_sha256": row["source_sha256"], "source_bytes": row["source_bytes"],
+                  "frame": "predictive-frames/x.ppcx", "frame_bytes": 4, "frame_sha256": hashlib.sha256(b"ppcx").hexdigest()}})
+    with pytest.raises(ValueError, match="not an unchanged BCTX frame"):
+        load()
+    write()
+    with pytest.raises(ValueError, match="no text configuration"):
+        load_predictive_mtp(package, None, device="cpu", tensor_cls=fake, check_inventory=False)
