@@ -71,6 +71,67 @@ class SharedProducts:
         return out
 
 
+def prepare_metadata(package, cache_dir):
+    """Verify the package's metadata sidecars (the model's configuration files) and return a
+    directory that holds them, outside the package: the package's own ``sidecars/`` directory when
+    it carries one, else ``cache_dir/<SHA-256 of model-assets.tar.xz>/sidecars``, extracted once and
+    re-checked file by file when it already exists (GCR/bitexact_context_serving.py:175-274).  A
+    builder-written package pins thirteen of them; anything else is refused, as is a cache inside
+    the package."""
+    import hashlib
+    import os
+    import shutil
+    import tempfile
+    from pathlib import Path, PurePosixPath
+
+    from . import bitexact_context_package as pkg
+    package, cache_dir = Path(package).resolve(), Path(cache_dir).resolve()
+    if cache_dir == package or package in cache_dir.parents:
+        raise ContextServingError("metadata cache must be outside the immutable package")
+    try:
+        manifest, _ = pkg.read_manifest(package)
+        members = pkg.read_metadata(package, manifest)
+    except pkg.PackageError as exc:
+        raise ContextServingError(str(exc)) from exc
+    pins = manifest.get("metadata_assets") or {}
+    if len(pins) != 13:
+        raise ContextServingError("BCTX v1 metadata inventory must contain 13 sidecars")
+    if (package / "sidecars").exists():  # checked against the pins by read_metadata
+        return package / "sidecars"
+    archive_sha = hashlib.sha256((package / "model-assets.tar.xz").read_bytes()).hexdigest()
+    cache_dir.mkdir(parents=True, exist_ok=True)
+    destination = cache_dir / archive_sha
+    if destination.is_symlink():
+        raise ContextServingError("metadata cache destination must not be a symlink")
+    if destination.exists():
+        if not destination.is_dir():
+            raise ContextServingError("metadata cache destination is not a directory")
+        present = {}
+        for path in destination.rglob("*"):
+            if path.is_symlink():
+                raise ContextServingError("metadata cache contains a symlink")
+            if path.is_file():
+                present[path.relative_to(destination).as_posix()] = path
+        if set(present) != set(pins):
+            raise ContextServingError("existing metadata cache inventory mismatch")
+        for name, pin in pins.items():
+            payload = present[name].read_bytes()
+            if len(payload) != pin["bytes"] or hashlib.sha256(payload).hexdigest() != pin["sha256"]:
+                raise ContextServingError(f"existing metadata cache integrity mismatch: {name}")
+    else:
+        staging = Path(tempfile.mkdtemp(prefix=archive_sha + ".partial-", dir=cache_dir))
+        try:
+            for name, payload in members.items():
+                target = staging.joinpath(*PurePosixPath(name).parts)
+                target.parent.mkdir(parents=True, exist_ok=True)
+                target.write_bytes(payload)
+            os.replace(staging, destination)
+        except Exception:
+            shutil.rmtree(staging, ignore_errors=True)
+            raise
+    return destination / "sidecars"
+
+
 def decode_errors(model):
     """Names of the coded modules of ``model`` whose device error word is set (a segment did
     not end on its checkpoint in some launch since the word was last cleared).  The fused

@@ -308,3 +308,29 @@ def test_loader_serves_the_builders_predictive_package_on_the_device(tmp_path):
         assert float((got.float() - want.float()).abs().max()) <= 3e-2 * float(want.float().abs().max())
     assert mlp.up_proj.weight_materializations == 1 and mlp.down_proj.weight_materializations == 1  # the two .weight reads above
     assert serving.decode_errors(model) == []
+
+
+def test_prepare_metadata_extracts_the_verified_sidecars_outside_the_package(tmp_path):
+    package = _package(tmp_path)
+    manifest, _ = pkg.read_manifest(package)
+    where = serving.prepare_metadata(package, tmp_path / "cache")
+    archive_sha = hashlib.sha256((package / "model-assets.tar.xz").read_bytes()).hexdigest()
+    assert where == (tmp_path / "cache" / archive_sha / "sidecars").resolve()
+    found = {p.relative_to(where.parent).as_posix(): p.read_bytes() for p in where.rglob("*") if p.is_file()}
+    assert found == pkg.read_metadata(package, manifest) and len(found) == 13
+    assert json.loads((where / "config.json").read_text())["hidden_size"] == 128
+    assert serving.prepare_metadata(package, tmp_path / "cache") == where  # found again, re-checked
+    (where / "config.json").write_bytes(b"{}")
+    with pytest.raises(serving.ContextServingError, match="existing metadata cache integrity mismatch"):
+        serving.prepare_metadata(package, tmp_path / "cache")
+    (where / "extra.json").write_bytes(b"{}")
+    with pytest.raises(serving.ContextServingError, match="existing metadata cache inventory mismatch"):
+        serving.prepare_metadata(package, tmp_path / "cache")
+    with pytest.raises(serving.ContextServingError, match="outside the immutable package"):
+        serving.prepare_metadata(package, package / "cache")
+    # a package that carries its sidecars as files is served from them
+    physical = tmp_path / "physical"
+    shutil.copytree(package, physical)
+    shutil.copytree(serving.prepare_metadata(package, tmp_path / "cache2"), physical / "sidecars")
+    assert serving.prepare_metadata(physical, tmp_path / "cache3") == (physical / "sidecars").resolve()
+    assert not (tmp_path / "cache3").exists()
