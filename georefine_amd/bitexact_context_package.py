@@ -42,6 +42,7 @@ SCHEMA = "bitexact-context-package-v1"
 # frames of some tensors are replaced by PPCX frames (``selected_candidates``); the context
 # package's manifest, with every tensor's receipt, is kept beside it, compressed and pinned.
 PREDICTIVE_SCHEMA = "bitexact-predictive-context-package-v1"
+LEGACY_PREDICTIVE_SCHEMA = "private-predictive-context-package-v1"  # older packages: no ``verify_on_load``
 CANDIDATE_SCHEMA = "ppcx-reference-conditioned-bf16-v1"
 
 
@@ -86,11 +87,19 @@ def read_manifest(package):
         manifest = json.loads(path.read_text(encoding="utf-8"), object_pairs_hook=_unique)
     except (OSError, json.JSONDecodeError) as exc:
         raise PackageError(f"cannot read BCTX manifest: {exc}") from exc
-    if (not isinstance(manifest, dict) or manifest.get("schema") not in (SCHEMA, PREDICTIVE_SCHEMA)
+    if (not isinstance(manifest, dict)
+            or manifest.get("schema") not in (SCHEMA, PREDICTIVE_SCHEMA, LEGACY_PREDICTIVE_SCHEMA)
             or manifest.get("complete") is not True):
         raise PackageError("unsupported or incomplete BCTX package manifest")
-    if manifest["schema"] == PREDICTIVE_SCHEMA:
+    # a predictive package keeps the receipts in its parent's manifest; of a tensor that a
+    # candidate replaces only the source identity still holds there (its context frame is gone),
+    # and the reference's loader asks nothing more of those rows
+    # (GCR/bitexact_predictive_serving.py:655-671)
+    predictive = manifest["schema"] != SCHEMA
+    replaced = ()
+    if predictive:
         manifest = dict(manifest, tensors=_parent_receipts(package, manifest))
+        replaced = manifest.get("selected_candidates") if isinstance(manifest.get("selected_candidates"), dict) else ()
     rows = manifest.get("tensors")
     if not isinstance(rows, list):
         raise PackageError("manifest tensors must be a list")
@@ -101,18 +110,19 @@ def read_manifest(package):
         name = row["name"]
         if name in entries:
             raise PackageError(f"duplicate tensor receipt: {name}")
-        if row.get("complete") is not True or row.get("dtype") != "BF16":
+        if (row.get("complete") is not True and not predictive) or row.get("dtype") != "BF16":
             raise PackageError(f"incomplete or unsupported tensor receipt: {name}")
-        if not _is_digest(row.get("source_sha256")) or not _is_digest(row.get("frame_sha256")):
+        if not _is_digest(row.get("source_sha256")) or not (_is_digest(row.get("frame_sha256")) or name in replaced):
             raise PackageError(f"invalid source/frame SHA: {name}")
         shape = row.get("shape")
         if not isinstance(shape, list) or not shape or any(type(d) is not int or d <= 0 for d in shape):
             raise PackageError(f"invalid tensor shape: {name}")
         if row.get("source_bytes") != 2 * math.prod(shape):
             raise PackageError(f"invalid BF16 source byte count: {name}")
-        if type(row.get("frame_bytes")) is not int or row["frame_bytes"] <= 0:
-            raise PackageError(f"invalid BCTX frame byte count: {name}")
-        frame_path(package, row.get("frame"))
+        if name not in replaced:
+            if type(row.get("frame_bytes")) is not int or row["frame_bytes"] <= 0:
+                raise PackageError(f"invalid BCTX frame byte count: {name}")
+            frame_path(package, row.get("frame"))
         entries[name] = row
     return manifest, entries
 
@@ -124,7 +134,7 @@ def _parent_receipts(package, manifest):
     446-450).  ``verify_on_load`` must be set, as the reference's reader demands of this schema."""
     import lzma
     package = Path(package)
-    if manifest.get("verify_on_load") is not True:
+    if manifest.get("schema") == PREDICTIVE_SCHEMA and manifest.get("verify_on_load") is not True:
         raise PackageError("predictive package lacks stable verification metadata")
     plain, packed = package / "baseline-manifest.json", package / "baseline-manifest.json.xz"
     if plain.is_file() == packed.is_file():
@@ -141,8 +151,8 @@ def _parent_receipts(package, manifest):
         parent = json.loads(raw, object_pairs_hook=_unique)
     except json.JSONDecodeError as exc:
         raise PackageError("baseline manifest is not JSON") from exc
-    if not isinstance(parent, dict) or parent.get("schema") != SCHEMA or parent.get("complete") is not True:
-        raise PackageError("baseline manifest is not a complete context-package manifest")
+    if not isinstance(parent, dict):
+        raise PackageError("baseline manifest is not an object")
     return parent.get("tensors")
 
 
@@ -569,7 +579,8 @@ def read_candidates(package, manifest, entries):
     frames = set()
     for name, c in selected.items():
         row = entries.get(name)
-        if row is None or not isinstance(c, dict) or c.get("name") != name or c.get("schema") != CANDIDATE_SCHEMA:
+        if (row is None or not isinstance(c, dict) or c.get("name") != name
+                or c.get("schema") != manifest.get("experimental_codec", CANDIDATE_SCHEMA)):
             raise PackageError(f"candidate schema/name mismatch: {name}")
         refs = c.get("references")
         wanted = {"single": 1, "mixbf16": 2}.get(c.get("mode"))

@@ -334,3 +334,30 @@ def test_prepare_metadata_extracts_the_verified_sidecars_outside_the_package(tmp
     shutil.copytree(serving.prepare_metadata(package, tmp_path / "cache2"), physical / "sidecars")
     assert serving.prepare_metadata(physical, tmp_path / "cache3") == (physical / "sidecars").resolve()
     assert not (tmp_path / "cache3").exists()
+
+
+def test_legacy_predictive_layout_remains_readable(tmp_path):
+    """Older predictive packages (GCR/bitexact_predictive_package.py:12, 47-57; the reference's
+    tests/test_bitexact_predictive_package.py:126-138): another schema name, no ``verify_on_load``,
+    the parent manifest stored plain.  Both forms of the parent manifest at once are refused."""
+    import lzma
+    package = _predictive_package(tmp_path)
+    manifest = json.loads((package / "manifest.json").read_text())
+    manifest["schema"] = pkg.LEGACY_PREDICTIVE_SCHEMA
+    manifest.pop("verify_on_load")
+    packed = package / "baseline-manifest.json.xz"
+    (package / "baseline-manifest.json").write_bytes(lzma.decompress(packed.read_bytes()))
+    stored = packed.read_bytes()
+    packed.unlink()
+    (package / "manifest.json").write_text(json.dumps(manifest))
+    read, entries = pkg.read_manifest(package)
+    assert read["schema"] == pkg.LEGACY_PREDICTIVE_SCHEMA and len(entries) == 5
+    assert pkg.verify(package)["predictive_candidates"] == 2
+    packed.write_bytes(stored)
+    with pytest.raises(pkg.PackageError, match="missing or ambiguous"):
+        pkg.read_manifest(package)
+    packed.unlink()
+    manifest["schema"] = pkg.PREDICTIVE_SCHEMA  # the current schema must say verify_on_load
+    (package / "manifest.json").write_text(json.dumps(manifest))
+    with pytest.raises(pkg.PackageError, match="stable verification metadata"):
+        pkg.read_manifest(package)
