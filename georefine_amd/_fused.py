@@ -381,6 +381,23 @@ def order_residuals(raw, rows, cols, seg_len, block, position, held):
     return np.ascontiguousarray(ordered).reshape(-1)
 
 
+def order_index(values, rows, spr, block, position, held):
+    """An index array of a frame (segment states or offsets, ``rows * spr + 1`` entries in the
+    frame's order: the end of a segment is the entry after it) in the blocked order of the
+    residuals: every row gets ``spr + 1`` entries of its own -- the last one is the end of its
+    stream, i.e. the next row's first entry -- and entry s of position q goes to
+    ``((q // block) * (spr + 1) + s) * block + q % block``.  The entries that a wave unit, or the
+    sixteen rows of a matrix-core wave, read at one visit are then one run of bytes instead of a
+    few bytes out of every row's own line.  Positions that no row has hold zeros."""
+    values = np.asarray(values)
+    per_row = np.empty((rows, spr + 1), dtype=values.dtype)
+    per_row[:, :spr] = values[:rows * spr].reshape(rows, spr)
+    per_row[:, spr] = values[spr::spr][:rows]
+    ordered = np.zeros((held, spr + 1), dtype=values.dtype)
+    ordered[position] = per_row
+    return np.ascontiguousarray(ordered.reshape(held // block, block, spr + 1).transpose(0, 2, 1)).reshape(-1)
+
+
 def order_records(raw, rows, cols, seg_len, block, position, held, record_symbols, record_bytes):
     """``order_residuals`` for records of another size: ``record_symbols`` consecutive symbols of a
     row in ``record_bytes`` bytes (the predictive codec's 32 five-bit residuals in 20 bytes, or
@@ -651,7 +668,13 @@ def validate_host(plan, tiling, use, *, row_pos=None, block=0, main_bytes=None):
     g = _hip_abi.GrfFusedTiling()
     for key, value in tiling["scalars"].items():
         setattr(g, key, value)
-    arrays = [np.ascontiguousarray(plan.seg_offset, dtype=np.uint32),
+    offsets = plan.seg_offset
+    if block:  # the library reads the index in the order the frame structure declares
+        if row_pos is None:
+            raise FusedUnsupported("the blocked order needs the rows' positions")
+        held = -(-(int(np.max(row_pos)) + 1) // block) * block
+        offsets = order_index(offsets, plan.rows, plan.spr, block, row_pos, held)
+    arrays = [np.ascontiguousarray(offsets, dtype=np.uint32),
               np.ascontiguousarray(tiling["tile_rows"], dtype=np.uint32),
               np.ascontiguousarray(tiling["tile_class"], dtype=np.uint8),
               np.ascontiguousarray(plan.row_class, dtype=np.uint8),

@@ -235,8 +235,12 @@ class HipContextTensor:
                 indexed["residual_stream"] = _fused.order_residuals(raw, rows_, cols_, seg, block, position, held)
                 indexed["row_pos"] = position
                 raw6_segment, raw6_block = seg, block
-            indexed.update(fused_seg_state=plan.seg_state, fused_seg_offset=plan.seg_offset, fused_lut=plan.lut,
-                           fused_tab=plan.tab)
+            states, offsets = plan.seg_state, plan.seg_offset
+            if raw6_segment:  # the segment index in the same blocked order (``_fused.order_index``)
+                spr_ = cols_ // seg
+                states = _fused.order_index(states, rows_, spr_, block, position, held)
+                offsets = _fused.order_index(offsets, rows_, spr_, block, position, held)
+            indexed.update(fused_seg_state=states, fused_seg_offset=offsets, fused_lut=plan.lut, fused_tab=plan.tab)
         return {"indexed": indexed, "plan": plan, "reason": reason, "stride": stride, "fused": fused,
                 "main_bytes": main_bytes, "raw6_segment": raw6_segment, "raw6_block": raw6_block}
 
@@ -351,12 +355,28 @@ class HipContextTensor:
             by_row = raw[:held * groups * spr * 12].view(held // old, groups, spr, old, 12).permute(0, 3, 1, 2, 4)
             by_row = by_row.reshape(held // residual_block, residual_block, groups, spr, 12)
             other.buffers["residual_stream"] = by_row.permute(0, 2, 3, 1, 4).contiguous().view(-1)
+            for name in ("fused_seg_state", "fused_seg_offset"):  # the index is in the same blocked order
+                kind = other.buffers[name].dtype
+                index = other.buffers[name].view(torch.int32).view(held // old, spr + 1, old).permute(0, 2, 1)
+                index = index.reshape(held // residual_block, residual_block, spr + 1).permute(0, 2, 1)
+                other.buffers[name] = index.contiguous().view(-1).view(kind)
             other._raw6_block = residual_block
         other.error = torch.zeros_like(self.error)
         other.resident_bytes = int(sum(t.numel() * t.element_size() for t in other.buffers.values())
                                    + other.error.numel() * other.error.element_size())
         other._bind()
         return other
+
+    def index_slot(self, row, segment):
+        """Where the checkpoint of ``segment`` (0..segments per row; the last is the end of the
+        row's stream) of ``row`` lies in ``buffers["fused_seg_state"]`` / ``["fused_seg_offset"]``:
+        in the blocked order of the resident residuals when the tensor keeps them so
+        (``_fused.order_index``), else in the frame's order."""
+        spr = self.shape[1] // self.fused_plan["seg_len"]
+        if not self._raw6_segment:
+            return row * spr + segment
+        q, block = int(self.buffers["row_pos"][row].item()), self._raw6_block
+        return ((q // block) * (spr + 1) + segment) * block + q % block
 
     def _tiling(self, m):
         """Device copy of the tiling used for m activation rows (0 = store sink).  The GEMV has

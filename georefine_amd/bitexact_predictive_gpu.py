@@ -260,7 +260,12 @@ class HipPredictiveTensor:
         """Upload the walker's derived arrays: segment index, per-label tables, store tiling."""
         import torch
         plan, b = self._plan, self.buffers
-        for name, array in (("fused_seg_state", plan.seg_state), ("fused_seg_offset", plan.seg_offset),
+        states, offsets = plan.seg_state, plan.seg_offset
+        if self._raw5_segment and "fused_seg_state" not in b:  # the index in the residuals' blocked order
+            spr, position = self.shape[1] // self._raw5_segment, b["row_pos"].cpu().numpy()
+            states = _fused.order_index(states, self.shape[0], spr, self._raw5_block, position, self._rows_held)
+            offsets = _fused.order_index(offsets, self.shape[0], spr, self._raw5_block, position, self._rows_held)
+        for name, array in (("fused_seg_state", states), ("fused_seg_offset", offsets),
                             ("fused_lut", plan.lut), ("fused_tab", plan.tab.view(np.int64))):
             if name not in b:  # (a clone already holds its copies)
                 b[name] = torch.from_numpy(np.ascontiguousarray(array)).to(self.device)
@@ -280,6 +285,16 @@ class HipPredictiveTensor:
         self.fused = f
         store = self._tiling_for(0)
         self.fused_plan = dict(sc, **store[3])
+
+    def index_slot(self, row, segment):
+        """Where the checkpoint of ``segment`` (0..segments per row; the last is the end of the
+        row's stream) of ``row`` lies in ``buffers["fused_seg_state"]`` / ``["fused_seg_offset"]``
+        (blocked order when the residuals are resident in it, else the frame's order)."""
+        spr = self.shape[1] // self._plan.seg_len
+        if not self._raw5_segment:
+            return row * spr + segment
+        q, block = int(self.buffers["row_pos"][row].item()), self._raw5_block
+        return ((q // block) * (spr + 1) + segment) * block + q % block
 
     def _tiling_for(self, key):
         """Device copy of a tiling: key 0 = store sink, "waves" = the GEMV (wave units, one tiling

@@ -354,14 +354,35 @@ __device__ __forceinline__ void fused_load_tables(uint8_t *lds, uint32_t blocks,
   }
 }
 
-// Byte range of one row piece (segments [seg_base, seg_base+nseg)) in the main stream.  The
+// Where the checkpoint of a segment lies in the index arrays (seg_state, seg_offset).  In the
+// frame's order (raw_interleaved == 0) segment s of row r is entry r * segs_per_row + s and its
+// end is the entry after it.  In the blocked order the residuals have (raw_interleaved = B rows
+// per block, rows by position) every row has segs_per_row + 1 entries -- the last one is the end
+// of its stream -- and entry s of position q lies at ((q / B) * (segs_per_row + 1) + s) * B + q % B:
+// the entries that a wave unit, or the sixteen rows of a GEMM wave, read at one visit are then
+// one run of bytes, as its residuals are, instead of a few bytes out of every row's own line.
+// `frame_order`: the segment's number in the frame's order, rpos: the row's position, s: the
+// segment in its row.  The entry of the segment's end is fused_seg_step further on.
+__device__ __forceinline__ uint32_t fused_seg_slot(const grf_bctx_fused &f, uint32_t frame_order, uint32_t rpos,
+                                                   uint32_t s) {
+  if (!f.raw_interleaved) return frame_order;
+  const uint32_t B = f.raw_interleaved, within = rpos & (B - 1);
+  return (rpos - within) * (f.segs_per_row + 1) + s * B + within;
+}
+__device__ __forceinline__ uint32_t fused_seg_step(const grf_bctx_fused &f) {
+  return f.raw_interleaved ? f.raw_interleaved : 1u;
+}
+
+// Byte range of one row piece (segments [s, s + nseg) of a row) in the main stream.  The
 // kernels fetch it one slab ahead: it is the first of two dependent global reads before a
 // slab's bytes can be copied.
 struct PieceSpan {
   uint32_t g0, g1;
-  __device__ __forceinline__ void fetch(const grf_bctx_fused &f, uint32_t seg_base, uint32_t nseg) {
-    g0 = f.seg_offset[seg_base];
-    g1 = f.seg_offset[seg_base + nseg];
+  __device__ __forceinline__ void fetch(const grf_bctx_fused &f, uint32_t frame_order, uint32_t rpos, uint32_t s,
+                                        uint32_t nseg) {
+    const uint32_t slot = fused_seg_slot(f, frame_order, rpos, s);
+    g0 = fused_index_entry(f.seg_offset, slot);
+    g1 = fused_index_entry(f.seg_offset, slot + nseg * fused_seg_step(f));
   }
 };
 
@@ -443,10 +464,11 @@ struct SegmentWalkT {
   // (A matrix has fewer than 2^32 elements, so element and byte offsets are 32-bit numbers.)
   __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t col0,
                                            uint32_t seg_in_row, uint32_t rpos) {
-    gofs = fused_index_entry(f.seg_offset, seg_);
-    eofs = fused_index_entry(f.seg_offset, seg_ + 1);
-    c.state = fused_index_entry(f.seg_state, seg_);
-    end_state = fused_index_entry(f.seg_state, seg_ + 1);
+    const uint32_t slot = fused_seg_slot(f, seg_, rpos, seg_in_row), next = slot + fused_seg_step(f);
+    gofs = fused_index_entry(f.seg_offset, slot);
+    eofs = fused_index_entry(f.seg_offset, next);
+    c.state = fused_index_entry(f.seg_state, slot);
+    end_state = fused_index_entry(f.seg_state, next);
     // a uniform base plus a 32-bit lane offset: the loads then take their address from a scalar
     // pair and one vector register, and no 64-bit address is worked out per group
     raw_base = f.raw6;

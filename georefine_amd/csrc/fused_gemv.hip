@@ -47,12 +47,32 @@ int validate_fused_host(const grf_bctx_fused &f, const grf_fused_tiling &g, Tili
   auto bad = [&](const std::string &why) { return grf::set_error(GRF_BAD_ARGUMENT, std::string(who) + ": " + why); };
   if (int rc = check_fused_frame(f, g, who, use, false)) return rc;
   if (!seg_offset || !tile_rows || !tile_class) return bad("null array");
-  const uint64_t segs = (uint64_t)f.rows * f.segs_per_row;
+  const uint32_t spr = f.segs_per_row;
+  // entry s (0..spr: the last is the row's end) of a row, in the order the frame structure says
+  // the index has: the frame's own, or the blocked order of the residuals (fused_seg_slot)
+  const uint32_t B = f.raw_interleaved;
+  if (B && !row_pos) return bad("the blocked index order needs the rows' positions");
+  if (row_pos) {  // positions first: the index is read through them
+    const uint64_t limit = ((uint64_t)f.rows + 15) / 16 * 16 + 16ull * f.nr;  // every class may start on a multiple of 16
+    for (uint32_t row = 0; row < f.rows; ++row)
+      if (row_pos[row] >= limit) return bad("row " + std::to_string(row) + " has a position beyond the rows the order can hold");
+  }
+  auto entry = [&](uint32_t row, uint32_t s) -> uint32_t {
+    if (!B) return seg_offset[(uint64_t)row * spr + s];
+    const uint32_t q = row_pos[row], within = q % B;
+    return seg_offset[(uint64_t)(q - within) * (spr + 1) + (uint64_t)s * B + within];
+  };
   // the index: offsets never decrease, stay inside the stream and end on its length
-  if (seg_offset[0] < 4) return bad("the first segment starts behind the stream's four-byte initial state");
-  for (uint64_t i = 0; i < segs; ++i)
-    if (seg_offset[i] > seg_offset[i + 1]) return bad("segment offsets decrease at segment " + std::to_string(i));
-  if (seg_offset[segs] != f.main_n_bytes) return bad("the last index entry is not the stream's length");
+  uint32_t lowest = 0xFFFFFFFFu, highest = 0;
+  for (uint32_t row = 0; row < f.rows; ++row) {
+    for (uint32_t s = 0; s < spr; ++s)
+      if (entry(row, s) > entry(row, s + 1))
+        return bad("segment offsets decrease at segment " + std::to_string(s) + " of row " + std::to_string(row));
+    lowest = std::min(lowest, entry(row, 0));
+    highest = std::max(highest, entry(row, spr));
+  }
+  if (lowest < 4) return bad("the first segment starts behind the stream's four-byte initial state");
+  if (highest != f.main_n_bytes) return bad("the last index entry is not the stream's length");
   // the tiling: slots name rows of the matrix, every row once, one row class per tile
   const uint32_t k = use == kGemmTiling && g.k_parts > 1 ? g.k_parts : 1;
   if (g.n_tiles % k) return bad("tile count is not a multiple of k_parts");
@@ -75,10 +95,10 @@ int validate_fused_host(const grf_bctx_fused &f, const grf_fused_tiling &g, Tili
   // every stream piece a workgroup or wave stages fits the LDS reserved for it: from the
   // 16-byte aligned start of its first segment to the end of its last, plus the 8 bytes the
   // refill's window reads from the cursor on
-  const uint32_t spr = f.segs_per_row;
   const uint32_t lanes = use == kGemmTiling ? 4u : g.lanes_per_row;
+  std::vector<uint32_t> off(spr + 1);
   for (uint32_t row = 0; row < f.rows; ++row) {
-    const uint32_t *off = seg_offset + (uint64_t)row * spr;
+    for (uint32_t s = 0; s <= spr; ++s) off[s] = entry(row, s);
     // the GEMM's waves start a piece of four segments at any multiple of four inside a slab,
     // and a slab at any multiple of lanes_per_row
     for (uint32_t b = 0; b < spr; b += g.lanes_per_row)

@@ -127,7 +127,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
   // the first slab's byte range is two dependent global reads away (row, then offsets):
   // start them before the tables are copied so that the latencies overlap
   grf::PieceSpan span{0, 0};
-  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, min(P, f.segs_per_row));
+  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, rpos, 0, min(P, f.segs_per_row));
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
     if (b) __syncthreads();  // everyone is done with the previous slab's LDS data
@@ -154,7 +154,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
     if (row != grf::kNoRow) {
       a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
       if (b + 1 < g.n_slabs)  // the next slab's byte range, while this one is walked
-        span.fetch(f, seg_base + P, min(P, f.segs_per_row - first_seg - P));
+        span.fetch(f, seg_base + P, rpos, first_seg + P, min(P, f.segs_per_row - first_seg - P));
     }
     __syncthreads();
     if (walks) {
@@ -359,12 +359,13 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
   // (Loads in a branch that only some lanes take make the compiler wait for every load in
   // flight where the branch ends, so lanes without a row read the matrix's first entries and
   // discard them.)
-  auto span_of = [&](uint32_t b, uint32_t row, uint32_t &g0, uint32_t &g1) {
-    const uint32_t first_seg = b << logp;
-    const uint32_t seg_base = row == grf::kNoRow ? 0 : mul24(row, f.segs_per_row) + first_seg;
-    const uint32_t past = row == grf::kNoRow ? 0 : min(P, f.segs_per_row - first_seg);
-    g0 = grf::fused_index_entry(f.seg_offset, seg_base);
-    g1 = grf::fused_index_entry(f.seg_offset, seg_base + past);  // (no row: an empty range)
+  auto span_of = [&](uint32_t b, uint32_t row, uint32_t rpos, uint32_t &g0, uint32_t &g1) {
+    const bool any = row != grf::kNoRow;
+    const uint32_t first_seg = any ? b << logp : 0;
+    const uint32_t slot = grf::fused_seg_slot(f, any ? mul24(row, f.segs_per_row) + first_seg : 0, any ? rpos : 0, first_seg);
+    const uint32_t past = any ? min(P, f.segs_per_row - first_seg) : 0;
+    g0 = grf::fused_index_entry(f.seg_offset, slot);
+    g1 = grf::fused_index_entry(f.seg_offset, slot + past * grf::fused_seg_step(f));  // (no row: an empty range)
   };
   auto advance = [&](uint32_t &grp, uint32_t &b) {  // the unit nwaves further on
     uint32_t &major = by_slab ? b : grp, &minor = by_slab ? grp : b;
@@ -378,8 +379,8 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     const uint32_t slot0 = grp * rpw + rl;
     row = (wave < units && slot0 < R) ? g.tile_rows[tile * R + slot0] : grf::kNoRow;
     if (row >= f.rows) row = grf::kNoRow;  // an empty slot, or a row the matrix does not have
-    span_of(b, row, g0, g1);
     rpos = row_position(f, row);
+    span_of(b, row, rpos, g0, g1);
   }
   for (uint32_t i = tid; i < R; i += nthreads) {
     uint32_t rw = g.tile_rows[tile * R + i];
@@ -424,7 +425,8 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     {  // the next unit's byte range, on its way during this unit's walk
       advance(grp, b);
       const uint32_t sn = grp * rpw + rl;
-      span_of(b, (u + nwaves < units && sn < R) ? rows[sn] : grf::kNoRow, g0, g1);
+      const bool more = u + nwaves < units && sn < R;
+      span_of(b, more ? rows[sn] : grf::kNoRow, more ? rows[R + sn] : 0, g0, g1);
     }
     __builtin_amdgcn_wave_barrier();
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -841,9 +843,10 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   auto span_of = [&](uint32_t b, uint32_t &g0, uint32_t &g1) {
     const uint32_t first = b * P + quad * 4;
     const bool any = row != grf::kNoRow && first < f.segs_per_row && quad * 4 < P;
-    const uint32_t base = any ? mul24(row, f.segs_per_row) + first : 0;
-    g0 = grf::fused_index_entry(f.seg_offset, base);
-    g1 = grf::fused_index_entry(f.seg_offset, base + (any ? min(4u, min(P - quad * 4, f.segs_per_row - first)) : 0));
+    const uint32_t slot = grf::fused_seg_slot(f, any ? mul24(row, f.segs_per_row) + first : 0, any ? rpos : 0, any ? first : 0);
+    const uint32_t past = any ? min(4u, min(P - quad * 4, f.segs_per_row - first)) : 0;
+    g0 = grf::fused_index_entry(f.seg_offset, slot);
+    g1 = grf::fused_index_entry(f.seg_offset, slot + past * grf::fused_seg_step(f));
   };
   uint32_t g0, g1;
   span_of(b_first, g0, g1);  // started before the table copy so that the latencies overlap

@@ -327,3 +327,31 @@ def test_host_validator_accepts_planned_tilings_and_names_what_is_wrong():
     shared[1] = shared[0]
     refused("share residual position", row_pos=shared, block=block)
     refused("interleaved residual order", row_pos=position, block=0)
+
+
+@pytest.mark.parametrize("rows,spr,block", [(37, 5, 4), (64, 80, 16), (10, 272, 2), (3, 1, 1), (100, 17, 8)])
+def test_index_in_the_blocked_order_keeps_every_checkpoint_and_each_rows_end(rows, spr, block):
+    """``order_index``: entry s of the row at position q lies at ((q // B) * (spr + 1) + s) * B + q % B
+    (the rule the kernels use, ``fused_seg_slot``), s = spr being the end of the row's stream,
+    which in the frame's order is the next row's first entry."""
+    rng = np.random.default_rng(rows * spr)
+    frame_order = np.cumsum(rng.integers(1, 50, size=rows * spr + 1)).astype(np.uint32)
+    classes = rng.integers(0, 4, size=rows)
+    order = np.argsort(classes, kind="stable")
+    position = np.empty(rows, dtype=np.uint32)
+    at = 0
+    for c in range(4):  # every class starts on a multiple of 16, as FramePlan.residual_order has it
+        members = order[classes[order] == c]
+        position[members] = at + np.arange(members.size)
+        at = -(-(at + members.size) // 16) * 16
+    held = max(-(-at // block) * block, block)
+    ordered = _fused.order_index(frame_order, rows, spr, block, position, held)
+    assert ordered.size == held * (spr + 1) and ordered.dtype == frame_order.dtype
+    q = position.astype(np.int64)
+    for s in (0, 1, spr // 2, spr - 1, spr):
+        slot = ((q // block) * (spr + 1) + s) * block + q % block
+        assert np.array_equal(ordered[slot], frame_order[np.arange(rows) * spr + s]), s
+    used = np.zeros(ordered.size, dtype=bool)
+    for s in range(spr + 1):
+        used[((q // block) * (spr + 1) + s) * block + q % block] = True
+    assert not ordered[~used].any()  # positions that no row has hold zeros

@@ -71,7 +71,7 @@ def test_gemm_checkpoint_mismatch_sets_error(oracle):
     from georefine_amd import bitexact_context_codec as codec
     words = weight_like(np.random.default_rng(29), 64, 512)
     frame, t = _tensor(words)
-    t.buffers["fused_seg_state"].view(torch.int32)[7] += 1  # forced from the host; the kernel finishes normally
+    t.buffers["fused_seg_state"].view(torch.int32)[t.index_slot(0, 1)] += 1  # forced from the host; the kernel finishes normally
     x = torch.zeros(32, 512, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(codec.CodecError):
         t.gemm(x, check=True)

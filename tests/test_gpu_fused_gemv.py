@@ -111,7 +111,7 @@ def test_fused_checkpoint_mismatch_sets_error(oracle):
     from georefine_amd import bitexact_context_codec as codec
     words = weight_like(np.random.default_rng(23), 64, 512)
     frame, t = _tensor(words)
-    t.buffers["fused_seg_state"].view(torch.int32)[5] += 1  # forced from the host; the kernel finishes normally
+    t.buffers["fused_seg_state"].view(torch.int32)[t.index_slot(2, 1)] += 1  # forced from the host; the kernel finishes normally
     x = torch.zeros(1, 512, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(codec.CodecError):
         t.linear(x, check=True)
@@ -178,7 +178,6 @@ def test_residual_order_fields_are_checked_and_any_block_size_decodes(oracle):
     blocks of 1, 2, 4, 8 or 16 rows gives the same words and products through every kernel; a
     block size that is not one of those, or positions without the interleaved order, are refused
     before anything is launched."""
-    import copy
     import ctypes
     import torch
     from georefine_amd import _fused
@@ -191,14 +190,16 @@ def test_residual_order_fields_are_checked_and_any_block_size_decodes(oracle):
     want_v, want_m = t.gemv(x[:2], check=True), t.gemm(x, check=True)
     indexed = index_frame(frame, 1024, fused_segment=t.fused_plan["seg_len"], raw6_residual=True)
     block0, position, held = t._plan.residual_order()
+    spr = 1024 // t.fused_plan["seg_len"]
     for block in (1, 2, 4, 8, 16):
-        other = copy.copy(t)
-        other.buffers = dict(t.buffers)
+        # the copy's arrays, re-ordered on the device, are what the host-side ordering gives
+        other = t.clone(residual_block=block)
         ordered = _fused.order_residuals(indexed["residual_stream"], 104, 1024, t.fused_plan["seg_len"], block,
                                          position, held)
-        other.buffers["residual_stream"] = torch.from_numpy(ordered).cuda()
-        other._raw6_block = block
-        other._bind()
+        assert np.array_equal(other.buffers["residual_stream"].cpu().numpy()[:ordered.size], ordered), block
+        for name, values in (("fused_seg_state", t._plan.seg_state), ("fused_seg_offset", t._plan.seg_offset)):
+            assert np.array_equal(other.buffers[name].cpu().numpy(),
+                                  _fused.order_index(values, 104, spr, block, position, held)), (name, block)
         assert other.fused.raw_interleaved == block
         assert np.array_equal(other.decode().view(torch.uint16).cpu().numpy(), words), block
         assert np.array_equal(other.decode(general=True).view(torch.uint16).cpu().numpy(), words), block

@@ -76,7 +76,7 @@ def test_group_reports_a_member_that_misses_its_checkpoints_and_rejects_mismatch
     group = HipLinearGroup(tensors)
     x = torch.zeros(1, 512, dtype=torch.bfloat16, device="cuda")
     group.linear(x, check=True)
-    tensors[1].buffers["fused_seg_state"].view(torch.int32)[3] += 1  # forced from the host; kernels finish normally
+    tensors[1].buffers["fused_seg_state"].view(torch.int32)[tensors[1].index_slot(1, 1)] += 1  # forced from the host; kernels finish normally
     with pytest.raises(codec.CodecError):
         group.linear(x, check=True)
     with pytest.raises(codec.CodecError):
@@ -137,7 +137,7 @@ def test_predictive_group_products():
     for i, y in enumerate(group.linear(x, biases, check=True)):  # above 128 rows: the members' own route
         assert close(y, i, 140), i
     assert group.linear(x[:0], biases)[1].shape == (0, 72)
-    members[1].buffers["fused_seg_state"].view(torch.int32)[3] += 1  # forced from the host; kernels finish normally
+    members[1].buffers["fused_seg_state"].view(torch.int32)[members[1].index_slot(1, 1)] += 1  # forced from the host; kernels finish normally
     with pytest.raises(ppcx.CodecError):
         group.linear(x[:1], biases, check=True)
     with pytest.raises(ppcx.CodecError):
