@@ -361,13 +361,20 @@ __device__ __forceinline__ void fused_load_tables(uint8_t *lds, uint32_t blocks,
 // of its stream -- and entry s of position q lies at ((q / B) * (segs_per_row + 1) + s) * B + q % B:
 // the entries that a wave unit, or the sixteen rows of a GEMM wave, read at one visit are then
 // one run of bytes, as its residuals are, instead of a few bytes out of every row's own line.
-// `frame_order`: the segment's number in the frame's order, rpos: the row's position, s: the
-// segment in its row.  The entry of the segment's end is fused_seg_step further on.
-__device__ __forceinline__ uint32_t fused_seg_slot(const grf_bctx_fused &f, uint32_t frame_order, uint32_t rpos,
-                                                   uint32_t s) {
-  if (!f.raw_interleaved) return frame_order;
+// `row`, rpos: the row and its position, s: the segment in its row.  The entry of the
+// segment's end is fused_seg_step further on.  NARROW: rows and segments per row are below
+// 2^24 (wave tilings), so the products take the full-rate 24-bit multiply.
+template <bool NARROW = false>
+__device__ __forceinline__ uint32_t fused_seg_slot(const grf_bctx_fused &f, uint32_t row, uint32_t rpos, uint32_t s) {
+  auto mul = [](uint32_t a, uint32_t b) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (NARROW) return (uint32_t)__umul24(a, b);
+#endif
+    return a * b;
+  };
+  if (!f.raw_interleaved) return mul(row, f.segs_per_row) + s;
   const uint32_t B = f.raw_interleaved, within = rpos & (B - 1);
-  return (rpos - within) * (f.segs_per_row + 1) + s * B + within;
+  return mul(rpos - within, f.segs_per_row + 1) + mul(s, B) + within;
 }
 __device__ __forceinline__ uint32_t fused_seg_step(const grf_bctx_fused &f) {
   return f.raw_interleaved ? f.raw_interleaved : 1u;
@@ -378,9 +385,9 @@ __device__ __forceinline__ uint32_t fused_seg_step(const grf_bctx_fused &f) {
 // slab's bytes can be copied.
 struct PieceSpan {
   uint32_t g0, g1;
-  __device__ __forceinline__ void fetch(const grf_bctx_fused &f, uint32_t frame_order, uint32_t rpos, uint32_t s,
+  __device__ __forceinline__ void fetch(const grf_bctx_fused &f, uint32_t row, uint32_t rpos, uint32_t s,
                                         uint32_t nseg) {
-    const uint32_t slot = fused_seg_slot(f, frame_order, rpos, s);
+    const uint32_t slot = fused_seg_slot(f, row, rpos, s);
     g0 = fused_index_entry(f.seg_offset, slot);
     g1 = fused_index_entry(f.seg_offset, slot + nseg * fused_seg_step(f));
   }
@@ -457,14 +464,15 @@ struct SegmentWalkT {
   Raw6x16 rr;      // the group being decoded
   uint32_t cw[4];
 
-  // Global reads for segment `seg_` (elem0 / col0: its first element / column; seg_in_row =
-  // col0 / seg_len, which the caller has without dividing; rpos: the row's position in the
-  // residual array, f.row_pos[row] or the row itself), issued before the wait for the stream
-  // bytes so that their latency overlaps it.
+  // Global reads for the segment whose checkpoint is entry `slot_` of the index arrays
+  // (fused_seg_slot; elem0 / col0: its first element / column; seg_in_row = col0 / seg_len,
+  // which the caller has without dividing; rpos: the row's position in the residual array,
+  // f.row_pos[row] or the row itself), issued before the wait for the stream bytes so that
+  // their latency overlaps it.
   // (A matrix has fewer than 2^32 elements, so element and byte offsets are 32-bit numbers.)
-  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t col0,
+  __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t slot_, uint32_t elem0, uint32_t col0,
                                            uint32_t seg_in_row, uint32_t rpos) {
-    const uint32_t slot = fused_seg_slot(f, seg_, rpos, seg_in_row), next = slot + fused_seg_step(f);
+    const uint32_t slot = slot_, next = slot + fused_seg_step(f);
     gofs = fused_index_entry(f.seg_offset, slot);
     eofs = fused_index_entry(f.seg_offset, next);
     c.state = fused_index_entry(f.seg_state, slot);

@@ -127,7 +127,7 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
   // the first slab's byte range is two dependent global reads away (row, then offsets):
   // start them before the tables are copied so that the latencies overlap
   grf::PieceSpan span{0, 0};
-  if (row != grf::kNoRow) span.fetch(f, row * f.segs_per_row, rpos, 0, min(P, f.segs_per_row));
+  if (row != grf::kNoRow) span.fetch(f, row, rpos, 0, min(P, f.segs_per_row));
   grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
   for (uint32_t b = 0; b < g.n_slabs; ++b) {
     if (b) __syncthreads();  // everyone is done with the previous slab's LDS data
@@ -145,16 +145,15 @@ __device__ __forceinline__ void fused_walk_body(uint8_t *lds, const grf_bctx_fus
     const uint32_t nseg = min(P, f.segs_per_row - first_seg);
     const uint32_t piece_off = L.stream + r * g.piece_cap;
     const bool walks = row != grf::kNoRow && p < nseg;
-    const uint32_t seg_base = row != grf::kNoRow ? row * f.segs_per_row + first_seg : 0;
     const uint32_t col0 = (first_seg + p) * S;
     const uint64_t elem0 = (uint64_t)row * K + col0;
     Walk w;
     uint32_t a0 = 0;
-    if (walks) w.prefetch(f, seg_base + p, (uint32_t)elem0, col0, first_seg + p, rpos);
+    if (walks) w.prefetch(f, grf::fused_seg_slot(f, row, rpos, first_seg + p), (uint32_t)elem0, col0, first_seg + p, rpos);
     if (row != grf::kNoRow) {
       a0 = grf::fused_stage_piece(lds, piece_off, f, span, p, P);
       if (b + 1 < g.n_slabs)  // the next slab's byte range, while this one is walked
-        span.fetch(f, seg_base + P, rpos, first_seg + P, min(P, f.segs_per_row - first_seg - P));
+        span.fetch(f, row, rpos, first_seg + P, min(P, f.segs_per_row - first_seg - P));
     }
     __syncthreads();
     if (walks) {
@@ -359,13 +358,14 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
   // (Loads in a branch that only some lanes take make the compiler wait for every load in
   // flight where the branch ends, so lanes without a row read the matrix's first entries and
   // discard them.)
+  const uint32_t seg_step = grf::fused_seg_step(f);
   auto span_of = [&](uint32_t b, uint32_t row, uint32_t rpos, uint32_t &g0, uint32_t &g1) {
     const bool any = row != grf::kNoRow;
     const uint32_t first_seg = any ? b << logp : 0;
-    const uint32_t slot = grf::fused_seg_slot(f, any ? mul24(row, f.segs_per_row) + first_seg : 0, any ? rpos : 0, first_seg);
+    const uint32_t slot = grf::fused_seg_slot<true>(f, any ? row : 0, any ? rpos : 0, first_seg);
     const uint32_t past = any ? min(P, f.segs_per_row - first_seg) : 0;
     g0 = grf::fused_index_entry(f.seg_offset, slot);
-    g1 = grf::fused_index_entry(f.seg_offset, slot + past * grf::fused_seg_step(f));  // (no row: an empty range)
+    g1 = grf::fused_index_entry(f.seg_offset, slot + mul24(past, seg_step));  // (no row: an empty range)
   };
   auto advance = [&](uint32_t &grp, uint32_t &b) {  // the unit nwaves further on
     uint32_t &major = by_slab ? b : grp, &minor = by_slab ? grp : b;
@@ -417,7 +417,7 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     const uint32_t a0 = grf::fused_stage_piece_dma(lds, L.stream + wave * rpw * g.piece_cap, g.piece_cap, f, g0, g1, lane, logp, rpw);
     Walk w;
     {  // every lane loads (see span_of); lanes that do not walk read segment 0's entries
-      const uint32_t seg = walks ? mul24(row, f.segs_per_row) + first_seg + p : 0;
+      const uint32_t seg = grf::fused_seg_slot<true>(f, walks ? row : 0, walks ? rpos : 0, walks ? first_seg + p : 0);
       w.prefetch(f, seg, walks ? mul24(row, K) + col0 : 0, walks ? col0 : 0, walks ? first_seg + p : 0, walks ? rpos : 0);
     }
     if (walks) w.start(piece_off, a0);
@@ -843,10 +843,10 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   auto span_of = [&](uint32_t b, uint32_t &g0, uint32_t &g1) {
     const uint32_t first = b * P + quad * 4;
     const bool any = row != grf::kNoRow && first < f.segs_per_row && quad * 4 < P;
-    const uint32_t slot = grf::fused_seg_slot(f, any ? mul24(row, f.segs_per_row) + first : 0, any ? rpos : 0, any ? first : 0);
+    const uint32_t slot = grf::fused_seg_slot<true>(f, any ? row : 0, any ? rpos : 0, any ? first : 0);
     const uint32_t past = any ? min(4u, min(P - quad * 4, f.segs_per_row - first)) : 0;
     g0 = grf::fused_index_entry(f.seg_offset, slot);
-    g1 = grf::fused_index_entry(f.seg_offset, slot + past * grf::fused_seg_step(f));
+    g1 = grf::fused_index_entry(f.seg_offset, slot + mul24(past, grf::fused_seg_step(f)));
   };
   uint32_t g0, g1;
   span_of(b_first, g0, g1);  // started before the table copy so that the latencies overlap
@@ -872,7 +872,7 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
     const uint32_t a0 = grf::fused_stage_piece_dma(lds, region, g.piece_cap, f, g0, g1, lane, 0, 16);
     Walk w;
     {
-      const uint32_t seg = active ? mul24(row, f.segs_per_row) + first_seg + p4 : 0;
+      const uint32_t seg = grf::fused_seg_slot<true>(f, active ? row : 0, active ? rpos : 0, active ? first_seg + p4 : 0);
       w.prefetch(f, seg, active ? mul24(row, K) + col0 : 0, active ? col0 : 0, active ? first_seg + p4 : 0, active ? rpos : 0);
     }
     if (active) w.start(piece_off, a0);  // (a0: of the lane's own row, which its four lanes share)

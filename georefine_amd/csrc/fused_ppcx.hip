@@ -142,7 +142,7 @@ struct PpcxWalk {
   // global reads of the segment, issued before the wait for the slab's stream bytes
   __device__ __forceinline__ void prefetch(const grf_bctx_fused &f, uint32_t seg_, uint32_t elem0, uint32_t,
                                            uint32_t seg_in_row, uint32_t rpos) {
-    const uint32_t slot = grf::fused_seg_slot(f, seg_, rpos, seg_in_row), next = slot + grf::fused_seg_step(f);
+    const uint32_t slot = seg_, next = slot + grf::fused_seg_step(f);  // (seg_: the entry, fused_seg_slot)
     gofs = grf::fused_index_entry(f.seg_offset, slot);
     eofs = grf::fused_index_entry(f.seg_offset, next);
     c.state = grf::fused_index_entry(f.seg_state, slot);
