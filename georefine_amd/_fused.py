@@ -474,6 +474,46 @@ def build_balanced_tiles(row_class, nr, unit_rows, slots, max_rows):
     return np.concatenate(out_rows), np.asarray(out_class, dtype=np.uint8), tallest
 
 
+GEMM_BALANCE = os.environ.get("GEOREFINE_GEMM_BALANCE", "3")  # "0": tiles of one height (experiments)
+
+
+def build_gemm_tiles(row_class, nr, r, first_tile=0, lead=0, cus=256):
+    """Row tiles of the matrix-core kernel: (tile_rows, tile_class, R, tall tiles).
+
+    A wave of that kernel holds a block of sixteen rows and issues the same instructions
+    whether the block is full or holds four rows, so tiles cut at one height r that is not a
+    multiple of 16 (68 rows: four blocks and a quarter) pay for a block they barely use.  The
+    same number of tiles is cut in whole blocks instead, heights differing by one block (of
+    1088 rows in 16 tiles: four tiles of 80 rows and twelve of 64), wherever that pays for
+    fewer blocks; waves whose block is empty leave at once.  The tall tiles then decide the
+    launch's length, so they should not share a compute unit: with every tile resident at
+    once, workgroup i and workgroup i + cus land on the same unit, and the tall tiles are
+    placed so that their launch positions (``first_tile`` + index) differ modulo ``cus``,
+    starting at position ``lead`` (the tall tiles other members of a grouped launch have
+    placed already)."""
+    tile_rows, tile_class = build_tiles(row_class, nr, r)
+    blocks = -(-r // 16)
+    paid = lambda rows_, height: int(((rows_.reshape(-1, height) != 0xFFFFFFFF).sum(axis=1) + 15).__floordiv__(16).sum())
+    if GEMM_BALANCE == "0" or r % 16 == 0:
+        return tile_rows, tile_class, r, 0
+    even = build_balanced_tiles(row_class, nr, 16, len(tile_class), 16 * blocks)
+    if even is None or paid(even[0], even[2]) >= paid(tile_rows, r):
+        return tile_rows, tile_class, r, 0
+    tile_rows, tile_class, r = even
+    table = tile_rows.reshape(-1, r)
+    height = ((table != 0xFFFFFFFF).sum(axis=1) + 15) // 16
+    tall = height == height.max()
+    n_tall = int(tall.sum()) if height.max() > height.min() else 0
+    if n_tall and GEMM_BALANCE != "1":
+        tall_at, short_at = np.flatnonzero(tall), np.flatnonzero(~tall)
+        start = (lead - first_tile) % cus if GEMM_BALANCE == "3" else 0
+        if start + n_tall > len(tile_class) or start > len(short_at):
+            start = 0
+        order = np.concatenate((short_at[:start], tall_at, short_at[start:]))
+        table, tile_class = table[order], tile_class[order]
+    return np.ascontiguousarray(table).reshape(-1), tile_class, r, n_tall
+
+
 class FramePlan:
     """Frame-level derived arrays (shared by every tiling) and a tiling factory."""
 
@@ -600,8 +640,10 @@ class FramePlan:
             self.spr, self.class_rows, lambda lanes: self.quad_cap(),
             lambda p_, r_, cap_: lds_bytes_gemm(self.nc, self.lognb, self.tabn, p_, r_, cap_),
             seg_len=self.seg_len, table_bytes=self.table_bytes(), split=GEMM_SPLIT)
-        tile_rows, tile_class = build_tiles(self.row_class, self.nr, r)  # the row tiles; the launch has k of each
-        assert len(tile_class) * k == n_tiles
+        # the row tiles; the launch has k of each
+        tile_rows, tile_class, r, _ = build_gemm_tiles(self.row_class, self.nr, r)
+        n_tiles = len(tile_class) * k
+        lds = lds_bytes_gemm(self.nc, self.lognb, self.tabn, p, r, cap)
         return dict(tile_rows=tile_rows, tile_class=tile_class,
                     scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=r, n_slabs=n_slabs,
                                  n_tiles=n_tiles, piece_cap=cap, scheme=SCHEME_WAVES, k_parts=k), lds=lds)
@@ -640,6 +682,22 @@ def plan_group(plans, m=None, gemm=False, waves=False):
         threads, p, r, n_slabs, _, cap, lds = choose_tiling(first.spr, class_rows, cap_fn, lds_fn,
                                                             seg_len=first.seg_len, table_bytes=table)
     tilings = []
+    if gemm:  # whole blocks of sixteen rows per tile; one slot stride and LDS demand for all members
+        cut, at, lead = [], 0, 0
+        for pl in plans:
+            cut.append(build_gemm_tiles(pl.row_class, pl.nr, r, first_tile=at, lead=lead))
+            at, lead = at + len(cut[-1][1]), lead + cut[-1][3]
+        height = max(c[2] for c in cut)
+        lds = lds_fn(p, height, cap)
+        for tile_rows, tile_class, r_, _ in cut:
+            if r_ != height:  # (a member the cut did not pay for: its slots widened to the common stride)
+                wide = np.full((len(tile_class), height), 0xFFFFFFFF, dtype=np.uint32)
+                wide[:, :r_] = tile_rows.reshape(-1, r_)
+                tile_rows = wide.reshape(-1)
+            tilings.append(dict(tile_rows=tile_rows, tile_class=tile_class,
+                                scalars=dict(threads=threads, lanes_per_row=p, rows_per_tile=height, n_slabs=n_slabs,
+                                             n_tiles=len(tile_class), piece_cap=cap, scheme=scheme), lds=lds))
+        return tilings
     for pl in plans:
         tile_rows, tile_class = build_tiles(pl.row_class, pl.nr, r)
         tilings.append(dict(tile_rows=tile_rows, tile_class=tile_class,

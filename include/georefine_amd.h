@@ -170,8 +170,11 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
 /* A BCTX frame prepared for the fused kernels: main rANS stream as in the frame,
  * residuals in the packed 6-bit form, segments of a length that divides the row
  * length, and per-row-class lookup tables laid out for LDS:
- *   seg_state / seg_offset  u32 [rows*segs_per_row + 1]; the extra last entry is
- *                           (2^23, main_n_bytes)
+ *   seg_state / seg_offset  the checkpoint index: rANS state and stream offset at the start
+ *                           of every segment.  With raw_interleaved == 0: u32
+ *                           [rows*segs_per_row + 1] in the frame's order; the extra last
+ *                           entry is (2^23, main_n_bytes).  With raw_interleaved == B: in
+ *                           the blocked order of the residuals (below)
  *   lut         u8  [nr][nc << lognb]        lognb = 16 - shift; sparse index of a
  *                                            symbol with slots in the bucket (best: the
  *                                            one owning most of them)
@@ -186,6 +189,12 @@ int grf_mix_predict(const uint16_t *up, const uint16_t *gate, const uint16_t *co
  * lies at (((q / B * G + t) * segs_per_row + s) * B + q % B) * 12.  The lanes of a wave unit
  * of the GEMV (B = 64 / lanes_per_row rows, at the same position of neighbouring segments)
  * then read one run of 768 bytes per visit, and every 128-byte line is used in a single visit.
+ * The index arrays follow the same order: every row holds segs_per_row + 1 entries (the last
+ * one the end of its last segment: the start of the next row's first in the frame's order, or
+ * (2^23, main_n_bytes)), and entry s of the row at position q lies at
+ * ((q / B) * (segs_per_row + 1) + s) * B + q % B, so that the B rows of a unit find their
+ * checkpoints side by side; the arrays hold (rows held) * (segs_per_row + 1) entries, and
+ * entries of positions no row has are never read.
  * row_pos: u32 [rows], a one-to-one map of the rows to positions below
  * ceil(max position / B) * B (the array holds that many rows; positions no row has are never
  * read).  The host side orders the rows by row class, as the tilings do, and starts every
@@ -270,8 +279,10 @@ int grf_bctx_gemv(const grf_bctx_fused *frame, const grf_fused_tiling *tiling, c
  * points check the scalars of the two structures on every call; what the kernels take on
  * trust from the arrays behind them is checked here, on HOST copies of those arrays (the
  * structures' own pointers are device addresses and are not read; they may be null):
- *   seg_offset  u32 [rows*segs_per_row + 1]: never decreasing, first entry >= 4, last entry
- *               == main_n_bytes (a kernel copies [offset[s] & ~15, offset[s + lanes]) to LDS)
+ *   seg_offset  in the order frame->raw_interleaved declares (the frame's: rows*segs_per_row
+ *               + 1 entries; blocked: the rows held times segs_per_row + 1, row_pos required):
+ *               never decreasing along a row, no entry below 4, the highest == main_n_bytes
+ *               (a kernel copies [offset[s] & ~15, offset[s + lanes]) to LDS)
  *   tile_rows / tile_class  as in grf_fused_tiling (for k_parts > 1: the n_tiles / k_parts row
  *               tiles): slots name rows of the matrix, every row exactly once (use 3: any rows,
  *               any number of times), classes below nr
@@ -382,7 +393,8 @@ uint32_t grf_bctx_fused_lds_bytes(const grf_bctx_fused *frame, const grf_fused_t
  * seg_len / 32, record t of segment s lies at index ((q / B * U + t) * segs_per_row + s) * B +
  * q % B -- the order grf_bctx_fused gives its 12-byte groups, for the same reason: the lanes of
  * a wave unit then read one run of bytes per visit.  grf_ppcx_bins_ordered writes a plane in
- * that order. */
+ * that order.  seg_state / seg_offset are then in the blocked order as well, exactly as
+ * grf_bctx_fused describes it (segs_per_row + 1 entries per row). */
 typedef struct grf_ppcx_fused {
   const uint8_t *main_bytes;
   const uint8_t *raw5;
