@@ -448,7 +448,7 @@ def build_balanced_tiles(row_class, nr, unit_rows, slots, max_rows):
     tiles = {rho: 1 for rho in live}
     height = lambda rho: -(-units[rho] // tiles[rho])
     for _ in range(slots - len(live)):  # the next tile to the class whose tiles are tallest
-        rho = max(live, key=lambda c: (height(c), units[c]))
+        rho = max(live, key=lambda c: (height(c), units[c] / tiles[c]))  # (among equals: the fullest tiles)
         if height(rho) <= 1:
             break
         tiles[rho] += 1

@@ -812,7 +812,9 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   const uint32_t tid = threadIdx.x, nthreads = blockDim.x;
   const uint32_t P = g.lanes_per_row, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t parts = g.k_parts > 1 ? g.k_parts : 1u, row_tiles = g.n_tiles / parts;
-  const uint32_t part = launch_tile / row_tiles, tile = launch_tile - part * row_tiles;  // (uniform: scalar divisions)
+  // (uniform: scalar divisions.  Part-major: with a tile's copies side by side instead, the same
+  // launch at six rows took 5 % longer on 5120 x 17408 cut in three)
+  const uint32_t part = launch_tile / row_tiles, tile = launch_tile - part * row_tiles;
   const uint32_t per_part = (g.n_slabs + parts - 1) / parts;
   const uint32_t b_first = part * per_part, b_past = min(g.n_slabs, b_first + per_part);
   const uint32_t cls = g.tile_class[tile];

@@ -355,3 +355,28 @@ def test_index_in_the_blocked_order_keeps_every_checkpoint_and_each_rows_end(row
     for s in range(spr + 1):
         used[((q // block) * (spr + 1) + s) * block + q % block] = True
     assert not ordered[~used].any()  # positions that no row has hold zeros
+
+
+def test_matrix_core_row_tiles_come_in_whole_blocks_and_spread_the_tall_ones():
+    """Rows that come 1088 to a class, cut into 16 tiles per class: 68 rows each would pay for
+    five blocks of sixteen per tile; the planner cuts four tiles of 80 and twelve of 64 instead
+    and places the tall ones where no two meet modulo the compute units."""
+    rng = np.random.default_rng(5)
+    row_class = np.repeat(np.arange(16), 1088).astype(np.uint8)
+    rng.shuffle(row_class)
+    placed = []
+    for first, lead in ((0, 0), (256, 64)):
+        tile_rows, tile_class, height, tall = _fused.build_gemm_tiles(row_class, 16, 68, first_tile=first, lead=lead)
+        table = tile_rows.reshape(-1, height)
+        held = table != 0xFFFFFFFF
+        assert (height, tall, len(tile_class)) == (80, 64, 256)
+        assert sorted(table[held].tolist()) == list(range(row_class.size))
+        assert all((row_class[row[keep]] == cls).all() for row, keep, cls in zip(table, held, tile_class))
+        assert set(held.sum(axis=1).tolist()) == {64, 80} and held[:, ::-1].cumsum(axis=1).min() >= 0
+        assert (np.diff(held.astype(np.int8), axis=1) <= 0).all()  # a tile's empty slots are at its end
+        placed += [(first + i) % 256 for i in np.flatnonzero(held.sum(axis=1) == 80)]
+    assert sorted(placed) == list(range(128))
+    # a height that is a multiple of sixteen already, or rows that do not profit: tiles as before
+    plain = _fused.build_tiles(row_class, 16, 64)
+    same = _fused.build_gemm_tiles(row_class, 16, 64)
+    assert same[2:] == (64, 0) and (same[0] == plain[0]).all() and (same[1] == plain[1]).all()
