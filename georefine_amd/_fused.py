@@ -629,7 +629,7 @@ class FramePlan:
 
     def _wave_limits(self):
         """Kernels over wave tilings address rows and segments with 24-bit multiplies."""
-        if self.rows >= 1 << 24 or self.cols >= 1 << 24:
+        if self.rows + 16 + 16 * self.nr >= 1 << 24 or self.cols >= 1 << 24:  # (row positions stay below 2^24 too)
             raise FusedUnsupported("wave tilings take fewer than 2^24 rows and columns")
 
     def gemm_tiling(self):

@@ -12,7 +12,9 @@ int check_fused_frame(const grf_bctx_fused &f, const grf_fused_tiling &g, const 
   if (f.seg_len == 0 || f.seg_len % 16 || (uint64_t)f.seg_len * f.segs_per_row != f.cols)
     return bad("segment length must be a multiple of 16 that divides the row length");
   if (!g.threads || g.threads % 64 || g.threads > (uint32_t)grf::kFusedMaxThreads) return bad("thread count");
-  if ((use == kGemmTiling || g.scheme == GRF_TILE_WAVES) && (f.rows >= (1u << 24) || f.cols >= (1u << 24)))
+  // (row positions too stay below 2^24: they go up to the rows rounded up to 16, plus 16 per row class)
+  if ((use == kGemmTiling || g.scheme == GRF_TILE_WAVES) &&
+      ((uint64_t)f.rows + 16 + 16ull * f.nr >= (1u << 24) || f.cols >= (1u << 24)))
     return grf::set_error(GRF_UNSUPPORTED, std::string(who) + ": wave tilings take fewer than 2^24 rows and columns");
   if (use == kGemmTiling) {  // waves of 16 rows x 4 segments with their own stream pieces
     if (g.scheme != GRF_TILE_WAVES) return bad("the GEMM takes a wave tiling (piece_cap for pieces of four segments)");

@@ -380,3 +380,14 @@ def test_matrix_core_row_tiles_come_in_whole_blocks_and_spread_the_tall_ones():
     plain = _fused.build_tiles(row_class, 16, 64)
     same = _fused.build_gemm_tiles(row_class, 16, 64)
     assert same[2:] == (64, 0) and (same[0] == plain[0]).all() and (same[1] == plain[1]).all()
+
+
+def test_wave_tilings_refuse_matrices_whose_row_positions_would_pass_24_bits():
+    """The wave bodies multiply rows and row positions with 24-bit multiplies; positions go up
+    to the rows rounded up to 16 plus 16 per row class."""
+    from types import SimpleNamespace
+    _fused.FramePlan._wave_limits(SimpleNamespace(rows=(1 << 24) - 16 - 16 * 16 - 1, cols=64, nr=16))
+    with pytest.raises(_fused.FusedUnsupported):
+        _fused.FramePlan._wave_limits(SimpleNamespace(rows=(1 << 24) - 16 - 16 * 16, cols=64, nr=16))
+    with pytest.raises(_fused.FusedUnsupported):
+        _fused.FramePlan._wave_limits(SimpleNamespace(rows=64, cols=1 << 24, nr=16))
