@@ -497,7 +497,9 @@ def build_gemm_tiles(row_class, nr, r, first_tile=0, lead=0, cus=256):
     if GEMM_BALANCE == "0" or r % 16 == 0:
         return tile_rows, tile_class, r, 0
     even = build_balanced_tiles(row_class, nr, 16, len(tile_class), 16 * blocks)
-    if even is None or paid(even[0], even[2]) >= paid(tile_rows, r):
+    # (as many tiles as planned: tiles shorter than a block that spread a small matrix over the
+    # workgroup slots stay as they are)
+    if even is None or len(even[1]) != len(tile_class) or paid(even[0], even[2]) >= paid(tile_rows, r):
         return tile_rows, tile_class, r, 0
     tile_rows, tile_class, r = even
     table = tile_rows.reshape(-1, r)

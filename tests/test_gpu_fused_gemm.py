@@ -170,3 +170,34 @@ def test_gemm_cut_along_k(oracle, monkeypatch, shape, forced):
     assert lib.grf_bctx_gemm(*args, space.data_ptr(), need, t.error.data_ptr(), stream) == 0
     torch.cuda.synchronize()
     assert torch.equal(y.view(torch.uint16), y_all[:64].view(torch.uint16))
+
+
+def test_row_tiles_in_whole_blocks_leave_every_bit_as_it_was(monkeypatch):
+    """The planner cuts the matrix-core row tiles in whole blocks of sixteen rows, some a block
+    taller than others, and moves the tall ones about the launch; a row's sum only depends on
+    the lanes per row and the cut along K, so the products keep their bits -- alone and in a
+    grouped launch -- against tiles of one height."""
+    import torch
+    from georefine_amd import _fused
+    from georefine_amd.bitexact_context_gpu import HipLinearGroup
+    rng = np.random.default_rng(77)
+    # 2176 rows in 16 classes: 136 to a class = 8.5 blocks of sixteen; tiles of 20 rows asked for
+    # (a matrix this small would get tiles shorter than a block, which are left alone)
+    words = [weight_like(rng, 2176, 640) for _ in range(2)]
+    x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(40, 640)))).view(torch.bfloat16).cuda()
+    monkeypatch.setenv("GEOREFINE_FUSED_GEMM_TILING", "8,20")
+    results = {}
+    for mode in ("0", "3"):
+        monkeypatch.setattr(_fused, "GEMM_BALANCE", mode)
+        ts = [_tensor(w, fused_segment=64, residual_block=16)[1] for w in words]
+        scalars = ts[0]._gemm_tiling()[3]
+        group = HipLinearGroup(ts)
+        ys = [t.gemm(x, check=True) for t in ts] + group.linear(x, check=True)
+        results[mode] = (scalars, [y.view(torch.uint16).clone() for y in ys])
+        print("balance", mode, scalars, flush=True)
+    for a, b in zip(results["0"][1], results["3"][1]):
+        assert torch.equal(a, b)
+    for a, b in zip(results["3"][1][:2], results["3"][1][2:]):
+        assert torch.equal(a, b)  # the grouped launch gives the members' own products
+    assert results["0"][0]["lanes_per_row"] == results["3"][0]["lanes_per_row"]
+    assert (results["0"][0]["rows_per_tile"], results["3"][0]["rows_per_tile"]) == (20, 32)
