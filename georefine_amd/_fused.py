@@ -474,7 +474,13 @@ def build_balanced_tiles(row_class, nr, unit_rows, slots, max_rows):
     return np.concatenate(out_rows), np.asarray(out_class, dtype=np.uint8), tallest
 
 
-GEMM_BALANCE = os.environ.get("GEOREFINE_GEMM_BALANCE", "3")  # "0": tiles of one height (experiments)
+GEMM_BALANCE = os.environ.get("GEOREFINE_GEMM_BALANCE", "1") != "0"  # "0": tiles of one height (experiments)
+
+
+def _blocks_paid(tile_rows, height):
+    """Blocks of sixteen rows that the waves of a launch walk: every tile's rows rounded up."""
+    held = (tile_rows.reshape(-1, height) != 0xFFFFFFFF).sum(axis=1)
+    return int(((held + 15) // 16).sum())
 
 
 def build_gemm_tiles(row_class, nr, r, first_tile=0, lead=0, cus=256):
@@ -492,23 +498,21 @@ def build_gemm_tiles(row_class, nr, r, first_tile=0, lead=0, cus=256):
     starting at position ``lead`` (the tall tiles other members of a grouped launch have
     placed already)."""
     tile_rows, tile_class = build_tiles(row_class, nr, r)
-    blocks = -(-r // 16)
-    paid = lambda rows_, height: int(((rows_.reshape(-1, height) != 0xFFFFFFFF).sum(axis=1) + 15).__floordiv__(16).sum())
-    if GEMM_BALANCE == "0" or r % 16 == 0:
+    if not GEMM_BALANCE or r % 16 == 0:
         return tile_rows, tile_class, r, 0
-    even = build_balanced_tiles(row_class, nr, 16, len(tile_class), 16 * blocks)
+    even = build_balanced_tiles(row_class, nr, 16, len(tile_class), 16 * -(-r // 16))
     # (as many tiles as planned: tiles shorter than a block that spread a small matrix over the
     # workgroup slots stay as they are)
-    if even is None or len(even[1]) != len(tile_class) or paid(even[0], even[2]) >= paid(tile_rows, r):
+    if even is None or len(even[1]) != len(tile_class) or _blocks_paid(even[0], even[2]) >= _blocks_paid(tile_rows, r):
         return tile_rows, tile_class, r, 0
     tile_rows, tile_class, r = even
     table = tile_rows.reshape(-1, r)
     height = ((table != 0xFFFFFFFF).sum(axis=1) + 15) // 16
     tall = height == height.max()
     n_tall = int(tall.sum()) if height.max() > height.min() else 0
-    if n_tall and GEMM_BALANCE != "1":
+    if n_tall:
         tall_at, short_at = np.flatnonzero(tall), np.flatnonzero(~tall)
-        start = (lead - first_tile) % cus if GEMM_BALANCE == "3" else 0
+        start = (lead - first_tile) % cus
         if start + n_tall > len(tile_class) or start > len(short_at):
             start = 0
         order = np.concatenate((short_at[:start], tall_at, short_at[start:]))

@@ -187,7 +187,7 @@ def test_row_tiles_in_whole_blocks_leave_every_bit_as_it_was(monkeypatch):
     x = torch.from_numpy(bf16_words(rng.normal(0, 1, size=(40, 640)))).view(torch.bfloat16).cuda()
     monkeypatch.setenv("GEOREFINE_FUSED_GEMM_TILING", "8,20")
     results = {}
-    for mode in ("0", "3"):
+    for mode in (False, True):
         monkeypatch.setattr(_fused, "GEMM_BALANCE", mode)
         ts = [_tensor(w, fused_segment=64, residual_block=16)[1] for w in words]
         scalars = ts[0]._gemm_tiling()[3]
@@ -195,9 +195,9 @@ def test_row_tiles_in_whole_blocks_leave_every_bit_as_it_was(monkeypatch):
         ys = [t.gemm(x, check=True) for t in ts] + group.linear(x, check=True)
         results[mode] = (scalars, [y.view(torch.uint16).clone() for y in ys])
         print("balance", mode, scalars, flush=True)
-    for a, b in zip(results["0"][1], results["3"][1]):
+    for a, b in zip(results[False][1], results[True][1]):
         assert torch.equal(a, b)
-    for a, b in zip(results["3"][1][:2], results["3"][1][2:]):
+    for a, b in zip(results[True][1][:2], results[True][1][2:]):
         assert torch.equal(a, b)  # the grouped launch gives the members' own products
-    assert results["0"][0]["lanes_per_row"] == results["3"][0]["lanes_per_row"]
-    assert (results["0"][0]["rows_per_tile"], results["3"][0]["rows_per_tile"]) == (20, 32)
+    assert results[False][0]["lanes_per_row"] == results[True][0]["lanes_per_row"]
+    assert (results[False][0]["rows_per_tile"], results[True][0]["rows_per_tile"]) == (20, 32)
