@@ -354,6 +354,41 @@ __device__ __forceinline__ void fused_load_tables(uint8_t *lds, uint32_t blocks,
   }
 }
 
+// The same tables copied without vector registers, by loads that write the LDS directly, the
+// waves taking the copy's 1 KiB (lookup bytes) and 256-byte (entries, which are only 8-byte
+// aligned) chunks in turn.  Nothing waits here: the copy is issued first thing in a workgroup
+// and is under way while the reads that lead to the first unit's stream bytes follow one
+// another; it is complete at the workgroup's barrier.  For lookups of at least 1 KiB a column
+// class (a chunk must not straddle two classes' blocks).
+__device__ __forceinline__ bool fused_tables_by_dma(const grf_bctx_fused &f) { return f.lognb >= 10; }
+__device__ __forceinline__ void fused_load_tables_dma(uint8_t *lds, uint32_t blocks, uint32_t block_pitch,
+                                                      const grf_bctx_fused &f, uint32_t cls, uint32_t wave,
+                                                      uint32_t nwaves, uint32_t lane) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  typedef __attribute__((address_space(3))) void lds_void;
+  const uint32_t lut_bytes = 1u << f.lognb, tab_bytes = (f.tabn + 1) * 8, tb = fused_table_bytes(f);
+  const uint8_t *lut = f.lut + (size_t)cls * f.nc * lut_bytes;
+  const uint8_t *tab = reinterpret_cast<const uint8_t *>(f.tab) + (size_t)cls * f.nc * tab_bytes;
+  const uint32_t lut_chunks = lut_bytes >> 10, tab_chunks = (tab_bytes + 255) >> 8;  // of one column class
+  const uint32_t n_lut = f.nc * lut_chunks, n_tab = f.nc * tab_chunks;
+  for (uint32_t c = wave; c < n_lut + n_tab; c += nwaves) {  // uniform
+    if (c < n_lut) {
+      const uint32_t cc = c / lut_chunks, k = c - cc * lut_chunks;
+      __builtin_amdgcn_global_load_lds(lut + (cc * lut_bytes + k * 1024 + lane * 16),
+                                       (lds_void *)(lds + (blocks + cc * block_pitch + tb + k * 1024)), 16, 0, 0);
+    } else {
+      const uint32_t t = c - n_lut, cc = t / tab_chunks, k = t - cc * tab_chunks;
+      const uint32_t o = k * 256 + lane * 4;
+      if (o < tab_bytes)
+        __builtin_amdgcn_global_load_lds(tab + (cc * tab_bytes + o), (lds_void *)(lds + (blocks + cc * block_pitch + k * 256)),
+                                         4, 0, 0);
+    }
+  }
+#else
+  (void)lds, (void)blocks, (void)block_pitch, (void)f, (void)cls, (void)wave, (void)nwaves, (void)lane;
+#endif
+}
+
 // Where the checkpoint of a segment lies in the index arrays (seg_state, seg_offset).  In the
 // frame's order (raw_interleaved == 0) segment s of row r is entry r * segs_per_row + s and its
 // end is the entry after it.  In the blocked order the residuals have (raw_interleaved = B rows

@@ -321,6 +321,8 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
   const uint32_t P = g.lanes_per_row, rpw = 64 / P, R = g.rows_per_tile, S = f.seg_len, K = f.cols;
   const uint32_t cls = g.tile_class[tile];
   const grf::FusedParams q{f.shift, L.block_pitch, grf::fused_table_bytes(f), f.whole_range};
+  const bool tables_by_dma = grf::fused_tables_by_dma(f);
+  if (tables_by_dma) grf::fused_load_tables_dma(lds, L.blocks, L.block_pitch, f, cls, wave, nwaves, lane);
   // P is a power of two: lane coordinates by shift and mask.  A unit is (row group grp, slab b),
   // numbered u = grp * n_slabs + b or, for long rows, u = b * groups + grp; a wave steps through
   // its units u = wave, wave + nwaves, ... by adding (nwaves / n, nwaves % n) to the pair with a
@@ -388,7 +390,10 @@ __device__ __forceinline__ void fused_wave_body(uint8_t *lds, const grf_bctx_fus
     rows[i] = rw;
     rows[R + i] = row_position(f, rw);
   }
-  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
+  if (!tables_by_dma) grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the tables' copy has landed)
+#endif
   __syncthreads();
   const uint32_t later_half = blockIdx.x >= gridDim.x / 2 ? 1u : 0u;
   uint32_t left = wave < units ? (units - 1 - wave) / nwaves : 0;  // units after the current one
@@ -827,6 +832,9 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
 #else
   const uint32_t wave = tid / 64;
 #endif
+  // (the tables' copy first: it is under way while the reads below follow one another)
+  const bool tables_by_dma = grf::fused_tables_by_dma(f);
+  if (tables_by_dma) grf::fused_load_tables_dma(lds, L.blocks, L.block_pitch, f, cls, wave, nthreads / 64, lane);
   const uint32_t rb = wave % shape.row_blocks, quad = wave / shape.row_blocks;
   const uint32_t r = rb * 16 + lane % 16, p4 = lane / 16;
   uint32_t row = r < R ? g.tile_rows[tile * R + r] : grf::kNoRow;
@@ -852,12 +860,15 @@ __device__ __forceinline__ void fused_gemm_body(uint8_t *lds, const grf_bctx_fus
   };
   uint32_t g0, g1;
   span_of(b_first, g0, g1);  // started before the table copy so that the latencies overlap
-  grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
+  if (!tables_by_dma) grf::fused_load_tables(lds, L.blocks, L.block_pitch, f, cls, tid, nthreads);
 
   float4v acc[MT];
 #pragma unroll
   for (int j = 0; j < MT; ++j) acc[j] = (float4v){0.f, 0.f, 0.f, 0.f};
   uint32_t bad = 0;
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the tables' copy has landed)
+#endif
   __syncthreads();  // the tables are in place
   const uint32_t later_half = blockIdx.x >= gridDim.x / 2 ? 1u : 0u;
 
